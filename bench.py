@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 matrix-multiplication path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config N] [--all] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM: one launch of the configuration's product through the C
+ABI (two launches for the attention pair). The default workload is the
+MulAndShift linear layer, fp32 X[32x128x512] x W[512x2048] + b[2048]: the first
+configuration the metric's target is quoted on. `--all` adds one line per
+configuration before the headline line; the LAST line printed is the headline.
+
+Each JSON line carries
+  value/unit       TFLOP/s = 2 M N K batch / time, over the timed steps
+  roofline         the same kernel timed with HIP events on its own stream,
+                   against the MI355X dense matrix peak of the data type
+  cpu_baseline     the CPU restatement of the reference's naive path (1 thread,
+                   as the reference runs it) on a bounded sample of the same product
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6}     # MI355X dense matrix peaks (datasheet)
+HBM_TBS = 8.0
+
+
+def configs():
+    """The five configurations of the baseline, 1-based."""
+    return {
+        1: dict(name="cfg1 fp32 _MatrixMul NN 4096x512 . 512x2048", dtype="f32", M=4096, N=2048, K=512, batch=1),
+        2: dict(name="cfg2 fp32 MulAndShift X[32x128x512] . W[512x2048] + b[2048]", dtype="f32", M=4096, N=2048, K=512, batch=1),
+        3: dict(name="cfg3 fp32 _MatrixMulBatched Q.K^T/8 then S.V, [256x128x64]", dtype="f32", M=128, N=128, K=64, batch=256),
+        4: dict(name="cfg4 fp16 _MatrixMul TN a[1024x8192]^T . b[1024x4096]", dtype="f16", M=8192, N=4096, K=1024, batch=1),
+        5: dict(name="cfg5 fp32 _MatrixMul NT H[4096x512] . W[30011x512]^T + C, beta=1", dtype="f32", M=4096, N=30011, K=512, batch=1),
+    }
+
+
+class Workload:
+    """Device buffers and the launch closure of one configuration."""
+
+    def __init__(self, idx, dev, oracle):
+        import torch
+        import niutensor_amd as nt
+        self.idx = idx
+        self.cfg = configs()[idx]
+        T, NT = nt.X_TRANS, nt.X_NOTRANS
+        g = lambda x: torch.from_numpy(x).to(dev)
+        if idx in (1, 2):
+            self.x = g(oracle.uniform((4096, 512), 1))
+            self.w = g(oracle.uniform((512, 2048), 2) if idx == 1 else oracle.normal((512, 2048), 2, 0, 0.02))
+            self.b = g(oracle.normal((2048,), 3, 0, 0.02))
+            self.c = torch.full((4096, 2048), float("nan"), device=dev)
+            bias = self.b if idx == 2 else None
+            self.run = lambda: nt.matrix_mul(self.x, NT, self.w, NT, self.c, 1.0, 0.0, bias=bias)
+            self.flops = 2.0 * 4096 * 2048 * 512
+            self.bytes = 4.0 * (4096 * 512 + 512 * 2048 + 4096 * 2048) + (8192 if idx == 2 else 0)
+            self.launches = 1
+        elif idx == 3:
+            self.q = g(oracle.normal((256, 128, 64), 1))
+            self.k = g(oracle.normal((256, 128, 64), 2))
+            self.v = g(oracle.normal((256, 128, 64), 3))
+            self.s = torch.empty((256, 128, 128), device=dev)
+            self.o = torch.empty((256, 128, 64), device=dev)
+
+            def run():
+                nt.matrix_mul_batched_strided(self.q, NT, self.k, T, self.s, 256, 8192, 8192, 16384,
+                                              128, 64, 128, 64, 128, 128, 0.125, 0.0)
+                nt.matrix_mul_batched_strided(self.s, NT, self.v, NT, self.o, 256, 16384, 8192, 8192,
+                                              128, 128, 128, 64, 128, 64, 1.0, 0.0)
+            self.run = run
+            self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
+            self.bytes = 2 * 4.0 * 256 * (128 * 64 + 128 * 64 + 128 * 128)
+            self.launches = 2
+        elif idx == 4:
+            self.a = g(oracle.normal((1024, 8192), 1, 0, 0.02)).half()
+            self.b = g(oracle.normal((1024, 4096), 2, 0, 0.02)).half()
+            self.c = torch.empty((8192, 4096), device=dev, dtype=torch.float16)
+            self.run = lambda: nt.matrix_mul(self.a, T, self.b, NT, self.c, 1.0, 0.0)
+            self.flops = 2.0 * 8192 * 4096 * 1024
+            self.bytes = 2.0 * (1024 * 8192 + 1024 * 4096 + 8192 * 4096)
+            self.launches = 1
+        elif idx == 5:
+            self.h = g(oracle.uniform((4096, 512), 1))
+            self.w = g(oracle.normal((30011, 512), 2, 0, 0.02))
+            self.c = torch.rand((4096, 30011), device=dev) * 2 - 1
+            self.run = lambda: nt.matrix_mul(self.h, NT, self.w, T, self.c, 1.0, 1.0)
+            self.flops = 2.0 * 4096 * 30011 * 512
+            self.bytes = 4.0 * (4096 * 512 + 30011 * 512 + 2 * 4096 * 30011)
+            self.launches = 1
+        else:
+            raise SystemExit("no such configuration: %d" % idx)
+
+
+class HipEvents:
+    """hipEvent timing on the stream the kernels are launched on."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(self.e0)) == 0
+        assert self.hip.hipEventCreate(C.byref(self.e1)) == 0
+
+    def time(self, fn, stream, reps):
+        assert self.hip.hipEventRecord(self.e0, stream) == 0
+        for _ in range(reps):
+            fn()
+        assert self.hip.hipEventRecord(self.e1, stream) == 0
+        assert self.hip.hipEventSynchronize(self.e1) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), self.e0, self.e1) == 0
+        return ms.value * 1e-3 / reps
+
+
+def cpu_baseline(idx, budget_s=12.0):
+    """The CPU restatement of the reference's naive path, one thread (the reference's default:
+    no parallel runner means one job), on a row sample of the same product sized for ~budget_s."""
+    import numpy as np
+    from oracle.binding import Oracle, X_NOTRANS, X_TRANS
+    o = Oracle(native=True)
+    cfg = configs()[idx]
+    M, N, K = cfg["M"], cfg["N"], cfg["K"]
+    # measured rates of this path: ~0.8 GFLOP/s when b is walked by column (NN), ~3 GFLOP/s when both are rows
+    rate = {1: 0.8e9, 2: 0.8e9, 3: 1.5e9, 4: 0.4e9, 5: 2.5e9}[idx]
+    if idx == 3:
+        nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
+        q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
+        t0 = time.perf_counter()
+        s = o.matmul_batched(q, X_NOTRANS, k, X_TRANS, None, 0.125)
+        o.matmul_batched(s, X_NOTRANS, v, X_NOTRANS)
+        dt = time.perf_counter() - t0
+        fl = nb * 4.0 * 128 * 128 * 64
+        sample = "%d of 256 batch items, both products" % nb
+    else:
+        rows = max(8, min(M, int(budget_s * rate / (2.0 * N * K))))
+        if idx in (1, 2):
+            a, b = o.uniform((rows, K), 1), o.uniform((K, N), 2)
+            bias = o.normal((N,), 3, 0, 0.02)
+            t0 = time.perf_counter()
+            if idx == 1:
+                o.matmul2d(a, X_NOTRANS, b, X_NOTRANS)
+            else:
+                o.mulandshift(a.reshape(1, rows, K), b, bias)
+            dt = time.perf_counter() - t0
+        elif idx == 4:
+            # fp32 arithmetic on the half-rounded values: the reference has no CPU half product
+            a = o.from_f16_bits(o.to_f16_bits(o.normal((K, rows), 1, 0, 0.02)))
+            b = o.from_f16_bits(o.to_f16_bits(o.normal((K, N), 2, 0, 0.02)))
+            t0 = time.perf_counter()
+            o.matmul2d(a, X_TRANS, b, X_NOTRANS)
+            dt = time.perf_counter() - t0
+        else:
+            a, b = o.uniform((rows, K), 1), o.normal((N, K), 2, 0, 0.02)
+            c = o.uniform((rows, N), 3)
+            t0 = time.perf_counter()
+            o.matmul2d(a, X_NOTRANS, b, X_TRANS, c, 1.0, 1.0)
+            dt = time.perf_counter() - t0
+        fl = 2.0 * rows * N * K
+        sample = "%d of %d result rows, all %d columns, K=%d" % (rows, M, N, K)
+    return {"value": round(fl / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": sample + " (%.1f s; %.2f GFLOP/s, -O3 -march=native)" % (dt, fl / dt / 1e9)}
+
+
+def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
+    import torch
+    wl = Workload(idx, dev, oracle)
+    cfg = wl.cfg
+    for _ in range(warmup):
+        wl.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        wl.run()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+
+    # the kernel alone: HIP events on the stream the launches go to, best of 5 groups
+    ev = HipEvents()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    reps = max(10, min(200, steps))
+    kt = min(ev.time(wl.run, stream, reps) for _ in range(5))
+    peak = PEAK_TFLOPS[cfg["dtype"]]
+    achieved = wl.flops / kt / 1e12
+    out = {
+        "metric": "TFLOP/s & % of dense matrix peak for MatrixMul/Batched (fp32, fp16), 1 GPU",
+        "value": round(wl.flops / wall / 1e12, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(wall * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": cfg["name"], "M": cfg["M"], "N": cfg["N"], "K": cfg["K"], "batch": cfg["batch"],
+                   "launches_per_step": wl.launches, "inputs": "resident in HBM", "flops_per_step": wl.flops,
+                   "algorithmic_bytes_per_step": wl.bytes},
+        "pct_of_peak": round(100.0 * wl.flops / wall / 1e12 / peak, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel_us": round(kt / wl.launches * 1e6, 2),
+                     "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)},
+    }
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline(idx)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-5 (default 2, the MulAndShift linear layer)")
+    ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the path has no multi-GPU part (each product is independent); "
+                         "run with --gpus 1")
+
+    import torch
+    import niutensor_amd as nt
+    from oracle.binding import Oracle
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a gfx950 GPU")
+    nt.load()
+    dev = torch.device("cuda:0")
+    oracle = Oracle()
+    if args.all:
+        for idx in (1, 3, 4, 5):
+            steps = args.steps if idx != 5 else max(5, args.steps // 10)
+            print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else 3, dev, oracle, not args.no_cpu)), flush=True)
+    print(json.dumps(bench_one(args.config, args.steps, args.warmup, dev, oracle, not args.no_cpu)), flush=True)
+
+
+if __name__ == "__main__":
+    main()

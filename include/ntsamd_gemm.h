@@ -1,0 +1,136 @@
+/*
+ * ntsamd_gemm.h - C ABI of the gfx950 (MI355X) matrix-multiplication library
+ * for NiuTensor.
+ *
+ * These entry points stand where the reference's `USE_CUDA` branch calls
+ * cuBLAS: each one receives exactly what the corresponding
+ * `_CudaBLASMatrixMUL*` function of source/tensor/core/arithmetic/XTensorBLAS.h
+ * receives, minus the cuBLAS handle, plus the device id and a stream.
+ *
+ * Conventions (all taken from the reference):
+ *   - matrices are dense, row-major; na,ma / nb,mb / nc,mc are the STORED row
+ *     and column counts, so lda = ma, ldb = mb, ldc = mc (XTensorBLAS.cu:64-71);
+ *   - transposedA / transposedB use MATRIX_TRANS_TYPE values: X_TRANS = 0,
+ *     X_NOTRANS = 1 (XDataType.h:36);
+ *   - data types use TENSOR_DATA_TYPE values: X_FLOAT = 2, X_FLOAT16 = 3
+ *     (XDataType.h:33). Supported triples (a, b, c): (X_FLOAT, X_FLOAT, X_FLOAT),
+ *     (X_FLOAT16, X_FLOAT16, X_FLOAT16) and (X_FLOAT16, X_FLOAT16, X_FLOAT);
+ *     anything else fails with "Unsupported data type!" (XTensorBLAS.cu:101-103);
+ *   - the result is c = alpha * op(a) * op(b) + beta * c. With beta == 0 the
+ *     kernels never read c, so the caller does not have to zero it first (the
+ *     reference calls SetZeroAll before every beta == 0 product,
+ *     MatrixMul2D.cu:154-155; that pass is no longer needed);
+ *   - alpha and beta arrive as float for every data type; half products
+ *     accumulate in fp32;
+ *   - c must not overlap a or b; all pointers are device pointers on `devID`.
+ *
+ * Every function returns 0 on success and a non-zero code on failure; the
+ * message of the last failure on the calling thread is available from
+ * ntsamd_last_error(). Nothing is thrown across this boundary. The library
+ * keeps no mutable global state, allocates no device memory, restores the
+ * caller's current device before returning, and issues its work on `stream`
+ * (NULL = the default stream, which is what the reference uses) without
+ * synchronising.
+ */
+#ifndef NTSAMD_GEMM_H
+#define NTSAMD_GEMM_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NTSAMD_X_TRANS 0
+#define NTSAMD_X_NOTRANS 1
+#define NTSAMD_X_FLOAT 2
+#define NTSAMD_X_FLOAT16 3
+
+/* return codes */
+#define NTSAMD_OK 0
+#define NTSAMD_ERR_ARGUMENT 1     /* bad shape, pointer, flag or count */
+#define NTSAMD_ERR_DATATYPE 2     /* "Unsupported data type!" */
+#define NTSAMD_ERR_DEVICE 3       /* no such device, or not a gfx950 device */
+#define NTSAMD_ERR_LAUNCH 4       /* the HIP runtime refused the launch */
+
+/* bias broadcast of the fused epilogue */
+#define NTSAMD_BIAS_NONE 0
+#define NTSAMD_BIAS_COL 1         /* c[i][j] += bias[j]                      */
+#define NTSAMD_BIAS_ROW 2         /* c[i][j] += bias[(i / rowDiv) % biasLen] */
+
+/* Message of the last failure on this thread ("" if none). */
+const char * ntsamd_last_error(void);
+
+/* Library version, "major.minor". */
+const char * ntsamd_version(void);
+
+/* Checks that `devID` exists and is a gfx950 device and loads the kernels'
+   code object on it. Optional: every entry point does this on first use.
+   Takes the place of GDevs.GetCudaHandle(devID) (XDevice.cpp:207-224); there
+   is no handle to create. */
+int ntsamd_init(int devID);
+
+/*
+ * One product. Replaces
+ *   _CudaBLASMatrixMUL(handle, a, transposedA, dataTypeA, b, transposedB, dataTypeB,
+ *                      c, dataTypeC, na, ma, nb, mb, nc, mc, alpha, beta)
+ * source/tensor/core/arithmetic/XTensorBLAS.h:36-40, XTensorBLAS.cu:38-104.
+ */
+int ntsamd_matrix_mul(int devID, void * stream,
+                      const void * a, int transposedA, int dataTypeA,
+                      const void * b, int transposedB, int dataTypeB,
+                      void * c, int dataTypeC,
+                      int na, int ma, int nb, int mb, int nc, int mc,
+                      float alpha, float beta);
+
+/*
+ * One product with the bias add fused into the epilogue:
+ *   c = alpha * op(a) * op(b) + beta * c + broadcast(bias).
+ * Replaces the pair the reference's MulAndShift issues (MulAndShift.cpp:69,88):
+ * _CudaBLASMatrixMUL into a temporary followed by _CudaSumDim
+ * (SumDim.cu:120-211; KernelAddWithRow :43-64 is NTSAMD_BIAS_COL,
+ * KernelAddWithCol :79-105 is NTSAMD_BIAS_ROW with rowDiv = the product of
+ * the result's dimensions after the broadcast one, last excluded).
+ * `bias` has the data type of c and `biasLen` elements; for NTSAMD_BIAS_COL
+ * biasLen must equal mc.
+ */
+int ntsamd_matrix_mul_bias(int devID, void * stream,
+                           const void * a, int transposedA, int dataTypeA,
+                           const void * b, int transposedB, int dataTypeB,
+                           void * c, int dataTypeC,
+                           int na, int ma, int nb, int mb, int nc, int mc,
+                           float alpha, float beta,
+                           const void * bias, int biasMode, int biasLen, int biasRowDiv);
+
+/*
+ * `count` products over equally spaced matrices; strides are in ELEMENTS and
+ * a stride of 0 shares one a or b among all products. Replaces
+ *   _CudaBLASMatrixMULBatchedStrided(handle, a, transposedA, dataTypeA, strideA, ...)
+ * source/tensor/core/arithmetic/XTensorBLAS.h:51-56, XTensorBLAS.cu:181-247.
+ */
+int ntsamd_matrix_mul_batched_strided(int devID, void * stream,
+                                      const void * a, int transposedA, int dataTypeA, long long strideA,
+                                      const void * b, int transposedB, int dataTypeB, long long strideB,
+                                      void * c, int dataTypeC, long long strideC,
+                                      int count, int na, int ma, int nb, int mb, int nc, int mc,
+                                      float alpha, float beta);
+
+/*
+ * `count` products over arbitrary same-shaped matrices. a, b and c are HOST
+ * arrays of `count` DEVICE pointers. Replaces
+ *   _CudaBLASMatrixMULBatched(handle, a, ..., count, na, ma, nb, mb, nc, mc, alpha, beta)
+ * source/tensor/core/arithmetic/XTensorBLAS.h:43-48, XTensorBLAS.cu:109-178,
+ * together with the staging the reference does before calling it
+ * (XTensorBLAS.cu:315-368: three device arrays allocated, filled by cudaMemcpy,
+ * freed afterwards). Here the pointers ride in the kernel arguments, so there
+ * is no allocation and no copy.
+ */
+int ntsamd_matrix_mul_batched(int devID, void * stream,
+                              const void * const * a, int transposedA, int dataTypeA,
+                              const void * const * b, int transposedB, int dataTypeB,
+                              void * const * c, int dataTypeC,
+                              int count, int na, int ma, int nb, int mb, int nc, int mc,
+                              float alpha, float beta);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,142 @@
+"""MI355X (gfx950) matrix multiplication for NiuTensor: Python plumbing.
+
+The product is the C-ABI library `lib/libntsamd.so` (hand-written HIP kernels,
+declared in `include/ntsamd_gemm.h`) and the C++ `nts::` host layer in `nts/`.
+This module only loads the library through ctypes so that tests and the
+benchmark can call the C ABI on buffers that PyTorch owns. There is no CPU
+fallback: if the library is missing, or there is no gfx950 device, calls fail.
+"""
+import ctypes as C
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libntsamd.so")
+HOST_LIB_PATH = os.path.join(HERE, "lib", "libnts_amd.so")
+
+X_TRANS, X_NOTRANS = 0, 1           # MATRIX_TRANS_TYPE, source/tensor/XDataType.h:36
+X_FLOAT, X_FLOAT16 = 2, 3           # TENSOR_DATA_TYPE, source/tensor/XDataType.h:33
+BIAS_NONE, BIAS_COL, BIAS_ROW = 0, 1, 2
+
+EXPORTS = (
+    "ntsamd_last_error",
+    "ntsamd_version",
+    "ntsamd_init",
+    "ntsamd_matrix_mul",
+    "ntsamd_matrix_mul_bias",
+    "ntsamd_matrix_mul_batched_strided",
+    "ntsamd_matrix_mul_batched",
+)
+
+
+class NtsAmdError(RuntimeError):
+    pass
+
+
+def build(jobs=8):
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+    subprocess.run(["make", "-s", "-C", os.path.join(HERE, "csrc"), "-j%d" % jobs], check=True)
+    subprocess.run(["make", "-s", "-C", os.path.join(HERE, "nts"), "-j%d" % jobs], check=True)
+
+
+_lib = None
+
+
+def load():
+    """Load libntsamd.so; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise NtsAmdError("%s is missing: run niutensor_amd.build() (or make -C niutensor_amd/csrc)" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    vp, ci, cf, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
+    L.ntsamd_last_error.restype = C.c_char_p
+    L.ntsamd_version.restype = C.c_char_p
+    L.ntsamd_init.argtypes = [ci]
+    L.ntsamd_matrix_mul.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf]
+    L.ntsamd_matrix_mul_bias.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, ci, ci, ci]
+    L.ntsamd_matrix_mul_batched_strided.argtypes = [ci, vp, vp, ci, ci, ll, vp, ci, ci, ll, vp, ci, ll,
+                                                    ci] + [ci] * 6 + [cf, cf]
+    L.ntsamd_matrix_mul_batched.argtypes = [ci, vp, C.POINTER(vp), ci, ci, C.POINTER(vp), ci, ci, C.POINTER(vp), ci,
+                                            ci] + [ci] * 6 + [cf, cf]
+    for name in EXPORTS[2:]:
+        getattr(L, name).restype = ci
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise NtsAmdError("ntsamd error %d: %s" % (rc, load().ntsamd_last_error().decode()))
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float32:
+        return X_FLOAT
+    if t.dtype == torch.float16:
+        return X_FLOAT16
+    raise NtsAmdError("Unsupported data type!")
+
+
+def _stream_ptr(t):
+    import torch
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _mat(t):
+    """Stored rows, columns of the last two dimensions of a dense tensor."""
+    assert t.is_contiguous()
+    return int(t.shape[-2]), int(t.shape[-1])
+
+
+def matrix_mul(a, transA, b, transB, c, alpha=1.0, beta=0.0, bias=None, bias_mode=BIAS_COL, bias_row_div=1):
+    """c = alpha * op(a) op(b) + beta * c (+ bias) on 2-D device tensors, through the C ABI."""
+    L = load()
+    na, ma = _mat(a)
+    nb, mb = _mat(b)
+    nc, mc = _mat(c)
+    dev = a.device.index
+    if bias is None:
+        rc = L.ntsamd_matrix_mul(dev, _stream_ptr(a), a.data_ptr(), transA, _dtype_code(a),
+                                 b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
+                                 na, ma, nb, mb, nc, mc, alpha, beta)
+    else:
+        rc = L.ntsamd_matrix_mul_bias(dev, _stream_ptr(a), a.data_ptr(), transA, _dtype_code(a),
+                                      b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
+                                      na, ma, nb, mb, nc, mc, alpha, beta,
+                                      bias.data_ptr(), bias_mode, bias.numel(), bias_row_div)
+    _check(rc)
+    return c
+
+
+def matrix_mul_batched_strided(a, transA, b, transB, c, count, strideA, strideB, strideC,
+                               na, ma, nb, mb, nc, mc, alpha=1.0, beta=0.0):
+    L = load()
+    rc = L.ntsamd_matrix_mul_batched_strided(a.device.index, _stream_ptr(a),
+                                             a.data_ptr(), transA, _dtype_code(a), strideA,
+                                             b.data_ptr(), transB, _dtype_code(b), strideB,
+                                             c.data_ptr(), _dtype_code(c), strideC,
+                                             count, na, ma, nb, mb, nc, mc, alpha, beta)
+    _check(rc)
+    return c
+
+
+def matrix_mul_batched(a_list, transA, b_list, transB, c_list, alpha=1.0, beta=0.0):
+    """Pointer-list batch over same-shaped 2-D device tensors."""
+    L = load()
+    n = len(a_list)
+    arr = C.c_void_p * n
+    pa = arr(*[t.data_ptr() for t in a_list])
+    pb = arr(*[t.data_ptr() for t in b_list])
+    pc = arr(*[t.data_ptr() for t in c_list])
+    a, b, c = a_list[0], b_list[0], c_list[0]
+    na, ma = _mat(a)
+    nb, mb = _mat(b)
+    nc, mc = _mat(c)
+    rc = L.ntsamd_matrix_mul_batched(a.device.index, _stream_ptr(a), pa, transA, _dtype_code(a),
+                                     pb, transB, _dtype_code(b), pc, _dtype_code(c),
+                                     n, na, ma, nb, mb, nc, mc, alpha, beta)
+    _check(rc)
+    return c_list

@@ -1,0 +1,98 @@
+/*
+ * Shared definitions of the gfx950 GEMM kernels: problem descriptor, vector
+ * types, workgroup-to-tile mapping.
+ *
+ * All matrices are dense and row-major. A "K-contiguous" operand stores the
+ * reduction index fastest (a with X_NOTRANS, b with X_TRANS); an
+ * "MN-contiguous" operand stores the output index fastest (a with X_TRANS,
+ * b with X_NOTRANS). The leading dimension is always the stored column count,
+ * as in the reference's BLAS calls (XTensorBLAS.cu:64-71: lda=ma, ldb=mb, ldc=mc).
+ */
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ntsamd {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+enum BiasMode { BIAS_NONE = 0, BIAS_COL = 1, BIAS_ROW = 2 };
+
+/* pointer-array batches travel in the kernel argument block: no device
+   allocation, no host-to-device copy. One launch covers PTR_BATCH_MAX items. */
+#define NTSAMD_PTR_BATCH_MAX 128
+struct PtrBatch {
+    const void * a[NTSAMD_PTR_BATCH_MAX];
+    const void * b[NTSAMD_PTR_BATCH_MAX];
+    void * c[NTSAMD_PTR_BATCH_MAX];
+};
+struct NoPtrs {
+    char unused;
+};
+
+struct GemmParams {
+    const void * a;
+    const void * b;
+    void * c;
+    const void * bias;
+    int M, N, K;
+    int lda, ldb, ldc;
+    long long strideA, strideB, strideC;   /* elements between batch items; 0 = shared operand */
+    float alpha, beta;
+    int biasMode;                          /* BiasMode */
+    int biasRowDiv, biasLen;               /* BIAS_ROW: index = (row / biasRowDiv) % biasLen */
+    int tilesM, tilesN;
+    int batch;
+    int groupM;                            /* tile rows that share a pass over the tile columns */
+};
+
+/* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and
+   every XCD has its own L2. Renumber so that each XCD works on one contiguous
+   range of tiles and the operand panels those tiles share stay in that L2. */
+__device__ __forceinline__ int xcd_contiguous_id(int id, int total)
+{
+    const int X = 8;
+    int per = total / X, rem = total % X;
+    int xcd = id % X, idx = id / X;
+    return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+struct TileCoord {
+    int batch, tm, tn;
+};
+
+__device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
+{
+    int total = p.tilesM * p.tilesN * p.batch;
+    int id = xcd_contiguous_id((int)blockIdx.x, total);
+    int perBatch = p.tilesM * p.tilesN;
+    TileCoord t;
+    t.batch = id / perBatch;
+    int r = id - t.batch * perBatch;
+    int perGroup = p.groupM * p.tilesN;
+    int g = r / perGroup;
+    int firstM = g * p.groupM;
+    int gsz = p.tilesM - firstM < p.groupM ? p.tilesM - firstM : p.groupM;
+    int q = r - g * perGroup;
+    t.tm = firstM + q % gsz;
+    t.tn = q / gsz;
+    return t;
+}
+
+/* tile shapes the dispatcher can pick from */
+enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_COUNT = 2 };
+
+template <int CFG> struct TileShape;
+template <> struct TileShape<CFG_128x128> { static constexpr int BM = 128, BN = 128, WGM = 2, WGN = 2; };
+template <> struct TileShape<CFG_64x64> { static constexpr int BM = 64, BN = 64, WGM = 2, WGN = 2; };
+
+int launch_f32(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,
+               bool vec, int cfg, hipStream_t stream);
+int launch_f16(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,
+               bool vec, bool outF32, int cfg, hipStream_t stream);
+
+}  // namespace ntsamd

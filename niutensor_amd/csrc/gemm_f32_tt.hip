@@ -1,0 +1,8 @@
+/* fp32 kernels for op(a),op(b) = tt (n: X_NOTRANS, t: X_TRANS); one file per pair so they build in parallel */
+#include "gemm_f32.h"
+namespace ntsamd {
+int launch_f32_tt(const GemmParams & p, const PtrBatch * ptrs, bool vec, int cfg, hipStream_t stream)
+{
+    return launch_f32_trans<false, true>(p, ptrs, vec, cfg, stream);
+}
+}

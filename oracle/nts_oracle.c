@@ -1,0 +1,507 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library (see nts_oracle.h).
+ *
+ * Plain-C restatement of the CPU path of the NiuTensor matrix-multiplication
+ * family. Build with -ffp-contract=off: the reference is compiled without FMA
+ * contraction for baseline x86-64, and the single fp32 accumulator with
+ * ascending k is what fixes the rounding of every output element.
+ */
+#include "nts_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---- 2-D product -------------------------------------------------------- */
+
+/* NN kernel: MatrixMul2DMultiTheading.cpp:59-145 (FAST_MATRIX branch) run as
+   one job over the whole of c (XMatrixSegment.cpp:44-49: no runner => 1 job).
+   Four loop bodies there differ only in whether alpha is multiplied per term
+   (alpha != 1) and whether c*beta is added (beta != 0). */
+static void mm_nn(const float *a, const float *b, float *c,
+                  int am, int bm, int cn, int cm, float alpha, float beta)
+{
+    int num = am;
+    for (int i = 0; i < cn; i++) {
+        float *p3 = c + (long)i * cm;
+        for (int j = 0; j < cm; j++) {
+            float r = 0;
+            const float *p1 = a + (long)i * am;
+            const float *p2 = b + j;
+            if (alpha == 1) {
+                for (int k = 0; k < num; k++) {
+                    r += (*p1) * (*p2);
+                    p1 += 1;
+                    p2 += bm;
+                }
+            }
+            else {
+                for (int k = 0; k < num; k++) {
+                    r += (*p1) * (*p2) * alpha;
+                    p1 += 1;
+                    p2 += bm;
+                }
+            }
+            if (beta == 0)
+                *p3 = r;
+            else
+                *p3 = *p3 * beta + r;
+            p3 += 1;
+        }
+    }
+}
+
+/* TN / NT / TT: MatrixMul2DParallel.cpp:67-128. alpha is always multiplied
+   inside the sum; the output is always c*beta + r (c was zeroed for beta==0). */
+static void mm_strided(const float *a, long aRowStep, long aKStep,
+                       const float *b, long bColStep, long bKStep,
+                       float *c, int cn, int cm, int num, float alpha, float beta)
+{
+    for (int i = 0; i < cn; i++) {
+        float *p3 = c + (long)i * cm;
+        for (int j = 0; j < cm; j++) {
+            float r = 0;
+            const float *p1 = a + i * aRowStep;
+            const float *p2 = b + j * bColStep;
+            for (int k = 0; k < num; k++) {
+                r += (*p1) * (*p2) * alpha;
+                p1 += aKStep;
+                p2 += bKStep;
+            }
+            *p3 = *p3 * beta + r;
+            p3 += 1;
+        }
+    }
+}
+
+int oracle_matmul2d(const float *a, int transA, const float *b, int transB, float *c,
+                    int na, int ma, int nb, int mb, int nc, int mc,
+                    float alpha, float beta)
+{
+    /* shape rule of MatrixMul2D.cpp:56-67 */
+    int am2 = transA == ORACLE_X_TRANS ? na : ma;
+    int an2 = transA == ORACLE_X_TRANS ? ma : na;
+    int bm2 = transB == ORACLE_X_TRANS ? nb : mb;
+    int bn2 = transB == ORACLE_X_TRANS ? mb : nb;
+    if (!(am2 == bn2 && an2 == nc && bm2 == mc))
+        return -1;
+
+    /* MatrixMul2DParallel.cpp:57-58: beta == 0 zeroes c first, so whatever c
+       held (NaN included) never reaches the result */
+    if (beta == 0)
+        memset(c, 0, sizeof(float) * (size_t)nc * (size_t)mc);
+
+    if (nc == 0 || mc == 0)
+        return 0;
+
+    if (transA == ORACLE_X_NOTRANS && transB == ORACLE_X_NOTRANS)
+        mm_nn(a, b, c, ma, mb, nc, mc, alpha, beta);
+    else if (transA == ORACLE_X_TRANS && transB == ORACLE_X_NOTRANS)
+        mm_strided(a, 1, ma, b, 1, mb, c, nc, mc, na, alpha, beta);   /* :67-86 */
+    else if (transA == ORACLE_X_NOTRANS && transB == ORACLE_X_TRANS)
+        mm_strided(a, ma, 1, b, mb, 1, c, nc, mc, ma, alpha, beta);   /* :88-107 */
+    else
+        mm_strided(a, 1, ma, b, mb, 1, c, nc, mc, na, alpha, beta);   /* :109-128 */
+    return 0;
+}
+
+/* ---- batched and N-D products ------------------------------------------- */
+
+int oracle_matmul_batched(const float *a, int transA, const int *aDims,
+                          const float *b, int transB, const int *bDims,
+                          float *c, const int *cDims, int order,
+                          float alpha, float beta)
+{
+    /* MatrixMulBatched.cpp:171-191 */
+    if (order < 2)
+        return -1;
+    int an = transA == ORACLE_X_TRANS ? aDims[order - 1] : aDims[order - 2];
+    int am = transA == ORACLE_X_TRANS ? aDims[order - 2] : aDims[order - 1];
+    int bn = transB == ORACLE_X_TRANS ? bDims[order - 1] : bDims[order - 2];
+    int bm = transB == ORACLE_X_TRANS ? bDims[order - 2] : bDims[order - 1];
+    int cn = cDims[order - 2];
+    int cm = cDims[order - 1];
+    if (!(am == bn && an == cn && bm == cm))
+        return -1;
+
+    long aBlock = (long)aDims[order - 1] * aDims[order - 2];
+    long bBlock = (long)bDims[order - 1] * bDims[order - 2];
+    long cBlock = (long)cDims[order - 1] * cDims[order - 2];
+    int blockNum = 1;
+    for (int i = 0; i < order - 2; i++) {
+        if (aDims[i] != cDims[i] || bDims[i] != cDims[i])
+            return -1;
+        blockNum *= aDims[i];
+    }
+
+    /* :201-210, one _MatrixMul2D per block */
+    for (int i = 0; i < blockNum; i++) {
+        int r = oracle_matmul2d(a + i * aBlock, transA, b + i * bBlock, transB, c + i * cBlock,
+                                aDims[order - 2], aDims[order - 1],
+                                bDims[order - 2], bDims[order - 1],
+                                cn, cm, alpha, beta);
+        if (r != 0)
+            return r;
+    }
+    return 0;
+}
+
+static long unit_num(const int *dims, int order)
+{
+    long n = 1;
+    for (int i = 0; i < order; i++)
+        n *= dims[i];
+    return n;
+}
+
+int oracle_matmul(const float *a, int transA, const int *aDims, int aOrder,
+                  const float *b, int transB, const int *bDims, int bOrder,
+                  float *c, const int *cDims, int cOrder,
+                  float alpha, float beta)
+{
+    /* MatrixMul.cpp:56-61 */
+    if (aOrder < 2 || bOrder < 2 || cOrder < 2)
+        return -1;
+    if (cOrder != aOrder + bOrder - 2)
+        return -1;
+
+    /* MatrixMul.cpp:65-78: a higher-order, untransposed a times a matrix b is
+       one 2-D product over the flattened leading dimensions */
+    if (transA == ORACLE_X_NOTRANS && aOrder > 2 && bOrder == 2) {
+        int ncolA = aDims[aOrder - 1];
+        int ncolC = cDims[cOrder - 1];
+        return oracle_matmul2d(a, transA, b, transB, c,
+                               (int)(unit_num(aDims, aOrder) / ncolA), ncolA,
+                               bDims[0], bDims[1],
+                               (int)(unit_num(cDims, cOrder) / ncolC), ncolC,
+                               alpha, beta);
+    }
+
+    /* MatrixMul.cpp:80-110 */
+    int an = transA == ORACLE_X_TRANS ? aDims[aOrder - 1] : aDims[aOrder - 2];
+    int am = transA == ORACLE_X_TRANS ? aDims[aOrder - 2] : aDims[aOrder - 1];
+    int bn = transB == ORACLE_X_TRANS ? bDims[bOrder - 1] : bDims[bOrder - 2];
+    int bm = transB == ORACLE_X_TRANS ? bDims[bOrder - 2] : bDims[bOrder - 1];
+    int cn = cDims[cOrder - 2];
+    int cm = cDims[cOrder - 1];
+    if (!(am == bn && an == cn && bm == cm))
+        return -1;
+
+    long aBlock = (long)aDims[aOrder - 1] * aDims[aOrder - 2];
+    long bBlock = (long)bDims[bOrder - 1] * bDims[bOrder - 2];
+    long cBlock = (long)cDims[cOrder - 1] * cDims[cOrder - 2];
+    int aBlockNum = 1, bBlockNum = 1;
+    for (int i = 0; i < aOrder - 2; i++) {
+        if (aDims[i] != cDims[i])
+            return -1;
+        aBlockNum *= aDims[i];
+    }
+    for (int i = 0; i < bOrder - 2; i++) {
+        if (bDims[i] != cDims[i - 2 + aOrder])
+            return -1;
+        bBlockNum *= bDims[i];
+    }
+
+    /* MatrixMul.cpp:121-146 pairs every block p of a with every block q of b;
+       the result block sits at p * bBlockNum + q. The CPU list path then runs
+       one _MatrixMul2D per pair (MatrixMulBatched.cpp:257-270). */
+    for (int p = 0; p < aBlockNum; p++) {
+        for (int q = 0; q < bBlockNum; q++) {
+            int r = oracle_matmul2d(a + p * aBlock, transA, b + q * bBlock, transB,
+                                    c + ((long)p * bBlockNum + q) * cBlock,
+                                    aDims[aOrder - 2], aDims[aOrder - 1],
+                                    bDims[bOrder - 2], bDims[bOrder - 1],
+                                    cn, cm, alpha, beta);
+            if (r != 0)
+                return r;
+        }
+    }
+    return 0;
+}
+
+/* ---- bias broadcast ------------------------------------------------------ */
+
+int oracle_broadcast_dim_index(const int *aDims, int aOrder, const int *bDims, int bOrder)
+{
+    /* Sum.cpp:235-238 */
+    if (aOrder < bOrder)
+        return -1;
+    if (aOrder == bOrder) {
+        int same = 1;
+        for (int i = 0; i < aOrder; i++)
+            if (aDims[i] != bDims[i])
+                same = 0;
+        if (same)
+            return -1;
+    }
+
+    /* Sum.cpp:240-259: b may have one dimension that is not 1; the answer is
+       the LAST dimension of a with that size */
+    int hitDim = -1;
+    int isHit = 0;
+    for (int i = 0; i < bOrder; i++) {
+        if (bDims[bOrder - 1 - i] == 1)
+            continue;
+        if (isHit)
+            return -1;
+        isHit = 1;
+        for (int j = 0; j < aOrder; j++) {
+            if (bDims[bOrder - 1 - i] == aDims[aOrder - 1 - j]) {
+                hitDim = aOrder - 1 - j;
+                break;
+            }
+        }
+    }
+    return hitDim;
+}
+
+int oracle_sumdim(const float *a, const int *aDims, int aOrder,
+                  const float *b, int bUnitNum, float *c, int n, float beta)
+{
+    /* SumDim.cpp:51 MODX */
+    if (aOrder != 0)
+        n = (int)(n - floor((double)n / aOrder) * aOrder);
+    if (aDims[n] != bUnitNum)
+        return -1;
+
+    long num = unit_num(aDims, aOrder);
+
+    /* SumDim.cpp:63-66 */
+    if (beta == 0) {
+        memmove(c, a, sizeof(float) * (size_t)num);
+        return 0;
+    }
+
+    /* SumDim.cpp:81-91 */
+    int stride = 1;
+    int blockSize = aDims[n];
+    for (int i = aOrder - 1; i >= 0; i--) {
+        if (i > n)
+            stride *= aDims[i];
+    }
+
+    if (stride > 1) {
+        /* SumDim.cpp:95-102 */
+        long j = 0;
+        for (long i = 0; i < num; i += stride, j++) {
+            const float *ap = a + i;
+            float bv = b[j % blockSize] * beta;
+            float *cp = c + i;
+            for (int k = 0; k < stride; k++)
+                cp[k] = ap[k] + bv;
+        }
+    }
+    else {
+        /* SumDim.cpp:103-117 */
+        for (long i = 0; i < num; i += blockSize) {
+            const float *ap = a + i;
+            float *cp = c + i;
+            if (beta == 1.0F) {
+                for (int j = 0; j < blockSize; j++)
+                    cp[j] = ap[j] + b[j];
+            }
+            else {
+                for (int j = 0; j < blockSize; j++)
+                    cp[j] = ap[j] + b[j] * beta;
+            }
+        }
+    }
+    return 0;
+}
+
+int oracle_mulandshift(const float *x, int transX, const int *xDims, int xOrder,
+                       const float *w, int transW, const int *wDims, int wOrder,
+                       const float *bias, const int *bDims, int bOrder,
+                       float *c, int *cDims, int *cOrder, float alpha)
+{
+    if (xOrder < 2 || wOrder < 2)
+        return -1;
+
+    /* MulAndShift.cpp:44-60 and :128-142 */
+    int xn = transX == ORACLE_X_TRANS ? xDims[xOrder - 1] : xDims[xOrder - 2];
+    int wm = transW == ORACLE_X_TRANS ? wDims[wOrder - 2] : wDims[wOrder - 1];
+    int order = xOrder + wOrder - 2;
+    int sub = 0;
+    for (int i = 0; i < xOrder - 2; i++)
+        cDims[sub++] = xDims[i];
+    for (int i = 0; i < wOrder - 2; i++)
+        cDims[sub++] = wDims[i];
+    cDims[sub++] = xn;
+    cDims[sub++] = wm;
+    *cOrder = order;
+
+    long num = unit_num(cDims, order);
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)(num > 0 ? num : 1));
+    if (!tmp)
+        return -1;
+
+    /* :69 / :151 */
+    int r = oracle_matmul(x, transX, xDims, xOrder, w, transW, wDims, wOrder,
+                          tmp, cDims, order, alpha, 0);
+    if (r != 0) {
+        free(tmp);
+        return -1;
+    }
+
+    int n;
+    if (bOrder == 0) {
+        /* :74-75 (first overload only): ScaleAndShift(tmp, c, 1, b) */
+        if (transX != ORACLE_X_NOTRANS || transW != ORACLE_X_NOTRANS) {
+            free(tmp);
+            return -2;
+        }
+        for (long i = 0; i < num; i++)
+            c[i] = tmp[i] * 1.0F + bias[0];
+        n = order;   /* no broadcast dimension */
+    }
+    else {
+        /* :77-92 */
+        n = oracle_broadcast_dim_index(cDims, order, bDims, bOrder);
+        if (n < 0 || n >= order) {
+            free(tmp);
+            return -2;   /* the reference aborts here ("TODO!") */
+        }
+        if (oracle_sumdim(tmp, cDims, order, bias, (int)unit_num(bDims, bOrder), c, n, 1.0F) != 0) {
+            free(tmp);
+            return -2;
+        }
+    }
+    free(tmp);
+    return n;
+}
+
+/* ---- comparator ---------------------------------------------------------- */
+
+int oracle_is_float_equal(float a, float b, float absError, float relError)
+{
+    /* CheckData.cpp:29-39 */
+    if (a == b)
+        return 1;
+    if (fabs(a - b) < absError)
+        return 1;
+    if (fabs(a) < fabs(b))
+        return fabs((a - b) / b) < relError ? 1 : 0;
+    else
+        return fabs((a - b) / a) < relError ? 1 : 0;
+}
+
+int oracle_check_data(const float *value, const float *answer, int num, float tolerance)
+{
+    for (int i = 0; i < num; i++)
+        if (!oracle_is_float_equal(value[i], answer[i], tolerance, 1e-4F))
+            return 0;
+    return 1;
+}
+
+/* ---- binary16 ------------------------------------------------------------ */
+
+uint16_t oracle_f32_to_f16(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t absx = x & 0x7fffffffu;
+
+    if (absx >= 0x7f800000u)                      /* Inf or NaN */
+        return (uint16_t)(sign | 0x7c00u | (absx > 0x7f800000u ? 0x0200u | ((absx >> 13) & 0x3ffu) : 0));
+    if (absx >= 0x477ff000u)                      /* rounds to >= 65520 => Inf */
+        return (uint16_t)(sign | 0x7c00u);
+    if (absx < 0x33000001u)                       /* <= 2^-25 => 0 (ties to even) */
+        return (uint16_t)sign;
+
+    int exp = (int)(absx >> 23) - 127;
+    uint32_t man = (absx & 0x7fffffu) | 0x800000u;   /* 24-bit significand */
+    int shift;
+    uint32_t base;
+    if (exp < -14) {                              /* sub-normal half */
+        shift = 13 + (-14 - exp);
+        base = 0;
+    }
+    else {
+        shift = 13;
+        base = (uint32_t)(exp + 15) << 10;
+        man &= 0x7fffffu;
+    }
+    uint32_t q = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u)))
+        q++;                                      /* a carry moves into the exponent */
+    return (uint16_t)(sign | (base + q));
+}
+
+float oracle_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    uint32_t x;
+    if (exp == 0) {
+        if (man == 0)
+            x = sign;
+        else {
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while (!(man & 0x400u));
+            x = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+        }
+    }
+    else if (exp == 31)
+        x = sign | 0x7f800000u | (man << 13);
+    else
+        x = sign | ((exp + 112u) << 23) | (man << 13);
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+void oracle_f32_to_f16_array(const float *src, uint16_t *dst, long n)
+{
+    for (long i = 0; i < n; i++)
+        dst[i] = oracle_f32_to_f16(src[i]);
+}
+
+void oracle_f16_to_f32_array(const uint16_t *src, float *dst, long n)
+{
+    for (long i = 0; i < n; i++)
+        dst[i] = oracle_f16_to_f32(src[i]);
+}
+
+/* ---- seeded fills -------------------------------------------------------- */
+
+static uint64_t splitmix64(uint64_t *s)
+{
+    uint64_t z = (*s += 0x9e3779b97f4a7c15ull);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+/* 53 random bits -> [0,1) */
+static double u01(uint64_t *s)
+{
+    return (double)(splitmix64(s) >> 11) * (1.0 / 9007199254740992.0);
+}
+
+void oracle_fill_uniform(float *x, long n, uint64_t seed, float lo, float hi)
+{
+    uint64_t s = seed;
+    for (long i = 0; i < n; i++)
+        x[i] = (float)(lo + (hi - lo) * u01(&s));
+}
+
+void oracle_fill_normal(float *x, long n, uint64_t seed, float mean, float std)
+{
+    uint64_t s = seed;
+    for (long i = 0; i < n; i += 2) {
+        double u1 = 1.0 - u01(&s);   /* (0,1] */
+        double u2 = u01(&s);
+        double r = sqrt(-2.0 * log(u1));
+        double t = 6.283185307179586476925286766559 * u2;
+        x[i] = (float)(mean + std * r * cos(t));
+        if (i + 1 < n)
+            x[i + 1] = (float)(mean + std * r * sin(t));
+    }
+}

@@ -1,0 +1,84 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library.
+ *
+ * CPU restatement of the NiuTensor matrix-multiplication family, used only as
+ * the checker for the gfx950 kernels (tests, smoke check, CPU baseline timing).
+ * Nothing in the product library may include or link this.
+ *
+ * Every function names the reference source (relative to the NiuTensor tree)
+ * whose arithmetic and loop order it follows.
+ */
+#ifndef NTS_ORACLE_H
+#define NTS_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* enum values of the reference, source/tensor/XDataType.h:33,36 */
+#define ORACLE_X_TRANS 0
+#define ORACLE_X_NOTRANS 1
+#define ORACLE_X_FLOAT 2
+#define ORACLE_X_FLOAT16 3
+
+/* 2-D: c = op(a) op(b) alpha + c beta, fp32, single accumulator, ascending k.
+   na,ma / nb,mb / nc,mc are the STORED row and column counts.
+   Follows MatrixMul2DParallel.cpp:43-129 (TN, NT, TT) and the FAST_MATRIX
+   branch of MatrixMul2DMultiTheading.cpp:59-145 (NN).
+   Returns 0, or -1 when the shapes do not match (MatrixMul2D.cpp:56-67). */
+int oracle_matmul2d(const float *a, int transA, const float *b, int transB, float *c,
+                    int na, int ma, int nb, int mb, int nc, int mc,
+                    float alpha, float beta);
+
+/* Same-order batched product, block i of a times block i of b.
+   Follows MatrixMulBatched.cpp:157-218. dims arrays hold `order` sizes each. */
+int oracle_matmul_batched(const float *a, int transA, const int *aDims,
+                          const float *b, int transB, const int *bDims,
+                          float *c, const int *cDims, int order,
+                          float alpha, float beta);
+
+/* N-D product: flatten rule and (p,q) block pairing of MatrixMul.cpp:52-208. */
+int oracle_matmul(const float *a, int transA, const int *aDims, int aOrder,
+                  const float *b, int transB, const int *bDims, int bOrder,
+                  float *c, const int *cDims, int cOrder,
+                  float alpha, float beta);
+
+/* Sum.cpp:233-260 */
+int oracle_broadcast_dim_index(const int *aDims, int aOrder, const int *bDims, int bOrder);
+
+/* c = a + b*beta, b broadcast along dimension n. CPU branch of SumDim.cpp:49-126. */
+int oracle_sumdim(const float *a, const int *aDims, int aOrder,
+                  const float *b, int bUnitNum, float *c, int n, float beta);
+
+/* c = alpha * op(x) op(w) + bias; MulAndShift.cpp:38-110 and :120-188.
+   cDims/cOrder are outputs (cDims must hold 8 ints). Returns the broadcast
+   dimension n (>=0), or a negative value where the reference aborts. */
+int oracle_mulandshift(const float *x, int transX, const int *xDims, int xOrder,
+                       const float *w, int transW, const int *wDims, int wOrder,
+                       const float *bias, const int *bDims, int bOrder,
+                       float *c, int *cDims, int *cOrder, float alpha);
+
+/* comparator of the reference tests, CheckData.cpp:29-39 */
+int oracle_is_float_equal(float a, float b, float absError, float relError);
+/* CheckData.cpp:78-97 with its fixed relative bound 1e-4 */
+int oracle_check_data(const float *value, const float *answer, int num, float tolerance);
+
+/* IEEE binary16 conversion, round to nearest even. The reference's own CPU
+   conversion is an integer cast (ConvertDataType.cpp:95-106), so this follows
+   IEEE 754 instead and is pinned against numpy.float16 in the tests. */
+uint16_t oracle_f32_to_f16(float f);
+float oracle_f16_to_f32(uint16_t h);
+void oracle_f32_to_f16_array(const float *src, uint16_t *dst, long n);
+void oracle_f16_to_f32_array(const uint16_t *src, float *dst, long n);
+
+/* portable seeded fills (splitmix64); the reference fills with libc rand()
+   (SetData.cpp:484), which is not reproducible across C libraries. */
+void oracle_fill_uniform(float *x, long n, uint64_t seed, float lo, float hi);
+void oracle_fill_normal(float *x, long n, uint64_t seed, float mean, float std);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,154 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library.
+ *
+ * C entry points around the REAL NiuTensor CPU implementation, compiled from
+ * the reference tree where it lies (see the Makefile beside this file). The
+ * resulting library is only used to validate the C restatement in
+ * nts_oracle.c and, optionally, as the CPU baseline. Every tensor here lives
+ * on the host (devID = -1), so the reference takes its naive CPU path
+ * (_MatrixMul2DParallel; no BLAS is linked).
+ */
+#include "XTensor.h"
+#include "XCall.h"
+#include "core/CHeader.h"
+#include "test/TMatrixMul.h"
+#include "test/TMatrixMul2D.h"
+#include "test/TMatrixMul2DParallel.h"
+#include "test/TMatrixMulBatched.h"
+#include "test/TSumDim.h"
+
+#include <string.h>
+
+using namespace nts;
+
+static XTensor * Make(const int * dims, int order, const float * data)
+{
+    XTensor * t = NewTensorV2(order, dims, X_FLOAT, 1.0F, -1, NULL);
+    if (data != NULL)
+        t->SetData(data, t->unitNum);
+    return t;
+}
+
+extern "C" {
+
+int ref_matmul2d(const float * a, int transA, const float * b, int transB, float * c,
+                 int na, int ma, int nb, int mb, int nc, int mc, float alpha, float beta)
+{
+    int ad[2] = {na, ma}, bd[2] = {nb, mb}, cd[2] = {nc, mc};
+    XTensor * ta = Make(ad, 2, a);
+    XTensor * tb = Make(bd, 2, b);
+    XTensor * tc = Make(cd, 2, c);
+    _MatrixMul2D(ta, (MATRIX_TRANS_TYPE)transA, tb, (MATRIX_TRANS_TYPE)transB, tc, alpha, beta);
+    memcpy(c, tc->data, sizeof(float) * (size_t)tc->unitNum);
+    delete ta; delete tb; delete tc;
+    return 0;
+}
+
+int ref_matmul(const float * a, int transA, const int * aDims, int aOrder,
+               const float * b, int transB, const int * bDims, int bOrder,
+               float * c, const int * cDims, int cOrder, float alpha, float beta)
+{
+    XTensor * ta = Make(aDims, aOrder, a);
+    XTensor * tb = Make(bDims, bOrder, b);
+    XTensor * tc = Make(cDims, cOrder, c);
+    _MatrixMul(ta, (MATRIX_TRANS_TYPE)transA, tb, (MATRIX_TRANS_TYPE)transB, tc, alpha, beta);
+    memcpy(c, tc->data, sizeof(float) * (size_t)tc->unitNum);
+    delete ta; delete tb; delete tc;
+    return 0;
+}
+
+int ref_matmul_batched(const float * a, int transA, const int * aDims,
+                       const float * b, int transB, const int * bDims,
+                       float * c, const int * cDims, int order, float alpha, float beta)
+{
+    XTensor * ta = Make(aDims, order, a);
+    XTensor * tb = Make(bDims, order, b);
+    XTensor * tc = Make(cDims, order, c);
+    _MatrixMulBatched(ta, (MATRIX_TRANS_TYPE)transA, tb, (MATRIX_TRANS_TYPE)transB, tc, alpha, beta);
+    memcpy(c, tc->data, sizeof(float) * (size_t)tc->unitNum);
+    delete ta; delete tb; delete tc;
+    return 0;
+}
+
+/* the allocating wrapper: returns the order of the result, fills cDims and c */
+int ref_matmul_alloc(const float * a, int transA, const int * aDims, int aOrder,
+                     const float * b, int transB, const int * bDims, int bOrder,
+                     float * c, int * cDims, float alpha)
+{
+    XTensor * ta = Make(aDims, aOrder, a);
+    XTensor * tb = Make(bDims, bOrder, b);
+    XTensor tc = MatrixMul(*ta, (MATRIX_TRANS_TYPE)transA, *tb, (MATRIX_TRANS_TYPE)transB, alpha);
+    for (int i = 0; i < tc.order; i++)
+        cDims[i] = tc.dimSize[i];
+    memcpy(c, tc.data, sizeof(float) * (size_t)tc.unitNum);
+    int order = tc.order;
+    delete ta; delete tb;
+    return order;
+}
+
+int ref_broadcast_dim_index(const int * aDims, int aOrder, const int * bDims, int bOrder)
+{
+    XTensor * ta = Make(aDims, aOrder, NULL);
+    XTensor * tb = Make(bDims, bOrder, NULL);
+    int n = GetBroadcastDimIndex(*ta, *tb);
+    delete ta; delete tb;
+    return n;
+}
+
+int ref_sumdim(const float * a, const int * aDims, int aOrder,
+               const float * b, const int * bDims, int bOrder, float * c, int n, float beta)
+{
+    XTensor * ta = Make(aDims, aOrder, a);
+    XTensor * tb = Make(bDims, bOrder, b);
+    XTensor * tc = Make(aDims, aOrder, NULL);
+    _SumDim(ta, tb, tc, n, beta);
+    memcpy(c, tc->data, sizeof(float) * (size_t)tc->unitNum);
+    delete ta; delete tb; delete tc;
+    return 0;
+}
+
+/* overload == 1: MulAndShift(x, w, b, alpha); overload == 2: with transpose flags.
+   Returns the order of the result. */
+int ref_mulandshift(int overload,
+                    const float * x, int transX, const int * xDims, int xOrder,
+                    const float * w, int transW, const int * wDims, int wOrder,
+                    const float * bias, const int * bDims, int bOrder,
+                    float * c, int * cDims, float alpha)
+{
+    XTensor * tx = Make(xDims, xOrder, x);
+    XTensor * tw = Make(wDims, wOrder, w);
+    XTensor * tb = Make(bDims, bOrder, bias);
+    XTensor tc;
+    if (overload == 1)
+        tc = MulAndShift(*tx, *tw, *tb, alpha);
+    else
+        tc = MulAndShift(*tx, (MATRIX_TRANS_TYPE)transX, *tw, (MATRIX_TRANS_TYPE)transW, *tb, alpha);
+    for (int i = 0; i < tc.order; i++)
+        cDims[i] = tc.dimSize[i];
+    memcpy(c, tc.data, sizeof(float) * (size_t)tc.unitNum);
+    int order = tc.order;
+    delete tx; delete tw; delete tb;
+    return order;
+}
+
+/* the reference's own known-answer tests for this path; bit i set = suite i passed */
+int ref_run_matmul_tests()
+{
+    int ok = 0;
+    if (TestMatrixMul()) ok |= 1;
+    if (TestMatrixMul2D()) ok |= 2;
+    if (TestMatrixMul2DParallel()) ok |= 4;
+    if (TestMatrixMulBatched()) ok |= 8;
+    if (TestSumDim()) ok |= 16;
+    return ok;
+}
+
+int ref_enum_values(int * out)
+{
+    out[0] = (int)X_TRANS; out[1] = (int)X_NOTRANS;
+    out[2] = (int)X_FLOAT; out[3] = (int)X_FLOAT16;
+    out[4] = (int)sizeof(XTensor);
+    return 0;
+}
+
+}

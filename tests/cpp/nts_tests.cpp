@@ -1,0 +1,478 @@
+/*
+ * Tests of the nts:: host layer on a gfx950 GPU, written the way the reference
+ * writes its own (source/tensor/test/TMatrixMul.cpp, TMatrixMul2D.cpp,
+ * TMatrixMulBatched.cpp): literal inputs, the operation, a comparison with the
+ * known answer through the reference's comparator (abs 1e-4 or rel 1e-4,
+ * core/utilities/CheckData.cpp:29-39). The GPU halves of those tests are what is
+ * reproduced here; cases the reference does not have (NT/TT, alpha/beta, fp16,
+ * MulAndShift, lists) are checked against the CPU oracle on seeded inputs.
+ *
+ *   nts_tests                run everything on device 0, exit 0 if all passed
+ *   nts_tests --abort NAME   provoke one fatal error (no GPU needed): the process
+ *                            must print the reference's message and abort
+ */
+#include "../../niutensor_amd/nts/XTensor.h"
+#include "../../niutensor_amd/nts/MatrixMul.h"
+#include "../../niutensor_amd/nts/MatrixMul2D.h"
+#include "../../niutensor_amd/nts/MatrixMulBatched.h"
+#include "../../niutensor_amd/nts/MulAndShift.h"
+#include "../../oracle/nts_oracle.h"
+
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <vector>
+
+using namespace nts;
+
+static const int DEV = 0;
+
+/* _CheckData of the reference for a device tensor: read back, compare element-wise */
+static bool CheckData(const XTensor * t, const void * answer, int num, float tolerance)
+{
+    if (t->data == NULL || answer == NULL || num != t->unitNum)
+        return false;
+    std::vector<float> host(num);
+    t->GetData(host.data());
+    return oracle_check_data(host.data(), (const float *)answer, num, tolerance) != 0;
+}
+
+static XTensor * NewGPU(int order, const int * dims, const float * data, TENSOR_DATA_TYPE type = X_FLOAT)
+{
+    XTensor * t = NewTensorV2(order, dims, type, 1.0F, DEV);
+    if (data != NULL) {
+        if (type == X_FLOAT)
+            t->SetData(data, t->unitNum);
+        else {
+            std::vector<uint16_t> h(t->unitNum);
+            oracle_f32_to_f16_array(data, h.data(), t->unitNum);
+            t->SetData(h.data(), t->unitNum);
+        }
+    }
+    return t;
+}
+
+/* ---- the reference's known-answer cases, GPU halves ------------------------- */
+
+/* TMatrixMul.cpp case 1 / TMatrixMul2D.cpp case 1 / TMatrixMulBatched.cpp case 1: (2,3) x (3,2) */
+static bool TestMatrixMul1()
+{
+    int d1[2] = {2, 3}, d2[2] = {3, 2}, dt[2] = {2, 2};
+    DTYPE sData1[2][3] = {{1.0F, 2.0F, 3.0F}, {-4.0F, 5.0F, 6.0F}};
+    DTYPE sData2[3][2] = {{0.0F, -1.0F}, {1.0F, 2.0F}, {2.0F, 1.0F}};
+    DTYPE answer[2][2] = {{8.0F, 6.0F}, {17.0F, 20.0F}};
+
+    XTensor * s1 = NewGPU(2, d1, &sData1[0][0]);
+    XTensor * s2 = NewGPU(2, d2, &sData2[0][0]);
+    XTensor * t = NewGPU(2, dt, NULL);
+    XTensor * t2 = NewGPU(2, dt, NULL);
+    XTensor * t3 = NewGPU(2, dt, NULL);
+    XTensor tUser, tUserB;
+    t->SetZeroAll();
+
+    _MatrixMul(s1, X_NOTRANS, s2, X_NOTRANS, t);
+    tUser = MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS);
+    _MatrixMul2D(s1, X_NOTRANS, s2, X_NOTRANS, t2);
+    _MatrixMulBatched(s1, X_NOTRANS, s2, X_NOTRANS, t3);
+    tUserB = MatrixMulBatched(*s1, X_NOTRANS, *s2, X_NOTRANS);
+
+    bool ok = CheckData(t, answer, 4, 1e-4F) && CheckData(&tUser, answer, 4, 1e-4F) &&
+              CheckData(t2, answer, 4, 1e-4F) && CheckData(t3, answer, 4, 1e-4F) &&
+              CheckData(&tUserB, answer, 4, 1e-4F);
+    delete s1; delete s2; delete t; delete t2; delete t3;
+    return ok;
+}
+
+/* TMatrixMul.cpp case 2 / TMatrixMul2D.cpp case 2: a stored (3,2), X_TRANS */
+static bool TestMatrixMul2()
+{
+    int d1[2] = {3, 2}, d2[2] = {3, 2}, dt[2] = {2, 2};
+    DTYPE sData1[3][2] = {{1.0F, -4.0F}, {2.0F, 5.0F}, {3.0F, 6.0F}};
+    DTYPE sData2[3][2] = {{0.0F, -1.0F}, {1.0F, 2.0F}, {2.0F, 1.0F}};
+    DTYPE answer[2][2] = {{8.0F, 6.0F}, {17.0F, 20.0F}};
+
+    XTensor * s1 = NewGPU(2, d1, &sData1[0][0]);
+    XTensor * s2 = NewGPU(2, d2, &sData2[0][0]);
+    XTensor * t = NewGPU(2, dt, NULL);
+    XTensor * t2 = NewGPU(2, dt, NULL);
+    XTensor tUser;
+
+    _MatrixMul(s1, X_TRANS, s2, X_NOTRANS, t);
+    tUser = MatrixMul(*s1, X_TRANS, *s2, X_NOTRANS);
+    _MatrixMul2D(s1, X_TRANS, s2, X_NOTRANS, t2);
+
+    bool ok = CheckData(t, answer, 4, 1e-4F) && CheckData(&tUser, answer, 4, 1e-4F) && CheckData(t2, answer, 4, 1e-4F);
+    delete s1; delete s2; delete t; delete t2;
+    return ok;
+}
+
+static DTYPE sData323[3][2][3] = {{{0.0F, -1.0F, 2.0F}, {2.0F, 1.0F, 3.0F}},
+                                  {{1.0F, 2.0F, 4.0F}, {3.0F, 1.0F, 2.0F}},
+                                  {{-1.0F, 3.0F, 2.0F}, {1.0F, -1.0F, 0.0F}}};
+static DTYPE sData232[2][3][2] = {{{1.0F, 2.0F}, {-4.0F, 3.0F}, {2.0F, 6.0F}},
+                                  {{1.0F, 2.0F}, {3.0F, 4.0F}, {5.0F, 6.0F}}};
+
+/* TMatrixMul.cpp case 3: (3,2,3) x (2,3,2) -> (3,2,2,2), every block of a with every block of b */
+static bool TestMatrixMul3()
+{
+    int d1[3] = {3, 2, 3}, d2[3] = {2, 3, 2}, dt[4] = {3, 2, 2, 2};
+    DTYPE answer[3][2][2][2] = {{{{8.0F, 9.0F}, {4.0F, 25.0F}}, {{7.0F, 8.0F}, {20.0F, 26.0F}}},
+                                {{{1.0F, 32.0F}, {3.0F, 21.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}},
+                                {{{-9.0F, 19.0F}, {5.0F, -1.0F}}, {{18.0F, 22.0F}, {-2.0F, -2.0F}}}};
+    XTensor * s1 = NewGPU(3, d1, &sData323[0][0][0]);
+    XTensor * s2 = NewGPU(3, d2, &sData232[0][0][0]);
+    XTensor * t = NewGPU(4, dt, NULL);
+    XTensor tUser;
+
+    _MatrixMul(s1, X_NOTRANS, s2, X_NOTRANS, t);
+    tUser = MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS);
+
+    bool ok = CheckData(t, answer, 24, 1e-4F) && CheckData(&tUser, answer, 24, 1e-4F) &&
+              tUser.order == 4 && tUser.dimSize[0] == 3 && tUser.dimSize[1] == 2;
+    delete s1; delete s2; delete t;
+    return ok;
+}
+
+/* TMatrixMul.cpp case 4: (3,2,3) x (3,2) -> (3,2,2), the flattened product */
+static bool TestMatrixMul4()
+{
+    int d1[3] = {3, 2, 3}, d2[2] = {3, 2}, dt[3] = {3, 2, 2};
+    DTYPE sData2[3][2] = {{1.0F, 2.0F}, {3.0F, 4.0F}, {5.0F, 6.0F}};
+    DTYPE answer[3][2][2] = {{{7.0F, 8.0F}, {20.0F, 26.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}, {{18.0F, 22.0F}, {-2.0F, -2.0F}}};
+    XTensor * s1 = NewGPU(3, d1, &sData323[0][0][0]);
+    XTensor * s2 = NewGPU(2, d2, &sData2[0][0]);
+    XTensor * t = NewGPU(3, dt, NULL);
+    XTensor tUser;
+
+    _MatrixMul(s1, X_NOTRANS, s2, X_NOTRANS, t);
+    tUser = MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS);
+
+    bool ok = CheckData(t, answer, 12, 1e-4F) && CheckData(&tUser, answer, 12, 1e-4F);
+    delete s1; delete s2; delete t;
+    return ok;
+}
+
+/* TMatrixMulBatched.cpp case 2: (2,2,3) x (2,3,2) -> (2,2,2), block i with block i */
+static bool TestMatrixMulBatched2()
+{
+    int d1[3] = {2, 2, 3}, d2[3] = {2, 3, 2}, dt[3] = {2, 2, 2};
+    DTYPE answer[2][2][2] = {{{8.0F, 9.0F}, {4.0F, 25.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}};
+    XTensor * s1 = NewGPU(3, d1, &sData323[0][0][0]);
+    XTensor * s2 = NewGPU(3, d2, &sData232[0][0][0]);
+    XTensor * t = NewGPU(3, dt, NULL);
+    XTensor tUser;
+
+    _MatrixMulBatched(s1, X_NOTRANS, s2, X_NOTRANS, t);
+    tUser = MatrixMulBatched(*s1, X_NOTRANS, *s2, X_NOTRANS);
+
+    bool ok = CheckData(t, answer, 8, 1e-4F) && CheckData(&tUser, answer, 8, 1e-4F);
+    delete s1; delete s2; delete t;
+    return ok;
+}
+
+/* ---- seeded cases against the CPU oracle ------------------------------------- */
+
+static float MaxRelErr(const std::vector<float> & got, const std::vector<float> & ref)
+{
+    float mx = 0;
+    for (size_t i = 0; i < ref.size(); i++)
+        mx = fmaxf(mx, fabsf(ref[i]));
+    float e = 0;
+    for (size_t i = 0; i < ref.size(); i++)
+        e = fmaxf(e, fabsf(got[i] - ref[i]) / mx);
+    return e;
+}
+
+static int Prod(const int * d, int n)
+{
+    int p = 1;
+    for (int i = 0; i < n; i++)
+        p *= d[i];
+    return p;
+}
+
+/* all four transposes with alpha, beta and ragged sizes: fp32 within 1e-5 * sqrt(K) of the oracle */
+static bool TestMatrixMulSeeded()
+{
+    bool ok = true;
+    int sizes[4][3] = {{37, 29, 53}, {130, 70, 33}, {256, 128, 64}, {5, 300, 17}};
+    for (int s = 0; s < 4; s++) {
+        int M = sizes[s][0], N = sizes[s][1], K = sizes[s][2];
+        for (int ta = 0; ta < 2; ta++) {
+            for (int tb = 0; tb < 2; tb++) {
+                int da[2] = {ta == X_TRANS ? K : M, ta == X_TRANS ? M : K};
+                int db[2] = {tb == X_TRANS ? N : K, tb == X_TRANS ? K : N};
+                int dc[2] = {M, N};
+                std::vector<float> a(M * K), b(K * N), c0(M * N), ref(M * N), got(M * N);
+                oracle_fill_uniform(a.data(), M * K, 100 + s, -1, 1);
+                oracle_fill_uniform(b.data(), K * N, 200 + s, -1, 1);
+                oracle_fill_uniform(c0.data(), M * N, 300 + s, -1, 1);
+                ref = c0;
+                oracle_matmul2d(a.data(), ta, b.data(), tb, ref.data(), da[0], da[1], db[0], db[1], M, N, 0.5F, 1.0F);
+                XTensor * ga = NewGPU(2, da, a.data());
+                XTensor * gb = NewGPU(2, db, b.data());
+                XTensor * gc = NewGPU(2, dc, c0.data());
+                _MatrixMul(ga, (MATRIX_TRANS_TYPE)ta, gb, (MATRIX_TRANS_TYPE)tb, gc, 0.5F, 1.0F);
+                gc->GetData(got.data());
+                float e = MaxRelErr(got, ref);
+                if (!(e <= 1e-5F * sqrtf((float)K))) {
+                    fprintf(stderr, "seeded %dx%dx%d ta=%d tb=%d err=%g\n", M, N, K, ta, tb, e);
+                    ok = false;
+                }
+                delete ga; delete gb; delete gc;
+            }
+        }
+    }
+    return ok;
+}
+
+/* a transposed N-D a against one matrix is NOT flattened: a batch that shares b */
+static bool TestMatrixMulTransposedND()
+{
+    int da[3] = {4, 6, 10}, db[2] = {6, 7}, dc[3] = {4, 10, 7};
+    std::vector<float> a(240), b(42), ref(280), got(280);
+    oracle_fill_uniform(a.data(), 240, 1, -1, 1);
+    oracle_fill_uniform(b.data(), 42, 2, -1, 1);
+    oracle_matmul(a.data(), X_TRANS, da, 3, b.data(), X_NOTRANS, db, 2, ref.data(), dc, 3, 1.0F, 0.0F);
+    XTensor * ga = NewGPU(3, da, a.data());
+    XTensor * gb = NewGPU(2, db, b.data());
+    XTensor tUser = MatrixMul(*ga, X_TRANS, *gb, X_NOTRANS);
+    bool ok = tUser.order == 3 && tUser.dimSize[0] == 4 && tUser.dimSize[1] == 10 && tUser.dimSize[2] == 7;
+    tUser.GetData(got.data());
+    ok = ok && MaxRelErr(got, ref) < 1e-5F;
+    delete ga; delete gb;
+    return ok;
+}
+
+/* attention-shaped batch: S = Q K^T / 8, then S V */
+static bool TestMatrixMulBatchedAttention()
+{
+    int dq[3] = {6, 50, 24}, dk[3] = {6, 40, 24}, ds[3] = {6, 50, 40}, dv[3] = {6, 40, 24}, dout[3] = {6, 50, 24};
+    std::vector<float> q(Prod(dq, 3)), k(Prod(dk, 3)), v(Prod(dv, 3)), s(Prod(ds, 3)), o(Prod(dout, 3));
+    oracle_fill_normal(q.data(), q.size(), 1, 0, 1);
+    oracle_fill_normal(k.data(), k.size(), 2, 0, 1);
+    oracle_fill_normal(v.data(), v.size(), 3, 0, 1);
+    oracle_matmul_batched(q.data(), X_NOTRANS, dq, k.data(), X_TRANS, dk, s.data(), ds, 3, 0.125F, 0.0F);
+    oracle_matmul_batched(s.data(), X_NOTRANS, ds, v.data(), X_NOTRANS, dv, o.data(), dout, 3, 1.0F, 0.0F);
+    XTensor * gq = NewGPU(3, dq, q.data());
+    XTensor * gk = NewGPU(3, dk, k.data());
+    XTensor * gv = NewGPU(3, dv, v.data());
+    XTensor gs = BMMul(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+    XTensor go = BMMul(gs, *gv);
+    std::vector<float> hs(s.size()), ho(o.size());
+    gs.GetData(hs.data());
+    go.GetData(ho.data());
+    bool ok = MaxRelErr(hs, s) < 8e-5F && MaxRelErr(ho, o) < 8e-5F;
+    delete gq; delete gk; delete gv;
+    return ok;
+}
+
+/* MulAndShift: last-dimension bias (fused column add), an earlier-dimension bias,
+   the transposed overload, a scalar bias; and the autograd edge it records */
+static bool TestMulAndShift()
+{
+    bool ok = true;
+    int dx[3] = {4, 6, 10}, dw[2] = {10, 8};
+    std::vector<float> x(240), w(80), ref(192), got(192);
+    oracle_fill_uniform(x.data(), 240, 21, -1, 1);
+    oracle_fill_normal(w.data(), 80, 22, 0, 0.02F);
+    XTensor * gx = NewGPU(3, dx, x.data());
+    XTensor * gw = NewGPU(2, dw, w.data());
+    gw->enableGrad = true;
+
+    int biasShapes[4][3] = {{8, 0, 0}, {1, 8, 0}, {6, 0, 0}, {4, 1, 1}};
+    int biasOrders[4] = {1, 2, 1, 3};
+    int expectN[4] = {2, 2, 1, 0};
+    for (int i = 0; i < 4; i++) {
+        int nb = Prod(biasShapes[i], biasOrders[i]);
+        std::vector<float> bias(nb);
+        oracle_fill_normal(bias.data(), nb, 23 + i, 0, 0.02F);
+        int cd[8], co = 0;
+        int n = oracle_mulandshift(x.data(), X_NOTRANS, dx, 3, w.data(), X_NOTRANS, dw, 2,
+                                   bias.data(), biasShapes[i], biasOrders[i], ref.data(), cd, &co, 0.5F);
+        XTensor * gb = NewGPU(biasOrders[i], biasShapes[i], bias.data());
+        gb->enableGrad = true;
+        XTensor c = MulAndShift(*gx, *gw, *gb, 0.5F);
+        c.GetData(got.data());
+        bool shape = c.order == 3 && c.dimSize[0] == 4 && c.dimSize[1] == 6 && c.dimSize[2] == 8;
+        bool edge = c.income.typeID == MATH_MULANDSHIFT && c.income.tailNum == 3 && c.income.paramNum == 4 &&
+                    c.income.params[0].i == n && c.income.params[1].i == X_NOTRANS && c.income.params[3].f == 0.5F;
+        float e = MaxRelErr(got, ref);
+        if (!(shape && edge && n == expectN[i] && e < 4e-5F)) {
+            fprintf(stderr, "mulandshift bias %d: n=%d shape=%d edge=%d err=%g\n", i, n, shape, edge, e);
+            ok = false;
+        }
+        delete gb;
+    }
+
+    /* the overload with transpose flags: w stored (8, 10) */
+    {
+        std::vector<float> wt(80), bias(8);
+        for (int i = 0; i < 10; i++)
+            for (int j = 0; j < 8; j++)
+                wt[j * 10 + i] = w[i * 8 + j];
+        oracle_fill_normal(bias.data(), 8, 30, 0, 0.02F);
+        int dwt[2] = {8, 10}, dbias[1] = {8}, cd[8], co = 0;
+        oracle_mulandshift(x.data(), X_NOTRANS, dx, 3, wt.data(), X_TRANS, dwt, 2, bias.data(), dbias, 1, ref.data(), cd, &co, 1.0F);
+        XTensor * gwt = NewGPU(2, dwt, wt.data());
+        XTensor * gb = NewGPU(1, dbias, bias.data());
+        XTensor c = MulAndShift(*gx, X_NOTRANS, *gwt, X_TRANS, *gb);
+        c.GetData(got.data());
+        if (!(MaxRelErr(got, ref) < 4e-5F && c.income.tailNum == 0))
+            ok = false;
+        delete gwt; delete gb;
+    }
+
+    /* scalar bias (order 0), first overload only */
+    {
+        float shift = 0.25F;
+        int none[1] = {0};
+        XTensor * gb = NewGPU(0, none, &shift);
+        int cd[8], co = 0;
+        oracle_mulandshift(x.data(), X_NOTRANS, dx, 3, w.data(), X_NOTRANS, dw, 2, &shift, none, 0, ref.data(), cd, &co, 1.0F);
+        XTensor c = MulAndShift(*gx, *gw, *gb);
+        c.GetData(got.data());
+        if (!(MaxRelErr(got, ref) < 4e-5F))
+            ok = false;
+        delete gb;
+    }
+    delete gx; delete gw;
+    return ok;
+}
+
+/* fp16 tensors: fp32 accumulation, result within 1e-2 of the fp32 oracle on the rounded inputs */
+static bool TestMatrixMulHalf()
+{
+    bool ok = true;
+    int M = 96, N = 80, K = 72;
+    for (int ta = 0; ta < 2; ta++) {
+        for (int tb = 0; tb < 2; tb++) {
+            int da[2] = {ta == X_TRANS ? K : M, ta == X_TRANS ? M : K};
+            int db[2] = {tb == X_TRANS ? N : K, tb == X_TRANS ? K : N};
+            int dc[2] = {M, N};
+            std::vector<float> a(M * K), b(K * N), ref(M * N), got(M * N);
+            std::vector<uint16_t> h(M * N);
+            oracle_fill_normal(a.data(), M * K, 41, 0, 0.5F);
+            oracle_fill_normal(b.data(), K * N, 42, 0, 0.5F);
+            /* round the inputs to half first: both sides then multiply the same numbers */
+            std::vector<uint16_t> ha(M * K), hb(K * N);
+            oracle_f32_to_f16_array(a.data(), ha.data(), M * K);
+            oracle_f16_to_f32_array(ha.data(), a.data(), M * K);
+            oracle_f32_to_f16_array(b.data(), hb.data(), K * N);
+            oracle_f16_to_f32_array(hb.data(), b.data(), K * N);
+            oracle_matmul2d(a.data(), ta, b.data(), tb, ref.data(), da[0], da[1], db[0], db[1], M, N, 1.0F, 0.0F);
+            XTensor * ga = NewGPU(2, da, a.data(), X_FLOAT16);
+            XTensor * gb = NewGPU(2, db, b.data(), X_FLOAT16);
+            XTensor * gc = NewGPU(2, dc, NULL, X_FLOAT16);
+            _MatrixMul2D(ga, (MATRIX_TRANS_TYPE)ta, gb, (MATRIX_TRANS_TYPE)tb, gc);
+            gc->GetData(h.data());
+            oracle_f16_to_f32_array(h.data(), got.data(), M * N);
+            float e = MaxRelErr(got, ref);
+            if (!(e < 1e-2F)) {
+                fprintf(stderr, "half ta=%d tb=%d err=%g\n", ta, tb, e);
+                ok = false;
+            }
+            delete ga; delete gb; delete gc;
+        }
+    }
+    return ok;
+}
+
+/* the edge a product records for autograd, and the wrapper that reuses a formed c */
+static bool TestMatrixMulLinkAndReuse()
+{
+    int d1[2] = {2, 3}, d2[2] = {3, 2};
+    DTYPE sData1[2][3] = {{1.0F, 2.0F, 3.0F}, {-4.0F, 5.0F, 6.0F}};
+    DTYPE sData2[3][2] = {{0.0F, -1.0F}, {1.0F, 2.0F}, {2.0F, 1.0F}};
+    DTYPE twice[2][2] = {{16.0F, 12.0F}, {34.0F, 40.0F}};
+    XTensor * s1 = NewGPU(2, d1, &sData1[0][0]);
+    XTensor * s2 = NewGPU(2, d2, &sData2[0][0]);
+    s1->enableGrad = true;
+    s2->enableGrad = true;
+    XTensor c;
+    MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS, c, 1.0F, 0.0F);     /* forms c */
+    MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS, c, 1.0F, 1.0F);     /* accumulates into it */
+    bool ok = CheckData(&c, twice, 4, 1e-4F);
+    ok = ok && c.income.typeID == MATH_MATRIXMUL && c.income.tailNum == 2 && c.income.tails[0] == s1 &&
+         c.income.paramNum == 3 && c.income.params[0].i == X_NOTRANS && c.income.params[2].f == 1.0F;
+    XTensor d = MatrixMulBatched(*s1, X_NOTRANS, *s2, X_NOTRANS, 2.0F);
+    ok = ok && d.income.typeID == MATH_MATRIXMULBATCHED && d.income.params[2].f == 2.0F && CheckData(&d, twice, 4, 1e-4F);
+    s1->enableGrad = false;
+    XTensor e = MatrixMul(*s1, *s2);
+    ok = ok && e.income.tailNum == 0;
+    delete s1; delete s2;
+    return ok;
+}
+
+/* beta == 0 must not let the old contents of c through (the reference zeroes c first) */
+static bool TestBetaZeroIgnoresOldContents()
+{
+    int d1[2] = {64, 32}, d2[2] = {32, 48}, dt[2] = {64, 48};
+    std::vector<float> a(64 * 32), b(32 * 48), junk(64 * 48, NAN), ref(64 * 48), got(64 * 48);
+    oracle_fill_uniform(a.data(), a.size(), 51, -1, 1);
+    oracle_fill_uniform(b.data(), b.size(), 52, -1, 1);
+    oracle_matmul2d(a.data(), X_NOTRANS, b.data(), X_NOTRANS, ref.data(), 64, 32, 32, 48, 64, 48, 1.0F, 0.0F);
+    XTensor * ga = NewGPU(2, d1, a.data());
+    XTensor * gb = NewGPU(2, d2, b.data());
+    XTensor * gc = NewGPU(2, dt, junk.data());
+    _MatrixMul(ga, X_NOTRANS, gb, X_NOTRANS, gc);
+    gc->GetData(got.data());
+    bool ok = MaxRelErr(got, ref) < 6e-5F;
+    delete ga; delete gb; delete gc;
+    return ok;
+}
+
+/* ---- fatal errors: same message, same ending as the reference ---------------- */
+
+static int Provoke(const char * name)
+{
+    /* view tensors (a negative size: shape only, no allocation) on device 0:
+       every check below fires before the GPU is touched */
+    int d23[2] = {-2, 3}, d32[2] = {-3, 2}, d22[2] = {-2, 2}, d223[3] = {-2, 2, 3};
+    XTensor a(2, d23, X_FLOAT, 1.0F, 0, NULL), b(2, d32, X_FLOAT, 1.0F, 0, NULL), c(2, d22, X_FLOAT, 1.0F, 0, NULL);
+    XTensor h(2, d32, X_FLOAT16, 1.0F, 0, NULL), t3(3, d223, X_FLOAT, 1.0F, 0, NULL);
+    XTensor host(2, d22, X_FLOAT, 1.0F, -1, NULL);
+    if (!strcmp(name, "unmatched"))
+        _MatrixMul2D(&a, X_NOTRANS, &a, X_NOTRANS, &c);
+    else if (!strcmp(name, "datatype"))
+        _MatrixMul(&a, X_NOTRANS, &h, X_NOTRANS, &c);
+    else if (!strcmp(name, "order"))
+        _MatrixMulBatched(&t3, X_NOTRANS, &b, X_NOTRANS, &c);
+    else if (!strcmp(name, "wrongorder"))
+        _MatrixMul(&t3, X_NOTRANS, &b, X_NOTRANS, &c);
+    else if (!strcmp(name, "empty"))
+        _MatrixMul(NULL, X_NOTRANS, &b, X_NOTRANS, &c);
+    else if (!strcmp(name, "host"))
+        _MatrixMul2D(&host, X_NOTRANS, &host, X_NOTRANS, &host);
+    else if (!strcmp(name, "biasshape")) {
+        XTensor bias(2, d22, X_FLOAT, 1.0F, 0, NULL);
+        MulAndShift(a, b, bias);
+    }
+    else
+        return 2;
+    return 0;   /* not reached when the error fires */
+}
+
+#define RUN(t) { bool r_ = t(); printf(">> %-36s %s\n", #t, r_ ? "passed" : "FAILED"); fflush(stdout); all = all && r_; }
+
+int main(int argc, char ** argv)
+{
+    if (argc == 3 && !strcmp(argv[1], "--abort"))
+        return Provoke(argv[2]);
+
+    bool all = true;
+    RUN(TestMatrixMul1);
+    RUN(TestMatrixMul2);
+    RUN(TestMatrixMul3);
+    RUN(TestMatrixMul4);
+    RUN(TestMatrixMulBatched2);
+    RUN(TestMatrixMulSeeded);
+    RUN(TestMatrixMulTransposedND);
+    RUN(TestMatrixMulBatchedAttention);
+    RUN(TestMulAndShift);
+    RUN(TestMatrixMulHalf);
+    RUN(TestMatrixMulLinkAndReuse);
+    RUN(TestBetaZeroIgnoresOldContents);
+    printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
+    return all ? 0 : 1;
+}

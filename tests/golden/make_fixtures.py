@@ -1,0 +1,130 @@
+"""Writes tests/golden/ref_generated.npz from the COMPILED reference (oracle/_ref/libnts_ref.so).
+
+Run in a container that holds the NiuTensor tree (`make -C oracle ref` first):
+
+    python tests/golden/make_fixtures.py
+
+The file holds inputs and the outputs the real NiuTensor CPU implementation
+produced for them, for the parts of the path its own tests do not cover:
+NT/TT products, alpha/beta, N-D dispatch (flatten rule, (p,q) pairing, a
+transposed N-D a against a shared 2-D b), the allocating wrapper's result
+shape, GetBroadcastDimIndex, and MulAndShift (no TMulAndShift exists in the
+reference). Only data is stored; the tests compare the C restatement and the
+GPU path against it.
+"""
+import itertools
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle.binding import Oracle, Reference, X_TRANS, X_NOTRANS  # noqa: E402
+
+
+def main():
+    o = Oracle()
+    r = Reference()
+    out = {}
+    index = []
+
+    def put(name, **arrays):
+        index.append(name)
+        for k, v in arrays.items():
+            out["%s/%s" % (name, k)] = np.asarray(v)
+
+    seed = 1000
+
+    # 2-D products: every transpose pair, alpha/beta, ragged sizes
+    for (M, N, K) in ((5, 7, 3), (19, 13, 21), (1, 9, 4), (9, 1, 40)):
+        for ta, tb in itertools.product((X_NOTRANS, X_TRANS), repeat=2):
+            for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+                seed += 3
+                a = o.uniform((K, M) if ta == X_TRANS else (M, K), seed)
+                b = o.uniform((N, K) if tb == X_TRANS else (K, N), seed + 1)
+                c0 = o.uniform((M, N), seed + 2)
+                c = r.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                put("mm2d_%dx%dx%d_%d%d_a%g_b%g" % (M, N, K, ta, tb, alpha, beta), kind="matmul2d",
+                    a=a, b=b, c0=c0, c=c, params=[ta, tb], scal=[alpha, beta])
+
+    # N-D dispatch of _MatrixMul
+    nd_cases = [
+        ((3, 2, 3), X_NOTRANS, (3, 4), X_NOTRANS),          # flatten rule
+        ((2, 3, 5, 4), X_NOTRANS, (6, 4), X_TRANS),         # flatten rule, b transposed
+        ((3, 4, 5), X_TRANS, (4, 6), X_NOTRANS),            # transposed N-D a, shared b: no flattening
+        ((3, 2, 3), X_NOTRANS, (2, 3, 2), X_NOTRANS),       # (p,q) pairing
+        ((2, 4, 3), X_TRANS, (3, 5, 4), X_TRANS),           # (p,q) pairing, both transposed
+        ((2, 2, 3, 4), X_NOTRANS, (2, 4, 5), X_NOTRANS),    # order 4 x order 3
+        ((6, 5), X_NOTRANS, (3, 5, 2), X_NOTRANS),          # 2-D a against N-D b
+    ]
+    for i, (sa, ta, sb, tb) in enumerate(nd_cases):
+        for alpha, beta in ((1.0, 0.0), (0.75, 1.0)):
+            seed += 3
+            a = o.uniform(sa, seed)
+            b = o.uniform(sb, seed + 1)
+            calloc, shape = r.matmul_alloc(a, ta, b, tb, alpha)
+            c0 = o.uniform(shape, seed + 2)
+            c = r.matmul(a, ta, b, tb, c0.copy(), alpha, beta)
+            put("mmnd_%d_a%g_b%g" % (i, alpha, beta), kind="matmul", a=a, b=b, c0=c0, c=c, calloc=calloc,
+                params=[ta, tb], scal=[alpha, beta])
+
+    # same-order batched products
+    for i, (sa, ta, sb, tb) in enumerate([
+        ((4, 6, 5), X_NOTRANS, (4, 7, 5), X_TRANS),
+        ((2, 3, 5, 6), X_TRANS, (2, 3, 5, 4), X_NOTRANS),
+        ((3, 8, 8), X_NOTRANS, (3, 8, 8), X_NOTRANS),
+        ((5, 4, 9), X_TRANS, (5, 3, 4), X_TRANS),
+    ]):
+        for alpha, beta in ((0.125, 0.0), (1.0, 1.0)):
+            seed += 3
+            a = o.uniform(sa, seed)
+            b = o.uniform(sb, seed + 1)
+            c = r.matmul_batched(a, ta, b, tb, None, alpha, 0.0)
+            c0 = o.uniform(c.shape, seed + 2)
+            c = r.matmul_batched(a, ta, b, tb, c0.copy(), alpha, beta)
+            put("bmm_%d_a%g_b%g" % (i, alpha, beta), kind="matmul_batched", a=a, b=b, c0=c0, c=c,
+                params=[ta, tb], scal=[alpha, beta])
+
+    # GetBroadcastDimIndex over small shapes
+    rows = []
+    dims = (1, 2, 3)
+    for ao in (1, 2, 3):
+        for ashape in itertools.product(dims, repeat=ao):
+            for bo in (1, 2, 3):
+                for bshape in itertools.product(dims, repeat=bo):
+                    n = r.broadcast_dim_index(ashape, bshape)
+                    rows.append(list(ashape) + [0] * (3 - ao) + [ao] + list(bshape) + [0] * (3 - bo) + [bo] + [n])
+    put("broadcast_dim_index", kind="broadcast", table=np.array(rows, np.int32))
+
+    # MulAndShift: both overloads; bias on the last dimension and on an earlier one
+    mas = [
+        (1, (6, 5), None, (5, 4), None, (4,), 1.0),
+        (1, (3, 4, 5), None, (5, 7), None, (7,), 1.0),
+        (1, (3, 4, 5), None, (5, 7), None, (1, 7), 0.5),
+        (1, (2, 3, 4, 5), None, (5, 6), None, (6,), 2.0),
+        (1, (3, 4, 5), None, (5, 7), None, (4,), 1.0),            # bias matches dim 1: column broadcast
+        (1, (3, 4, 5), None, (5, 7), None, (3, 1, 1), 1.0),        # bias matches dim 0
+        (1, (7, 7, 5), None, (5, 7), None, (7,), 1.0),             # several dims of size 7: the last one wins
+        (2, (6, 5), X_NOTRANS, (4, 5), X_TRANS, (4,), 1.0),
+        (2, (5, 6), X_TRANS, (5, 4), X_NOTRANS, (4,), 0.5),
+        (2, (3, 4, 5), X_NOTRANS, (7, 5), X_TRANS, (7,), 1.0),
+        (2, (5, 6), X_TRANS, (4, 5), X_TRANS, (6,), 1.0),          # bias matches the row dimension
+    ]
+    for i, (ov, sx, tx, sw, tw, sb, alpha) in enumerate(mas):
+        seed += 3
+        x = o.uniform(sx, seed)
+        w = o.normal(sw, seed + 1, 0.0, 0.5)
+        bias = o.normal(sb, seed + 2, 0.0, 0.5)
+        c = r.mulandshift(x, w, bias, alpha, tx, tw)
+        put("mas_%d" % i, kind="mulandshift", x=x, w=w, bias=bias, c=c,
+            params=[ov, X_NOTRANS if tx is None else tx, X_NOTRANS if tw is None else tw], scal=[alpha])
+
+    out["index"] = np.array(index)
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_generated.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, len(index), "cases", os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,121 @@
+"""The C-ABI boundary without a GPU: the library loads, exports what include/ntsamd_gemm.h
+declares, and rejects bad calls with the reference's messages before touching a device.
+Also the fatal-error behaviour of the nts:: host layer (message to stderr, then abort)."""
+import ctypes as C
+import os
+import re
+import signal
+import subprocess
+
+import pytest
+
+import niutensor_amd as nt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ntsamd_gemm.h")
+NTS_TESTS = os.path.join(ROOT, "tests", "cpp", "build", "nts_tests")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ntsamd_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) == 7
+    assert sorted(nt.EXPORTS) == names
+    lib = C.CDLL(nt.LIB_PATH)
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_no_vendor_blas_is_linked():
+    out = subprocess.run(["ldd", nt.LIB_PATH], capture_output=True, text=True).stdout
+    for banned in ("rocblas", "hipblas", "cublas", "MIOpen", "torch"):
+        assert banned not in out, out
+    out = subprocess.run(["ldd", nt.HOST_LIB_PATH], capture_output=True, text=True).stdout
+    for banned in ("rocblas", "hipblas", "cublas", "nts_oracle", "torch"):
+        assert banned not in out, out
+
+
+def test_version_and_empty_error():
+    L = nt.load()
+    assert L.ntsamd_version().decode() == "0.1"
+
+
+# Every call below must be rejected (or found empty) BEFORE a device is involved: the
+# pointers are made up, so none of these argument lists may describe a runnable product.
+def call_mm(L, ta=nt.X_NOTRANS, tb=nt.X_NOTRANS, types=(2, 2, 2), dims=(2, 3, 3, 2, 2, 2), ptr=0x1000):
+    return L.ntsamd_matrix_mul(0, None, ptr, ta, types[0], ptr, tb, types[1], ptr, types[2], *dims, 1.0, 0.0)
+
+
+def test_argument_errors_need_no_device():
+    L = nt.load()
+    # unsupported data types: X_INT, X_DOUBLE, mixed
+    for types in ((0, 0, 0), (4, 4, 4), (2, 3, 2), (2, 2, 3)):
+        assert call_mm(L, types=types) == 2
+        assert L.ntsamd_last_error().decode() == "Unsupported data type!"
+    # transpose flags are the enum values 0 / 1, nothing else
+    assert call_mm(L, ta=2) == 1
+    assert "X_TRANS (0) or X_NOTRANS (1)" in L.ntsamd_last_error().decode()
+    # shapes that do not multiply, in each transpose layout
+    assert call_mm(L, dims=(2, 3, 2, 3, 2, 3)) == 1
+    assert L.ntsamd_last_error().decode() == "Unmatched matrices in multiplication!"
+    assert call_mm(L, ta=nt.X_TRANS, dims=(2, 3, 3, 2, 2, 2)) == 1
+    assert call_mm(L, dims=(2, 3, 3, 2, 2, 3)) == 1
+    assert call_mm(L, dims=(-2, 3, 3, 2, 2, 2)) == 1
+    # null pointers
+    assert call_mm(L, ptr=None) == 1
+    assert L.ntsamd_last_error().decode() == "Empty matrices in multiplication!"
+    # batch errors
+    rc = L.ntsamd_matrix_mul_batched_strided(0, None, 0x1000, 1, 2, 6, 0x1000, 1, 2, 6, 0x1000, 2, 1,
+                                             3, 2, 3, 3, 2, 2, 2, 1.0, 0.0)
+    assert rc == 1 and "overlap" in L.ntsamd_last_error().decode()
+    rc = L.ntsamd_matrix_mul_batched_strided(0, None, 0x1000, 1, 2, 6, 0x1000, 1, 2, 6, 0x1000, 2, 4,
+                                             -1, 2, 3, 3, 2, 2, 2, 1.0, 0.0)
+    assert rc == 1
+    # bias errors
+    rc = L.ntsamd_matrix_mul_bias(0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 3, 2, 2, 2, 1.0, 0.0,
+                                  0x1000, nt.BIAS_COL, 3, 1)
+    assert rc == 1 and L.ntsamd_last_error().decode() == "Wrong tensor size!"
+    rc = L.ntsamd_matrix_mul_bias(0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 3, 2, 2, 2, 1.0, 0.0,
+                                  None, nt.BIAS_COL, 2, 1)
+    assert rc == 1
+
+
+def test_empty_products_succeed_without_a_device():
+    L = nt.load()
+    # zero rows, zero columns, zero batch items: nothing to do, no device needed
+    assert call_mm(L, dims=(0, 3, 3, 2, 0, 2)) == 0
+    assert call_mm(L, dims=(2, 3, 3, 0, 2, 0)) == 0
+    rc = L.ntsamd_matrix_mul_batched_strided(0, None, 0x1000, 1, 2, 6, 0x1000, 1, 2, 6, 0x1000, 2, 4,
+                                             0, 2, 3, 3, 2, 2, 2, 1.0, 0.0)
+    assert rc == 0
+
+
+def test_invalid_device_is_an_error():
+    L = nt.load()
+    rc = L.ntsamd_init(12345)
+    assert rc == 3 and "device" in L.ntsamd_last_error().decode()
+    rc = L.ntsamd_init(-1)
+    assert rc == 3
+
+
+@pytest.mark.parametrize("case,message", [
+    ("unmatched", "Unmatched tensors in multiplication!"),
+    ("datatype", "Input tensors should have the same data type!"),
+    ("order", "Input tensor and output tensor must have same order!"),
+    ("wrongorder", "wrong tensor order"),
+    ("empty", "Empty input tensors!"),
+    ("host", "does not replace"),
+    ("biasshape", "TODO!"),
+])
+def test_nts_layer_fatal_errors(case, message):
+    """CheckNTErrors / ShowNTErrors of the reference: '[ERROR] ...' on stderr, then std::terminate."""
+    assert os.path.exists(NTS_TESTS), "build tests/cpp first (__graft_entry__.build())"
+    p = subprocess.run([NTS_TESTS, "--abort", case], capture_output=True, text=True, timeout=60)
+    assert p.returncode == -signal.SIGABRT, (p.returncode, p.stderr)
+    assert p.stderr.startswith("[ERROR]"), p.stderr
+    assert message in p.stderr

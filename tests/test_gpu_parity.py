@@ -1,0 +1,471 @@
+"""Parity of the gfx950 kernels with the CPU oracle, through the C ABI.
+
+Same seeded inputs on both sides at sizes the oracle finishes in seconds; the
+committed fixtures (known answers of the reference's tests, outputs of the
+compiled reference); and, at the full benchmark sizes, double-precision checks
+on sampled rows plus size-independent properties (scaling, accumulation,
+transposition). Limits are in tests/tolerance.py.
+"""
+import itertools
+import os
+
+import numpy as np
+import pytest
+
+import niutensor_amd as nt
+from niutensor_amd import BIAS_COL, BIAS_ROW, X_NOTRANS, X_TRANS
+from tolerance import assert_fp16, assert_fp32, fp32_limit, normwise
+
+pytestmark = pytest.mark.gpu
+
+TRANS = list(itertools.product((X_NOTRANS, X_TRANS), repeat=2))
+
+
+def torch_():
+    import torch
+    return torch
+
+
+def dev_tensor(x, gpu, half=False):
+    torch = torch_()
+    t = torch.from_numpy(np.ascontiguousarray(x)).to(gpu)
+    return t.half() if half else t
+
+
+def stored(shape_mk, trans):
+    """Stored shape of an operand whose logical shape is (rows, cols) after trans()."""
+    return (shape_mk[1], shape_mk[0]) if trans == X_TRANS else shape_mk
+
+
+def magnitude(oracle, a, ta, b, tb, alpha, beta=0.0, c0=None, bias=None):
+    mag = abs(alpha) * oracle.matmul2d(np.abs(a), ta, np.abs(b), tb)
+    if beta != 0:
+        mag = mag + abs(beta) * np.abs(c0)
+    if bias is not None:
+        mag = mag + np.abs(bias)
+    return mag
+
+
+@pytest.fixture(autouse=True)
+def name_the_case(request):
+    # a GPU fault can take the box with it: say which test is running first
+    print("\n[gpu-case] %s" % request.node.nodeid, flush=True)
+    os.environ.pop("NTSAMD_TILE_CFG", None)
+    yield
+    os.environ.pop("NTSAMD_TILE_CFG", None)
+
+
+# ---- fixtures held by the reference and by the compiled reference ------------
+
+def test_known_answers_2d(gpu, oracle, known_answers):
+    torch = torch_()
+    for case in known_answers:
+        if case["op"] not in ("matmul2d",) and not (case["op"] in ("matmul", "matmul_batched") and np.ndim(case["a"]) == 2):
+            continue
+        a = dev_tensor(np.array(case["a"], np.float32), gpu)
+        b = dev_tensor(np.array(case["b"], np.float32), gpu)
+        ans = np.array(case["answer"], np.float32)
+        c = torch.full(ans.shape, float("nan"), device=gpu)
+        nt.matrix_mul(a, case["transA"], b, case["transB"], c)
+        assert oracle.check_data(c.cpu().numpy(), ans, 1e-4), case["name"]
+        assert np.array_equal(c.cpu().numpy(), ans), case["name"]
+
+
+def test_known_answers_batched_and_paired(gpu, oracle, known_answers):
+    torch = torch_()
+    by_name = {c["name"]: c for c in known_answers}
+    # TMatrixMulBatched case 2: block i with block i, one strided batch
+    case = by_name["TMatrixMulBatched.case2"]
+    a = dev_tensor(np.array(case["a"], np.float32), gpu)
+    b = dev_tensor(np.array(case["b"], np.float32), gpu)
+    c = torch.empty((2, 2, 2), device=gpu)
+    nt.matrix_mul_batched_strided(a, X_NOTRANS, b, X_NOTRANS, c, 2, 6, 6, 4, 2, 3, 3, 2, 2, 2)
+    assert np.array_equal(c.cpu().numpy(), np.array(case["answer"], np.float32))
+    # TMatrixMul case 3: every block of a with every block of b; not equally spaced, so a pointer list
+    case = by_name["TMatrixMul.case3"]
+    a = dev_tensor(np.array(case["a"], np.float32), gpu)
+    b = dev_tensor(np.array(case["b"], np.float32), gpu)
+    c = torch.empty((3, 2, 2, 2), device=gpu)
+    al, bl, cl = [], [], []
+    for p in range(3):
+        for q in range(2):
+            al.append(a[p]); bl.append(b[q]); cl.append(c[p, q])
+    nt.matrix_mul_batched(al, X_NOTRANS, bl, X_NOTRANS, cl)
+    assert np.array_equal(c.cpu().numpy(), np.array(case["answer"], np.float32))
+    # TMatrixMul case 4: the flattened product
+    case = by_name["TMatrixMul.case4"]
+    a = dev_tensor(np.array(case["a"], np.float32).reshape(6, 3), gpu)
+    b = dev_tensor(np.array(case["b"], np.float32), gpu)
+    c = torch.empty((6, 2), device=gpu)
+    nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c)
+    assert np.array_equal(c.cpu().numpy().reshape(3, 2, 2), np.array(case["answer"], np.float32))
+
+
+def test_compiled_reference_fixture(gpu, generated):
+    """Outputs of the real NiuTensor CPU code (tests/golden/ref_generated.npz)."""
+    torch = torch_()
+    n = 0
+    for name in generated.of_kind("matmul2d"):
+        d = generated.case(name)
+        ta, tb = (int(v) for v in d["params"])
+        alpha, beta = (float(v) for v in d["scal"])
+        c = dev_tensor(d["c0"], gpu)
+        nt.matrix_mul(dev_tensor(d["a"], gpu), ta, dev_tensor(d["b"], gpu), tb, c, alpha, beta)
+        K = d["a"].shape[0] if ta == X_TRANS else d["a"].shape[1]
+        assert_fp32(c.cpu().numpy(), d["c"], K, what=name)
+        n += 1
+    for name in generated.of_kind("matmul_batched"):
+        d = generated.case(name)
+        ta, tb = (int(v) for v in d["params"])
+        alpha, beta = (float(v) for v in d["scal"])
+        a, b, c0 = d["a"], d["b"], d["c0"]
+        c = dev_tensor(c0, gpu)
+        count = int(np.prod(a.shape[:-2]))
+        nt.matrix_mul_batched_strided(dev_tensor(a, gpu), ta, dev_tensor(b, gpu), tb, c, count,
+                                      a.shape[-1] * a.shape[-2], b.shape[-1] * b.shape[-2], c0.shape[-1] * c0.shape[-2],
+                                      a.shape[-2], a.shape[-1], b.shape[-2], b.shape[-1], c0.shape[-2], c0.shape[-1],
+                                      alpha, beta)
+        K = a.shape[-2] if ta == X_TRANS else a.shape[-1]
+        assert_fp32(c.cpu().numpy(), d["c"], K, what=name)
+        n += 1
+    for name in generated.of_kind("mulandshift"):
+        d = generated.case(name)
+        ov, tx, tw = (int(v) for v in d["params"])
+        x, w, bias, cref = d["x"], d["w"], d["bias"], d["c"]
+        if not (tx == X_NOTRANS and w.ndim == 2):
+            continue
+        # the flattened product with the bias in the epilogue, as the host layer issues it
+        rows = int(np.prod(x.shape[:-1]))
+        x2 = dev_tensor(x.reshape(rows, x.shape[-1]), gpu)
+        c = torch.full((rows, cref.shape[-1]), float("nan"), device=gpu)
+        hit = [i for i in range(cref.ndim) if cref.shape[i] == bias.size][-1]
+        if hit == cref.ndim - 1:
+            mode, div = BIAS_COL, 1
+        else:
+            mode, div = BIAS_ROW, int(np.prod(cref.shape[hit + 1:-1]))
+        nt.matrix_mul(x2, tx, dev_tensor(w, gpu), tw, c, float(d["scal"][0]), 0.0,
+                      bias=dev_tensor(bias.ravel(), gpu), bias_mode=mode, bias_row_div=div)
+        assert_fp32(c.cpu().numpy().reshape(cref.shape), cref, x.shape[-1], what=name)
+        n += 1
+    assert n > 45
+
+
+# ---- seeded inputs against the oracle ------------------------------------------
+
+SHAPES = [(1, 1, 1), (5, 7, 3), (37, 29, 53), (64, 64, 16), (63, 65, 17), (127, 129, 31), (128, 128, 64),
+          (130, 70, 33), (200, 24, 100), (256, 384, 128), (300, 260, 101), (1, 300, 40), (300, 1, 40), (96, 96, 1)]
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_fp32_against_oracle(gpu, oracle, ta, tb):
+    torch = torch_()
+    for cfg in ("0", "1"):
+        os.environ["NTSAMD_TILE_CFG"] = cfg
+        for i, (M, N, K) in enumerate(SHAPES):
+            a = oracle.uniform(stored((M, K), ta), 1000 + i)
+            b = oracle.uniform(stored((K, N), tb), 2000 + i)
+            c0 = oracle.uniform((M, N), 3000 + i)
+            for alpha, beta in ((1.0, 0.0), (0.5, 1.0), (-1.25, 0.5)):
+                ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                c = dev_tensor(c0, gpu) if beta != 0 else torch.full((M, N), float("nan"), device=gpu)
+                nt.matrix_mul(dev_tensor(a, gpu), ta, dev_tensor(b, gpu), tb, c, alpha, beta)
+                assert_fp32(c.cpu().numpy(), ref, K, magnitude(oracle, a, ta, b, tb, alpha, beta, c0),
+                            what="cfg%s %dx%dx%d alpha=%g beta=%g" % (cfg, M, N, K, alpha, beta))
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_fp16_against_oracle(gpu, oracle, ta, tb):
+    torch = torch_()
+    for cfg in ("0", "1"):
+        os.environ["NTSAMD_TILE_CFG"] = cfg
+        for i, (M, N, K) in enumerate(SHAPES):
+            # round the inputs to half first; the oracle then runs in fp32 on those values
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 4000 + i, 0, 0.5)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 5000 + i, 0, 0.5)))
+            c0 = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((M, N), 6000 + i)))
+            for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+                ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                c = dev_tensor(c0, gpu, True) if beta != 0 else torch.full((M, N), float("nan"), device=gpu).half()
+                nt.matrix_mul(dev_tensor(a, gpu, True), ta, dev_tensor(b, gpu, True), tb, c, alpha, beta)
+                assert_fp16(c.float().cpu().numpy(), ref, what="cfg%s %dx%dx%d alpha=%g beta=%g" % (cfg, M, N, K, alpha, beta))
+
+
+def test_fp16_bits_match_the_oracle_conversion(gpu, oracle):
+    """Small integers: every product and sum is exact in fp32 and representable in half,
+    so the half result must equal the oracle's result bit for bit (RNE store)."""
+    rng = np.random.default_rng(3)
+    a = rng.integers(-4, 5, (70, 40)).astype(np.float32)
+    b = rng.integers(-4, 5, (40, 50)).astype(np.float32)
+    ref = oracle.matmul2d(a, X_NOTRANS, b, X_NOTRANS)
+    torch = torch_()
+    c = torch.empty((70, 50), device=gpu, dtype=torch.float16)
+    nt.matrix_mul(dev_tensor(a, gpu, True), X_NOTRANS, dev_tensor(b, gpu, True), X_NOTRANS, c)
+    assert np.array_equal(c.cpu().numpy().view(np.uint16), oracle.to_f16_bits(ref))
+    # rounding of a half result: alpha makes values that need RNE
+    c2 = torch.empty((70, 50), device=gpu, dtype=torch.float16)
+    nt.matrix_mul(dev_tensor(a, gpu, True), X_NOTRANS, dev_tensor(b, gpu, True), X_NOTRANS, c2, 1.0 / 3.0)
+    want = oracle.to_f16_bits((ref * np.float32(1.0 / 3.0)).astype(np.float32))
+    assert np.array_equal(c2.cpu().numpy().view(np.uint16), want)
+
+
+def test_half_in_float_out(gpu, oracle):
+    torch = torch_()
+    a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((45, 77), 1)))
+    b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((31, 77), 2)))
+    ref = oracle.matmul2d(a, X_NOTRANS, b, X_TRANS)
+    c = torch.empty((45, 31), device=gpu)
+    nt.matrix_mul(dev_tensor(a, gpu, True), X_NOTRANS, dev_tensor(b, gpu, True), X_TRANS, c)
+    assert_fp32(c.cpu().numpy(), ref, 77)
+
+
+def test_unaligned_operands_take_the_generic_path(gpu, oracle):
+    """Base pointers and leading dimensions that rule out 16-byte loads."""
+    torch = torch_()
+    M, N, K = 70, 52, 36
+    for ta, tb in TRANS:
+        a = oracle.uniform(stored((M, K), ta), 7)
+        b = oracle.uniform(stored((K, N), tb), 8)
+        ref = oracle.matmul2d(a, ta, b, tb)
+        for half in (False, True):
+            # shift both operands by one element inside a larger buffer
+            abuf = torch.zeros(a.size + 1, device=gpu, dtype=torch.float16 if half else torch.float32)
+            bbuf = torch.zeros(b.size + 1, device=gpu, dtype=abuf.dtype)
+            abuf[1:] = dev_tensor(a.ravel(), gpu, half)
+            bbuf[1:] = dev_tensor(b.ravel(), gpu, half)
+            av = abuf[1:].view(a.shape)
+            bv = bbuf[1:].view(b.shape)
+            c = torch.empty((M, N), device=gpu, dtype=abuf.dtype)
+            nt.matrix_mul(av, ta, bv, tb, c)
+            if half:
+                ah = oracle.from_f16_bits(oracle.to_f16_bits(a))
+                bh = oracle.from_f16_bits(oracle.to_f16_bits(b))
+                assert_fp16(c.float().cpu().numpy(), oracle.matmul2d(ah, ta, bh, tb))
+            else:
+                assert_fp32(c.cpu().numpy(), ref, K)
+
+
+def test_beta_zero_ignores_old_contents_and_scaling_is_exact(gpu, oracle):
+    torch = torch_()
+    a = dev_tensor(oracle.uniform((200, 96), 11), gpu)
+    b = dev_tensor(oracle.uniform((96, 136), 12), gpu)
+    junk = torch.full((200, 136), float("nan"), device=gpu)
+    junk[::2] = float("inf")
+    c1 = torch.zeros((200, 136), device=gpu)
+    nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c1)
+    nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, junk)
+    assert torch.equal(c1, junk)
+    c2 = torch.empty_like(c1)
+    nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c2, 2.0, 0.0)
+    assert torch.equal(c2, 2 * c1)                       # alpha = 2 only shifts exponents
+    c3 = c1.clone()
+    nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c3, 1.0, 1.0)
+    assert torch.equal(c3, 2 * c1)                       # beta = 1 on top of the product doubles it
+    # (A B)^T = B^T A^T through the transposed kernels
+    ct = torch.empty((136, 200), device=gpu)
+    nt.matrix_mul(b, X_TRANS, a, X_TRANS, ct)
+    assert normwise(ct.t().cpu().numpy(), c1.cpu().numpy()) < 1e-6
+
+
+# ---- batches --------------------------------------------------------------------
+
+@pytest.mark.parametrize("half", (False, True))
+def test_strided_batches(gpu, oracle, half):
+    torch = torch_()
+    check = assert_fp16 if half else (lambda g, r, what="": assert_fp32(g, r, 24, what=what))
+
+    def prep(x):
+        return oracle.from_f16_bits(oracle.to_f16_bits(x)) if half else x
+
+    q = prep(oracle.normal((2, 5, 50, 24), 1))
+    k = prep(oracle.normal((2, 5, 40, 24), 2))
+    v = prep(oracle.normal((2, 5, 40, 24), 3))
+    s_ref = oracle.matmul_batched(q, X_NOTRANS, k, X_TRANS, None, 0.125)
+    dt = torch.float16 if half else torch.float32
+    s = torch.full((2, 5, 50, 40), float("nan"), device=gpu, dtype=dt)
+    nt.matrix_mul_batched_strided(dev_tensor(q, gpu, half), X_NOTRANS, dev_tensor(k, gpu, half), X_TRANS, s,
+                                  10, 50 * 24, 40 * 24, 50 * 40, 50, 24, 40, 24, 50, 40, 0.125, 0.0)
+    check(s.float().cpu().numpy(), s_ref, "QK^T")
+    s_in = prep(s_ref)
+    o_ref = oracle.matmul_batched(s_in, X_NOTRANS, v, X_NOTRANS)
+    o = torch.empty((2, 5, 50, 24), device=gpu, dtype=dt)
+    nt.matrix_mul_batched_strided(dev_tensor(s_in, gpu, half), X_NOTRANS, dev_tensor(v, gpu, half), X_NOTRANS, o,
+                                  10, 50 * 40, 40 * 24, 50 * 24, 50, 40, 40, 24, 50, 24)
+    check(o.float().cpu().numpy(), o_ref, "SV")
+    # stride 0: one b shared by the whole batch (a transposed N-D a against one matrix)
+    at = prep(oracle.uniform((7, 24, 33), 4))
+    w = prep(oracle.uniform((24, 18), 5))
+    ref = oracle.matmul(at, X_TRANS, w, X_NOTRANS)
+    c = torch.empty((7, 33, 18), device=gpu, dtype=dt)
+    nt.matrix_mul_batched_strided(dev_tensor(at, gpu, half), X_TRANS, dev_tensor(w, gpu, half), X_NOTRANS, c,
+                                  7, 24 * 33, 0, 33 * 18, 24, 33, 24, 18, 33, 18)
+    check(c.float().cpu().numpy(), ref, "shared b")
+    # stride 0 on a, accumulate
+    a1 = prep(oracle.uniform((20, 24), 6))
+    bb = prep(oracle.uniform((6, 24, 10), 7))
+    c0 = prep(oracle.uniform((6, 20, 10), 8))
+    ref = np.stack([oracle.matmul2d(a1, X_NOTRANS, bb[i].copy(), X_NOTRANS, c0[i].copy(), 1.0, 1.0) for i in range(6)])
+    c = dev_tensor(c0, gpu, half)
+    nt.matrix_mul_batched_strided(dev_tensor(a1, gpu, half), X_NOTRANS, dev_tensor(bb, gpu, half), X_NOTRANS, c,
+                                  6, 0, 240, 200, 20, 24, 24, 10, 20, 10, 1.0, 1.0)
+    check(c.float().cpu().numpy(), ref, "shared a")
+
+
+def test_pointer_lists(gpu, oracle):
+    torch = torch_()
+    # more items than one launch carries in its arguments (128), unequal spacing
+    a = oracle.uniform((20, 9, 14), 1)
+    b = oracle.uniform((15, 14, 6), 2)
+    ga, gb = dev_tensor(a, gpu), dev_tensor(b, gpu)
+    c = torch.full((20, 15, 9, 6), float("nan"), device=gpu)
+    al, bl, cl = [], [], []
+    for p in range(20):
+        for q in range(15):
+            al.append(ga[p]); bl.append(gb[q]); cl.append(c[p, q])
+    assert len(al) == 300
+    nt.matrix_mul_batched(al, X_NOTRANS, bl, X_NOTRANS, cl, 0.5, 0.0)
+    assert_fp32(c.cpu().numpy(), oracle.matmul(a, X_NOTRANS, b, X_NOTRANS, None, 0.5), 14)
+    # half, transposed items
+    ah = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((3, 16, 40), 3)))
+    bh = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((3, 24, 16), 4)))
+    gah, gbh = dev_tensor(ah, gpu, True), dev_tensor(bh, gpu, True)
+    ch = torch.empty((3, 40, 24), device=gpu, dtype=torch.float16)
+    nt.matrix_mul_batched([gah[i] for i in (2, 0, 1)], X_TRANS, [gbh[i] for i in (2, 0, 1)], X_TRANS,
+                          [ch[i] for i in (2, 0, 1)])
+    assert_fp16(ch.float().cpu().numpy(), oracle.matmul_batched(ah, X_TRANS, bh, X_TRANS))
+
+
+# ---- fused bias -------------------------------------------------------------------
+
+@pytest.mark.parametrize("half", (False, True))
+def test_fused_bias(gpu, oracle, half):
+    torch = torch_()
+
+    def prep(x):
+        return oracle.from_f16_bits(oracle.to_f16_bits(x)) if half else x
+
+    x = prep(oracle.uniform((6, 20, 48), 1))
+    w = prep(oracle.normal((48, 72), 2, 0, 0.05))
+    dt = torch.float16 if half else torch.float32
+    for bshape in ((72,), (20,), (6, 1, 1)):
+        bias = prep(oracle.normal(bshape, 3, 0, 0.05))
+        ref, n = oracle.mulandshift(x, w, bias, 0.5)
+        c = torch.full((120, 72), float("nan"), device=gpu, dtype=dt)
+        if n == 2:
+            mode, div = BIAS_COL, 1
+        else:
+            mode, div = BIAS_ROW, int(np.prod(ref.shape[n + 1:-1]))
+        nt.matrix_mul(dev_tensor(x.reshape(120, 48), gpu, half), X_NOTRANS, dev_tensor(w, gpu, half), X_NOTRANS, c, 0.5, 0.0,
+                      bias=dev_tensor(bias.ravel(), gpu, half), bias_mode=mode, bias_row_div=div)
+        got = c.float().cpu().numpy().reshape(ref.shape)
+        if half:
+            assert_fp16(got, ref, what=str(bshape))
+        else:
+            mag = 0.5 * oracle.matmul(np.abs(x), X_NOTRANS, np.abs(w), X_NOTRANS) + np.abs(ref - oracle.matmul(x, X_NOTRANS, w, X_NOTRANS, None, 0.5))
+            assert_fp32(got, ref, 48, mag, what=str(bshape))
+
+
+def test_runs_on_the_callers_stream(gpu, oracle):
+    torch = torch_()
+    a = dev_tensor(oracle.uniform((256, 128), 1), gpu)
+    b = dev_tensor(oracle.uniform((128, 192), 2), gpu)
+    c = torch.zeros((256, 192), device=gpu)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c)
+    side.synchronize()
+    assert_fp32(c.cpu().numpy(), oracle.matmul2d(a.cpu().numpy(), X_NOTRANS, b.cpu().numpy(), X_NOTRANS), 128)
+    assert torch.cuda.current_device() == 0
+
+
+# ---- the benchmark configurations at full size ---------------------------------------
+
+def sampled_f64(a, ta, b, tb, rows, alpha=1.0):
+    A = (a.T if ta == X_TRANS else a)[rows].astype(np.float64)
+    B = (b.T if tb == X_TRANS else b).astype(np.float64)
+    return alpha * (A @ B)
+
+
+def test_config1_and_2_linear_layer(gpu, oracle):
+    """fp32 [4096x512] x [512x2048], plain and with the bias of MulAndShift."""
+    torch = torch_()
+    x = oracle.uniform((4096, 512), 1)
+    w = oracle.normal((512, 2048), 2, 0, 0.02)
+    bias = oracle.normal((2048,), 3, 0, 0.02)
+    gx, gw, gb = dev_tensor(x, gpu), dev_tensor(w, gpu), dev_tensor(bias, gpu)
+    c = torch.full((4096, 2048), float("nan"), device=gpu)
+    nt.matrix_mul(gx, X_NOTRANS, gw, X_NOTRANS, c)
+    rows = np.random.default_rng(0).choice(4096, 96, replace=False)
+    got = c.cpu().numpy()
+    assert_fp32(got[rows], sampled_f64(x, X_NOTRANS, w, X_NOTRANS, rows), 512)
+    # the oracle itself on a slab of rows (it needs ~1 s per 400 rows here)
+    ref = oracle.matmul2d(x[:256].copy(), X_NOTRANS, w, X_NOTRANS)
+    assert_fp32(got[:256], ref, 512, magnitude(oracle, x[:256].copy(), X_NOTRANS, w, X_NOTRANS, 1.0))
+    cb = torch.full((4096, 2048), float("nan"), device=gpu)
+    nt.matrix_mul(gx, X_NOTRANS, gw, X_NOTRANS, cb, bias=gb)
+    # the epilogue adds bias[column] to the same accumulators
+    assert normwise((cb - c).cpu().numpy(), np.broadcast_to(bias, (4096, 2048))) < 1e-5
+    ref_b, n = oracle.mulandshift(x[:64].copy().reshape(1, 64, 512), w, bias)
+    assert n == 2
+    assert_fp32(cb.cpu().numpy()[:64], ref_b[0], 512)
+
+
+def test_config3_attention_batches(gpu, oracle):
+    torch = torch_()
+    q = oracle.normal((256, 128, 64), 1)
+    k = oracle.normal((256, 128, 64), 2)
+    v = oracle.normal((256, 128, 64), 3)
+    gq, gk, gv = dev_tensor(q, gpu), dev_tensor(k, gpu), dev_tensor(v, gpu)
+    s = torch.full((256, 128, 128), float("nan"), device=gpu)
+    nt.matrix_mul_batched_strided(gq, X_NOTRANS, gk, X_TRANS, s, 256, 8192, 8192, 16384, 128, 64, 128, 64, 128, 128, 0.125)
+    s_ref = oracle.matmul_batched(q, X_NOTRANS, k, X_TRANS, None, 0.125)
+    assert_fp32(s.cpu().numpy(), s_ref, 64)
+    o = torch.full((256, 128, 64), float("nan"), device=gpu)
+    nt.matrix_mul_batched_strided(s, X_NOTRANS, gv, X_NOTRANS, o, 256, 16384, 8192, 8192, 128, 128, 128, 64, 128, 64)
+    o_ref = oracle.matmul_batched(s.cpu().numpy(), X_NOTRANS, v, X_NOTRANS)
+    assert_fp32(o.cpu().numpy(), o_ref, 128)
+
+
+def test_config4_half_tn(gpu, oracle):
+    """fp16, a stored [1024x8192] with X_TRANS, b [1024x4096]: fp32 accumulation, half result."""
+    torch = torch_()
+    a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((1024, 8192), 1, 0, 0.02)))
+    b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((1024, 4096), 2, 0, 0.02)))
+    ga, gb = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True)
+    c = torch.full((8192, 4096), float("nan"), device=gpu, dtype=torch.float16)
+    nt.matrix_mul(ga, X_TRANS, gb, X_NOTRANS, c)
+    got = c.float().cpu().numpy()
+    rows = np.random.default_rng(1).choice(8192, 64, replace=False)
+    assert_fp16(got[rows], sampled_f64(a, X_TRANS, b, X_NOTRANS, rows))
+    # the fp32 oracle on a block of result rows (columns of the stored a)
+    sub = np.ascontiguousarray(a[:, :96])
+    assert_fp16(got[:96], oracle.matmul2d(sub, X_TRANS, b, X_NOTRANS))
+    # scaling by 2 is exact in half as well, for results that are normal halves
+    c2 = torch.empty_like(c)
+    nt.matrix_mul(ga, X_TRANS, gb, X_NOTRANS, c2, 2.0)
+    normal = c.abs() > 2.0 ** -13      # above the first binade, where a value just below 2^-14 may round up into it
+    assert normal.float().mean() > 0.9
+    assert int((c2[normal] != (2 * c)[normal]).sum()) == 0
+    assert torch.equal(c2[normal], (2 * c)[normal])
+
+
+def test_config5_ragged_vocab_projection(gpu, oracle):
+    """fp32 H[4096x512] x W[30011x512]^T accumulated into C[4096x30011] with beta = 1."""
+    torch = torch_()
+    h = oracle.uniform((4096, 512), 1)
+    w = oracle.normal((30011, 512), 2, 0, 0.02)
+    c0 = oracle.uniform((4096, 30011), 3)
+    gh, gw = dev_tensor(h, gpu), dev_tensor(w, gpu)
+    c = dev_tensor(c0, gpu)
+    nt.matrix_mul(gh, X_NOTRANS, gw, X_TRANS, c, 1.0, 1.0)
+    got = c.cpu().numpy()
+    rows = np.random.default_rng(2).choice(4096, 48, replace=False)
+    want = sampled_f64(h, X_NOTRANS, w, X_TRANS, rows) + c0[rows]
+    assert_fp32(got[rows], want, 512)
+    # the oracle on the last rows (the ragged right edge is in every row)
+    ref = oracle.matmul2d(h[-24:].copy(), X_NOTRANS, w, X_TRANS, c0[-24:].copy(), 1.0, 1.0)
+    assert_fp32(got[-24:], ref, 512)
+    # accumulate once more: c + h w^T again = c0 + 2 h w^T
+    nt.matrix_mul(gh, X_NOTRANS, gw, X_TRANS, c, 1.0, 1.0)
+    want2 = 2 * sampled_f64(h, X_NOTRANS, w, X_TRANS, rows) + c0[rows]
+    assert_fp32(c.cpu().numpy()[rows], want2, 512)
