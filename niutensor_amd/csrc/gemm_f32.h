@@ -5,79 +5,79 @@
  *
  * One workgroup computes a BM x BN tile of c; its WGM x WGN waves each own a
  * (BM/WGM) x (BN/WGN) sub-tile held as 32x32 accumulator blocks of
- * v_mfma_f32_32x32x2_f32. Both operands are staged through LDS in k-major
- * rows (S[k][mn]), so a wave's operand fetch is 32 consecutive floats per
- * half-wave whatever the transpose flags are; K-contiguous sources are
- * transposed on the way into LDS. Two LDS stages: global loads for slab t+1
- * are issued before the MFMA work on slab t and parked in registers.
+ * v_mfma_f32_32x32x2_f32 (lane l feeds row/column l%32 at k slot l/32).
+ *
+ * Operand staging in LDS, chosen per operand by how it lies in memory:
+ *   MN-contiguous (a with X_TRANS, b with X_NOTRANS): rows of k, S[k][mn].
+ *       16-byte global loads and 16-byte LDS writes along mn; a fragment is
+ *       32 consecutive floats per half-wave: no bank conflicts, no padding.
+ *   K-contiguous (a with X_NOTRANS, b with X_TRANS): rows of mn, S[mn][k], row
+ *       pitch BKT+4 floats. 16-byte global loads and 16-byte LDS writes along
+ *       k; a lane fetches FOUR k values of its row with one 16-byte read, and
+ *       the pitch of 80 bytes puts the eight lanes of a 128-byte LDS phase in
+ *       eight different 16-byte bank groups.
+ * The order in which k values meet inside a slab is free as long as both
+ * operands agree, so MFMA step t of a slab takes k = 8*(t/4) + 4*(l/32) + t%4:
+ * that is what makes the four-at-once fetch of the K-contiguous layout line up
+ * with single-row fetches of the other layout.
+ *
+ * Pipeline, per slab of BKT values of k: the wave holds all its fragments of
+ * the current slab in registers and issues MFMAs only from them; the next
+ * slab travels global -> registers (one slab ahead) -> the other LDS stage
+ * (first half of the MFMAs) -> one barrier -> the second register set (second
+ * half of the MFMAs). The 16-byte global loads are buffer loads: the slab's
+ * base address lives in scalar registers and advances by a scalar add, the
+ * per-lane offset never changes, and reads past the end of the matrix return
+ * zero in hardware, so the steady-state loop has no address arithmetic and no
+ * predication on the vector side.
  */
 #pragma once
 #include "gemm_common.h"
 
 namespace ntsamd {
 
-/* four elements (row, k..k+3) of a K-contiguous operand; zero beyond K */
-template <bool VEC>
-__device__ __forceinline__ f32x4 ld4_kcontig(const float * __restrict__ rowPtr, int k, int K)
+template <int N>
+struct IntC {
+    static constexpr int value = N;
+};
+
+/* a raw buffer descriptor over [base, base + bytes): dword 3 selects 32-bit data, no swizzle */
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void * base, long long bytes)
 {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (VEC) {
-        /* K % 4 == 0 here: the group is entirely inside or entirely outside */
-        if (k < K)
-            v = *reinterpret_cast<const f32x4 *>(rowPtr + k);
-    }
-    else {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-            if (k + e < K)
-                v[e] = rowPtr[k + e];
-    }
-    return v;
+    /* bytes > 0 always: the base is inside the matrix */
+    int n = (unsigned long long)bytes >> 31 ? 0x7fffffff : (int)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, n, 0x00020000);
 }
 
-/* four elements (k, m..m+3) of an MN-contiguous operand; zero beyond K,
-   indices beyond the matrix edge are clamped (those outputs are never stored) */
-template <bool VEC>
-__device__ __forceinline__ f32x4 ld4_mncontig(const float * __restrict__ base, int ld, int k, int K, int m, int M)
+/* a byte offset no descriptor made by make_rsrc covers: the load returns zero */
+#define NTSAMD_OOB_OFFSET 0x7fffffff
+
+__device__ __forceinline__ f32x4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t rsrc, int byteOffset)
 {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (k < K) {
-        const float * r = base + (size_t)k * ld;
-        if (VEC) {
-            /* M % 4 == 0 here */
-            int mm = m < M - 4 ? m : M - 4;
-            v = *reinterpret_cast<const f32x4 *>(r + mm);
-        }
-        else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                int mm = m + e < M - 1 ? m + e : M - 1;
-                v[e] = r[mm];
-            }
-        }
-    }
-    return v;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byteOffset, 0, 0);
+    return __builtin_bit_cast(f32x4, v);
 }
 
 template <int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, typename PT>
-__global__ void __launch_bounds__(WGM * WGN * 64)
+__global__ void __launch_bounds__(WGM * WGN * 64, 2)
 gemm_f32_kernel(const GemmParams p, const PT tab)
 {
     constexpr int NT = WGM * WGN * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TI = WM / 32, TJ = WN / 32;
-    /* K-contiguous sources are written to LDS one float at a time, four k-rows
-       per lane; a row pitch of 2 mod 8 spreads those writes over all banks */
-    constexpr int LDA = AKC ? BM + 2 : BM;
-    constexpr int LDB = BKC ? BN + 2 : BN;
+    constexpr int KK = BKT / 2;           /* MFMA steps per slab */
+    constexpr int LDK = BKT + 4;          /* row pitch of a K-contiguous operand in LDS */
     constexpr int NA = BM * BKT / 4 / NT;
     constexpr int NB = BN * BKT / 4 / NT;
+    constexpr int ASIZE = AKC ? BM * LDK : BKT * BM;
+    constexpr int BSIZE = BKC ? BN * LDK : BKT * BN;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 blocks");
     static_assert((BM * BKT / 4) % NT == 0 && (BN * BKT / 4) % NT == 0, "loads must divide evenly");
-    static_assert(BKT % 4 == 0, "slab depth");
+    static_assert(BKT % 8 == 0, "slab depth");
 
-    __shared__ __attribute__((aligned(16))) float As[2][BKT * LDA];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BKT * LDB];
+    __shared__ __attribute__((aligned(16))) float As[2][ASIZE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BSIZE];
 
     const TileCoord tc = tile_of_workgroup(p);
     const float * __restrict__ A;
@@ -101,82 +101,182 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    /* per-thread staging slots */
-    const float * aRow[NA];
-    const float * bRow[NB];
-    int aK[NA], aMN[NA], bK[NB], bMN[NB];
+    /* ---- staging slots: which 4 elements of the slab each thread moves ------ */
+    int aOff[NA], bOff[NB];        /* 16-byte path: byte offset from the slab base */
+    int aLds[NA], bLds[NB];        /* float index in the LDS stage */
+    int aK[NA], bK[NB];            /* k of the slot's first element inside the slab */
+    int aMN[NA], bMN[NB];          /* row (K-contiguous) or first column (MN-contiguous) inside the tile */
 #pragma unroll
     for (int s = 0; s < NA; s++) {
         int g = tid + s * NT;
         if (AKC) {
-            aMN[s] = g / (BKT / 4);
+            int row = g / (BKT / 4);
             aK[s] = (g % (BKT / 4)) * 4;
-            int row = m0 + aMN[s];
-            row = row < M - 1 ? row : M - 1;
-            aRow[s] = A + (size_t)row * p.lda;
+            aMN[s] = row;
+            aLds[s] = row * LDK + aK[s];
+            int r = m0 + row < M - 1 ? row : M - 1 - m0;        /* rows past the edge repeat the last one */
+            aOff[s] = (r * p.lda + aK[s]) * 4;
         }
         else {
             aK[s] = g / (BM / 4);
             aMN[s] = (g % (BM / 4)) * 4;
-            aRow[s] = A;
+            aLds[s] = aK[s] * BM + aMN[s];
+            int c = m0 + aMN[s] < M - 4 ? aMN[s] : M - 4 - m0;  /* 16-byte path: M % 4 == 0 */
+            aOff[s] = (aK[s] * p.lda + c) * 4;
         }
     }
 #pragma unroll
     for (int s = 0; s < NB; s++) {
         int g = tid + s * NT;
         if (BKC) {
-            bMN[s] = g / (BKT / 4);
+            int row = g / (BKT / 4);
             bK[s] = (g % (BKT / 4)) * 4;
-            int row = n0 + bMN[s];
-            row = row < N - 1 ? row : N - 1;
-            bRow[s] = B + (size_t)row * p.ldb;
+            bMN[s] = row;
+            bLds[s] = row * LDK + bK[s];
+            int r = n0 + row < N - 1 ? row : N - 1 - n0;
+            bOff[s] = (r * p.ldb + bK[s]) * 4;
         }
         else {
             bK[s] = g / (BN / 4);
             bMN[s] = (g % (BN / 4)) * 4;
-            bRow[s] = B;
+            bLds[s] = bK[s] * BN + bMN[s];
+            int c = n0 + bMN[s] < N - 4 ? bMN[s] : N - 4 - n0;
+            bOff[s] = (bK[s] * p.ldb + c) * 4;
         }
     }
 
+    /* first element of the tile's operand panels, and one past the end of each matrix */
+    const float * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
+    const float * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
+    const float * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
+    const float * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+
     f32x4 ra[NA], rb[NB];
 
-    auto load_global = [&](int k0) {
+    auto load_global = [&](auto TAIL, int k0) {
+        constexpr bool mayHangOver = decltype(TAIL)::value != 0;
+        if constexpr (VEC) {
+            const float * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
+            const float * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
+            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, (long long)(aEnd - ab) * 4);
+            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, (long long)(bEnd - bb) * 4);
+            /* only the last slab can hang over K. Rows of k past the end of an MN-contiguous
+               matrix are past the end of the buffer and read as zero by themselves; a
+               K-contiguous row would run on into the next row instead, so those lanes are
+               sent out of range explicitly */
+            const bool tail = mayHangOver && k0 + BKT > K;
 #pragma unroll
-        for (int s = 0; s < NA; s++) {
-            if (AKC)
-                ra[s] = ld4_kcontig<VEC>(aRow[s], k0 + aK[s], K);
-            else
-                ra[s] = ld4_mncontig<VEC>(aRow[s], p.lda, k0 + aK[s], K, m0 + aMN[s], M);
+            for (int s = 0; s < NA; s++) {
+                int off = aOff[s];
+                if (AKC && tail && k0 + aK[s] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                ra[s] = buffer_load_f32x4(ar, off);
+            }
+#pragma unroll
+            for (int s = 0; s < NB; s++) {
+                int off = bOff[s];
+                if (BKC && tail && k0 + bK[s] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                rb[s] = buffer_load_f32x4(br, off);
+            }
         }
+        else {
+            /* generic path: any alignment, element by element, predicated */
 #pragma unroll
-        for (int s = 0; s < NB; s++) {
-            if (BKC)
-                rb[s] = ld4_kcontig<VEC>(bRow[s], k0 + bK[s], K);
-            else
-                rb[s] = ld4_mncontig<VEC>(bRow[s], p.ldb, k0 + bK[s], K, n0 + bMN[s], N);
+            for (int s = 0; s < NA; s++) {
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (AKC) {
+                    int r = m0 + aMN[s] < M - 1 ? m0 + aMN[s] : M - 1;
+                    const float * rp = A + (size_t)r * p.lda;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k0 + aK[s] + e < K)
+                            v[e] = rp[k0 + aK[s] + e];
+                }
+                else if (k0 + aK[s] < K) {
+                    const float * rp = A + (size_t)(k0 + aK[s]) * p.lda;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int c = m0 + aMN[s] + e < M - 1 ? m0 + aMN[s] + e : M - 1;
+                        v[e] = rp[c];
+                    }
+                }
+                ra[s] = v;
+            }
+#pragma unroll
+            for (int s = 0; s < NB; s++) {
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (BKC) {
+                    int r = n0 + bMN[s] < N - 1 ? n0 + bMN[s] : N - 1;
+                    const float * rp = B + (size_t)r * p.ldb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k0 + bK[s] + e < K)
+                            v[e] = rp[k0 + bK[s] + e];
+                }
+                else if (k0 + bK[s] < K) {
+                    const float * rp = B + (size_t)(k0 + bK[s]) * p.ldb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int c = n0 + bMN[s] + e < N - 1 ? n0 + bMN[s] + e : N - 1;
+                        v[e] = rp[c];
+                    }
+                }
+                rb[s] = v;
+            }
         }
     };
 
     auto store_lds = [&](int buf) {
 #pragma unroll
-        for (int s = 0; s < NA; s++) {
-            if (AKC) {
+        for (int s = 0; s < NA; s++)
+            *reinterpret_cast<f32x4 *>(&As[buf][aLds[s]]) = ra[s];
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    As[buf][(aK[s] + e) * LDA + aMN[s]] = ra[s][e];
-            }
-            else
-                *reinterpret_cast<f32x4 *>(&As[buf][aK[s] * LDA + aMN[s]]) = ra[s];
+        for (int s = 0; s < NB; s++)
+            *reinterpret_cast<f32x4 *>(&Bs[buf][bLds[s]]) = rb[s];
+    };
+
+    /* ---- fragments: two register sets, [set][...] ----------------------------
+       K-contiguous operand: one f32x4 per block and per group of four steps;
+       MN-contiguous operand: one float per block and per step */
+    f32x4 fa4[2][AKC ? KK / 4 : 1][TI];
+    float fa1[2][AKC ? 1 : KK][TI];
+    f32x4 fb4[2][BKC ? KK / 4 : 1][TJ];
+    float fb1[2][BKC ? 1 : KK][TJ];
+
+    auto read_frags = [&](auto SET, int buf) {
+        constexpr int set = decltype(SET)::value;
+        if constexpr (AKC) {
+            const float * as = &As[buf][(wm0 + l32) * LDK + 4 * lh];
+#pragma unroll
+            for (int q = 0; q < KK / 4; q++)
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+                    fa4[set][q][i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * LDK + 8 * q);
         }
+        else {
+            const float * as = &As[buf][4 * lh * BM + wm0 + l32];
 #pragma unroll
-        for (int s = 0; s < NB; s++) {
-            if (BKC) {
+            for (int t = 0; t < KK; t++)
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    Bs[buf][(bK[s] + e) * LDB + bMN[s]] = rb[s][e];
-            }
-            else
-                *reinterpret_cast<f32x4 *>(&Bs[buf][bK[s] * LDB + bMN[s]]) = rb[s];
+                for (int i = 0; i < TI; i++)
+                    fa1[set][t][i] = as[(8 * (t / 4) + (t % 4)) * BM + i * 32];
+        }
+        if constexpr (BKC) {
+            const float * bs = &Bs[buf][(wn0 + l32) * LDK + 4 * lh];
+#pragma unroll
+            for (int q = 0; q < KK / 4; q++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    fb4[set][q][j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * LDK + 8 * q);
+        }
+        else {
+            const float * bs = &Bs[buf][4 * lh * BN + wn0 + l32];
+#pragma unroll
+            for (int t = 0; t < KK; t++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    fb1[set][t][j] = bs[(8 * (t / 4) + (t % 4)) * BN + j * 32];
         }
     };
 
@@ -189,69 +289,152 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.f;
 
+    auto mfma_steps = [&](auto SET, int first, int last) {
+        constexpr int set = decltype(SET)::value;
+#pragma unroll
+        for (int t = first; t < last; t++)
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    float av = AKC ? fa4[set][t / 4][i][t % 4] : fa1[set][t][i];
+                    float bv = BKC ? fb4[set][t / 4][j][t % 4] : fb1[set][t][j];
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                }
+    };
+
     const int nk = (K + BKT - 1) / BKT;
-    if (nk > 0) {
-        load_global(0);
-        store_lds(0);
-    }
-    __syncthreads();
 
-    for (int kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk)
-            load_global((kt + 1) * BKT);
-
-        const float * as = &As[buf][lh * LDA + wm0 + l32];
-        const float * bs = &Bs[buf][lh * LDB + wn0 + l32];
+    /* One slab: fragments of slab kt are in register set SET and came from LDS stage SET.
+       FULL: slabs kt+1 and kt+2 exist and are complete, so nothing is conditional and the
+       slab is one straight run of instructions that the scheduler can interleave. */
+    auto slab = [&](auto SET, auto FULL, int kt) {
+        constexpr int set = decltype(SET)::value;
+        constexpr bool full = decltype(FULL)::value != 0;
+        if (full || kt + 1 < nk)
+            store_lds(set ^ 1);                  /* slab kt+1, fetched during slab kt-1 */
+        if (full)
+            load_global(IntC<0>(), (kt + 2) * BKT);
+        else if (kt + 2 < nk)
+            load_global(IntC<1>(), (kt + 2) * BKT);
+        mfma_steps(SET, 0, KK / 2);
+        if constexpr (full) {
+            /* An MFMA keeps the matrix pipe busy for 64 cycles but takes one issue slot:
+               spread the LDS writes, the buffer loads and their scalar bookkeeping
+               between the MFMAs instead of in front of them, so the pipe never waits
+               for this wave to get through a block of other work. */
 #pragma unroll
-        for (int kk = 0; kk < BKT / 2; kk++) {
-            float af[TI], bf[TJ];
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-                af[i] = as[kk * 2 * LDA + i * 32];
-#pragma unroll
-            for (int j = 0; j < TJ; j++)
-                bf[j] = bs[kk * 2 * LDB + j * 32];
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+            for (int g = 0; g < KK / 2 * TI * TJ; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* one MFMA */
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);     /* one LDS write */
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);     /* one global read */
+                __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);     /* some scalar / vector ALU */
+            }
         }
+        /* keep the compiler from sliding MFMAs across the barrier: the point of
+           the first half is to be in flight while the wave waits here */
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();                         /* stage set^1 complete; stage set no longer read by anyone */
+        __builtin_amdgcn_sched_barrier(0);
+        if (full || kt + 1 < nk)
+            read_frags(IntC<set ^ 1>(), set ^ 1);
+        mfma_steps(SET, KK / 2, KK);
+        if constexpr (full) {
+#pragma unroll
+            for (int g = 0; g < KK / 2 * TI * TJ; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* one MFMA */
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     /* one LDS read */
+                __builtin_amdgcn_sched_group_barrier(0x006, 2, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
 
-        if (kt + 1 < nk)
-            store_lds(buf ^ 1);
+    if (nk > 0) {
+        load_global(IntC<1>(), 0);
+        store_lds(0);
+        if (nk > 1)
+            load_global(IntC<1>(), BKT);
         __syncthreads();
+        read_frags(IntC<0>(), 0);
+        const int nkFull = K / BKT;              /* slabs that lie entirely inside K */
+        int kt = 0;
+        for (; kt + 3 < nkFull; kt += 2) {
+            slab(IntC<0>(), IntC<1>(), kt);
+            slab(IntC<1>(), IntC<1>(), kt + 1);
+        }
+        for (; kt < nk; kt += 2) {
+            slab(IntC<0>(), IntC<0>(), kt);
+            if (kt + 1 < nk)
+                slab(IntC<1>(), IntC<0>(), kt + 1);
+        }
     }
 
-    /* epilogue: accumulator register r of lane l is element
+    /* ---- epilogue: accumulator register r of lane l is element
        (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block, so a store covers
-       two rows of 32 consecutive floats and needs no alignment of ldc */
+       two rows of 32 consecutive floats and needs no alignment of ldc ---------- */
     const float alpha = p.alpha, beta = p.beta;
     const float * __restrict__ bias = static_cast<const float *>(p.bias);
+    const int biasMode = p.biasMode;
+
+    if constexpr (VEC) {
+        /* The wave's rows of c as one buffer that ends where c ends: rows past M drop
+           off its end and columns past N are sent out of range, so the stores (and the
+           loads for beta != 0) need no predicates. Row-indexed bias is not handled here. */
+        if (m0 + wm0 >= M)
+            return;
+        float * cw = C + (size_t)(m0 + wm0) * p.ldc;
+        __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 4);
+        const unsigned rowPitch = (unsigned)p.ldc * 4u;
 #pragma unroll
-    for (int j = 0; j < TJ; j++) {
-        const int col = n0 + wn0 + j * 32 + l32;
-        if (col >= N)
-            continue;
-        float bcol = 0.f;
-        if (p.biasMode == BIAS_COL)
-            bcol = bias[col];
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + (n0 + wn0 + j * 32 + l32)) * 4u
+                                          : (unsigned)NTSAMD_OOB_OFFSET;
+            float bcol = 0.f;
+            if (biasMode == BIAS_COL && col < N)
+                bcol = bias[col];
 #pragma unroll
-        for (int i = 0; i < TI; i++) {
+            for (int i = 0; i < TI; i++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (row < M) {
-                    float * cp = C + (size_t)row * p.ldc + col;
-                    float v = alpha * acc[i][j][r];
+                for (int r = 0; r < 16; r++) {
+                    const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    float v = alpha * acc[i][j][r] + bcol;
                     if (beta != 0.f)
-                        v += beta * (*cp);
-                    if (p.biasMode == BIAS_ROW)
-                        v += bias[(row / p.biasRowDiv) % p.biasLen];
-                    else
-                        v += bcol;
-                    *cp = v;
+                        v += beta * __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
+                }
+            }
+        }
+    }
+    else {
+        /* generic path: plain pointers, per-element bounds, every bias mode */
+#pragma unroll
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col >= N)
+                continue;
+            float bcol = 0.f;
+            if (biasMode == BIAS_COL)
+                bcol = bias[col];
+#pragma unroll
+            for (int i = 0; i < TI; i++) {
+                const int rowBase = m0 + wm0 + i * 32 + 4 * lh;
+                float * cb = C + (size_t)rowBase * p.ldc + col;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int dr = 8 * (r / 4) + (r % 4);
+                    if (rowBase + dr < M) {
+                        float * cp = cb + (size_t)dr * p.ldc;
+                        float v = alpha * acc[i][j][r];
+                        if (beta != 0.f)
+                            v += beta * (*cp);
+                        if (biasMode == BIAS_ROW)
+                            v += bias[((rowBase + dr) / p.biasRowDiv) % p.biasLen];
+                        else
+                            v += bcol;
+                        *cp = v;
+                    }
                 }
             }
         }

@@ -190,9 +190,14 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.groupM = 8;
 
     const int vecElems = kind == KIND_F32 ? 4 : 8;
+    /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column
+       only. It keeps a tile's byte offsets in 31 bits, so rows longer than 2M elements
+       go through the generic path, like everything unaligned and row-indexed bias */
     bool vec = !ptrs && kind != KIND_F16_F32OUT &&
                lda % vecElems == 0 && ldb % vecElems == 0 && aligned16(a) && aligned16(b) &&
-               strideA % vecElems == 0 && strideB % vecElems == 0;
+               strideA % vecElems == 0 && strideB % vecElems == 0 &&
+               lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) &&
+               biasMode != NTSAMD_BIAS_ROW;
     int cfg = choose_cfg(s.M, s.N, count);
     hipStream_t hs = static_cast<hipStream_t>(stream);
 
