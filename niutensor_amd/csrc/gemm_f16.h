@@ -6,74 +6,98 @@
  * half (:74-78); this kernel keeps alpha, beta and the accumulator in fp32 and
  * rounds once, to nearest even, when it stores a half result.
  *
- * v_mfma_f32_32x32x16_f16 wants eight consecutive k per lane, so both operands
- * sit in LDS as S[mn][k] rows (pitch BKT+8 halves: 16-byte fetches of 8
- * consecutive rows fall in distinct bank groups). MN-contiguous sources are
- * transposed on the way into LDS.
+ * v_mfma_f32_32x32x16_f16 takes, per lane, eight consecutive k of one row (A) or
+ * one column (B): lane l holds row/column l%32 and k = 8*(l/32) .. +7 of the step.
+ * Operand staging in LDS, chosen per operand by how it lies in memory:
+ *   K-contiguous (a with X_NOTRANS, b with X_TRANS): rows of mn, S[mn][k], pitch
+ *       BKT+8 halves. 16-byte global loads and LDS writes along k; a fragment is
+ *       one 16-byte LDS read, and the 80-byte pitch spreads the eight lanes of a
+ *       128-byte LDS phase over eight bank groups.
+ *   MN-contiguous (a with X_TRANS, b with X_NOTRANS): rows of k, S[k][mn], pitch
+ *       BMN+16 halves. 16-byte global loads and LDS writes along mn; a fragment is
+ *       two ds_read_b64_tr_b16: within 16 lanes the instruction hands lane c the
+ *       c-th half of each of the four rows that lanes 0-3, 4-7, 8-11, 12-15 point
+ *       at, which is exactly "four consecutive k of column c" when those lane
+ *       groups point at four consecutive k rows. The pitch of 32 bytes mod 128
+ *       keeps the four rows of one read in different bank groups.
+ *
+ * Pipeline per slab of BKT values of k, as in the fp32 kernel: all fragments of
+ * the current slab sit in registers; the next slab goes global -> registers (one
+ * slab ahead) -> the other LDS stage -> one barrier -> the second register set,
+ * and every one of those instructions is interleaved between MFMAs.
  */
 #pragma once
 #include "gemm_common.h"
+#include "gemm_f32.h"   /* make_rsrc, IntC, NTSAMD_OOB_OFFSET */
 
 namespace ntsamd {
 
 typedef _Float16 half_t;
 
-/* eight elements (row, k..k+7) of a K-contiguous operand; zero beyond K */
-template <bool VEC>
-__device__ __forceinline__ f16x8 ld8_kcontig(const half_t * __restrict__ rowPtr, int k, int K)
+__device__ __forceinline__ f16x8 buffer_load_f16x8(__amdgpu_buffer_rsrc_t rsrc, int byteOffset)
 {
-    f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (VEC) {
-        if (k < K)
-            v = *reinterpret_cast<const f16x8 *>(rowPtr + k);
-    }
-    else {
-#pragma unroll
-        for (int e = 0; e < 8; e++)
-            if (k + e < K)
-                v[e] = rowPtr[k + e];
-    }
-    return v;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byteOffset, 0, 0);
+    return __builtin_bit_cast(f16x8, v);
 }
 
-/* eight elements (k, m..m+7) of an MN-contiguous operand */
-template <bool VEC>
-__device__ __forceinline__ f16x8 ld8_mncontig(const half_t * __restrict__ base, int ld, int k, int K, int m, int M)
+/* transposing LDS read: see the header comment for what each lane receives */
+__device__ __forceinline__ f16x4 lds_read_tr16(const half_t * p)
 {
-    f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (k < K) {
-        const half_t * r = base + (size_t)k * ld;
-        if (VEC) {
-            int mm = m < M - 8 ? m : M - 8;
-            v = *reinterpret_cast<const f16x8 *>(r + mm);
-        }
-        else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                int mm = m + e < M - 1 ? m + e : M - 1;
-                v[e] = r[mm];
-            }
-        }
-    }
-    return v;
+    typedef __fp16 hv4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+    hv4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) hv4 *)(p));
+    return __builtin_bit_cast(f16x4, v);
 }
 
-template <typename OutT, int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, typename PT>
-__global__ void __launch_bounds__(WGM * WGN * 64)
+template <typename OutT>
+__device__ __forceinline__ void buffer_store_out(OutT v, __amdgpu_buffer_rsrc_t rsrc, int byteOffset);
+template <>
+__device__ __forceinline__ void buffer_store_out<float>(float v, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc, byteOffset, 0, 0);
+}
+template <>
+__device__ __forceinline__ void buffer_store_out<half_t>(half_t v, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rsrc, byteOffset, 0, 0);
+}
+template <typename OutT>
+__device__ __forceinline__ float buffer_load_out(__amdgpu_buffer_rsrc_t rsrc, int byteOffset);
+template <>
+__device__ __forceinline__ float buffer_load_out<float>(__amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byteOffset, 0, 0));
+}
+template <>
+__device__ __forceinline__ float buffer_load_out<half_t>(__amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    return (float)__builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rsrc, byteOffset, 0, 0));
+}
+
+template <typename OutT, int BM, int BN, int BKT, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool VEC, typename PT>
+__global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_kernel(const GemmParams p, const PT tab)
 {
     constexpr int NT = WGM * WGN * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TI = WM / 32, TJ = WN / 32;
-    constexpr int LDK = BKT + 8;
+    constexpr int KS = BKT / 16;          /* MFMA k steps per slab */
+    constexpr int LDK = BKT + 8;          /* pitch of a K-contiguous operand, halves */
+    constexpr int LDA = BM + 16;          /* pitch of an MN-contiguous a, halves */
+    constexpr int LDB = BN + 16;
     constexpr int NA = BM * BKT / 8 / NT;
     constexpr int NB = BN * BKT / 8 / NT;
+    constexpr int ASIZE = AKC ? BM * LDK : BKT * LDA;
+    constexpr int BSIZE = BKC ? BN * LDK : BKT * LDB;
+    constexpr int NMFMA = KS * TI * TJ;   /* MFMAs per slab */
+    constexpr int PRE = NMFMA / 4;        /* MFMAs issued before the slab's barrier */
+    constexpr int PREG = PRE > 0 ? PRE : 1;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 blocks");
     static_assert((BM * BKT / 8) % NT == 0 && (BN * BKT / 8) % NT == 0, "loads must divide evenly");
     static_assert(BKT % 16 == 0, "slab depth");
 
-    __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDK];
-    __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDK];
+    __shared__ __attribute__((aligned(16))) half_t As[2][ASIZE];
+    __shared__ __attribute__((aligned(16))) half_t Bs[2][BSIZE];
 
     const TileCoord tc = tile_of_workgroup(p);
     const half_t * __restrict__ A;
@@ -97,83 +121,185 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    const half_t * aRow[NA];
-    const half_t * bRow[NB];
-    int aK[NA], aMN[NA], bK[NB], bMN[NB];
+    /* ---- staging slots: which 8 halves of the slab each thread moves --------- */
+    int aOff[NA], bOff[NB];        /* 16-byte path: byte offset from the slab base */
+    int aLds[NA], bLds[NB];        /* half index in the LDS stage */
+    int aK[NA], bK[NB];            /* k of the slot's first element inside the slab */
+    int aMN[NA], bMN[NB];          /* row (K-contiguous) or first column (MN-contiguous) inside the tile */
 #pragma unroll
     for (int s = 0; s < NA; s++) {
         int g = tid + s * NT;
         if (AKC) {
-            aMN[s] = g / (BKT / 8);
+            int row = g / (BKT / 8);
             aK[s] = (g % (BKT / 8)) * 8;
-            int row = m0 + aMN[s];
-            row = row < M - 1 ? row : M - 1;
-            aRow[s] = A + (size_t)row * p.lda;
+            aMN[s] = row;
+            aLds[s] = row * LDK + aK[s];
+            int r = m0 + row < M - 1 ? row : M - 1 - m0;
+            aOff[s] = (r * p.lda + aK[s]) * 2;
         }
         else {
-            /* k fastest across lanes: the transposing LDS writes of one
-               instruction then land in one S row instead of one bank */
-            aK[s] = g % BKT;
-            aMN[s] = (g / BKT) * 8;
-            aRow[s] = A;
+            aK[s] = g / (BM / 8);
+            aMN[s] = (g % (BM / 8)) * 8;
+            aLds[s] = aK[s] * LDA + aMN[s];
+            int c = m0 + aMN[s] < M - 8 ? aMN[s] : M - 8 - m0;  /* 16-byte path: M % 8 == 0 */
+            aOff[s] = (aK[s] * p.lda + c) * 2;
         }
     }
 #pragma unroll
     for (int s = 0; s < NB; s++) {
         int g = tid + s * NT;
         if (BKC) {
-            bMN[s] = g / (BKT / 8);
+            int row = g / (BKT / 8);
             bK[s] = (g % (BKT / 8)) * 8;
-            int row = n0 + bMN[s];
-            row = row < N - 1 ? row : N - 1;
-            bRow[s] = B + (size_t)row * p.ldb;
+            bMN[s] = row;
+            bLds[s] = row * LDK + bK[s];
+            int r = n0 + row < N - 1 ? row : N - 1 - n0;
+            bOff[s] = (r * p.ldb + bK[s]) * 2;
         }
         else {
-            bK[s] = g % BKT;
-            bMN[s] = (g / BKT) * 8;
-            bRow[s] = B;
+            bK[s] = g / (BN / 8);
+            bMN[s] = (g % (BN / 8)) * 8;
+            bLds[s] = bK[s] * LDB + bMN[s];
+            int c = n0 + bMN[s] < N - 8 ? bMN[s] : N - 8 - n0;
+            bOff[s] = (bK[s] * p.ldb + c) * 2;
         }
     }
 
+    const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
+    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
+    const half_t * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
+    const half_t * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+
     f16x8 ra[NA], rb[NB];
 
-    auto load_global = [&](int k0) {
+    auto load_global = [&](auto TAIL, int k0) {
+        constexpr bool mayHangOver = decltype(TAIL)::value != 0;
+        if constexpr (VEC) {
+            const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
+            const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
+            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, (long long)(aEnd - ab) * 2);
+            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, (long long)(bEnd - bb) * 2);
+            /* rows of k past the end of an MN-contiguous matrix read as zero by themselves;
+               a K-contiguous row would run on into the next row, so those lanes are sent
+               out of range explicitly (last slab only) */
+            const bool tail = mayHangOver && k0 + BKT > K;
 #pragma unroll
-        for (int s = 0; s < NA; s++) {
-            if (AKC)
-                ra[s] = ld8_kcontig<VEC>(aRow[s], k0 + aK[s], K);
-            else
-                ra[s] = ld8_mncontig<VEC>(aRow[s], p.lda, k0 + aK[s], K, m0 + aMN[s], M);
+            for (int s = 0; s < NA; s++) {
+                int off = aOff[s];
+                if (AKC && tail && k0 + aK[s] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                ra[s] = buffer_load_f16x8(ar, off);
+            }
+#pragma unroll
+            for (int s = 0; s < NB; s++) {
+                int off = bOff[s];
+                if (BKC && tail && k0 + bK[s] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                rb[s] = buffer_load_f16x8(br, off);
+            }
         }
+        else {
+            /* generic path: any alignment, element by element, predicated */
 #pragma unroll
-        for (int s = 0; s < NB; s++) {
-            if (BKC)
-                rb[s] = ld8_kcontig<VEC>(bRow[s], k0 + bK[s], K);
-            else
-                rb[s] = ld8_mncontig<VEC>(bRow[s], p.ldb, k0 + bK[s], K, n0 + bMN[s], N);
+            for (int s = 0; s < NA; s++) {
+                f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (AKC) {
+                    int r = m0 + aMN[s] < M - 1 ? m0 + aMN[s] : M - 1;
+                    const half_t * rp = A + (size_t)r * p.lda;
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (k0 + aK[s] + e < K)
+                            v[e] = rp[k0 + aK[s] + e];
+                }
+                else if (k0 + aK[s] < K) {
+                    const half_t * rp = A + (size_t)(k0 + aK[s]) * p.lda;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        int c = m0 + aMN[s] + e < M - 1 ? m0 + aMN[s] + e : M - 1;
+                        v[e] = rp[c];
+                    }
+                }
+                ra[s] = v;
+            }
+#pragma unroll
+            for (int s = 0; s < NB; s++) {
+                f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (BKC) {
+                    int r = n0 + bMN[s] < N - 1 ? n0 + bMN[s] : N - 1;
+                    const half_t * rp = B + (size_t)r * p.ldb;
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (k0 + bK[s] + e < K)
+                            v[e] = rp[k0 + bK[s] + e];
+                }
+                else if (k0 + bK[s] < K) {
+                    const half_t * rp = B + (size_t)(k0 + bK[s]) * p.ldb;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        int c = n0 + bMN[s] + e < N - 1 ? n0 + bMN[s] + e : N - 1;
+                        v[e] = rp[c];
+                    }
+                }
+                rb[s] = v;
+            }
         }
     };
 
     auto store_lds = [&](int buf) {
 #pragma unroll
-        for (int s = 0; s < NA; s++) {
-            if (AKC)
-                *reinterpret_cast<f16x8 *>(&As[buf][aMN[s] * LDK + aK[s]]) = ra[s];
-            else {
+        for (int s = 0; s < NA; s++)
+            *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = ra[s];
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    As[buf][(aMN[s] + e) * LDK + aK[s]] = ra[s][e];
-            }
+        for (int s = 0; s < NB; s++)
+            *reinterpret_cast<f16x8 *>(&Bs[buf][bLds[s]]) = rb[s];
+    };
+
+    /* ---- fragments: two register sets, [set][k step][block] ------------------- */
+    f16x8 fa[2][KS][TI], fb[2][KS][TJ];
+
+    /* lane's place in a transposing read: which of the four k rows, which 4 columns */
+    const int trRow = (lane & 15) >> 2;
+    const int trCol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    auto read_frags = [&](auto SET, int buf) {
+        constexpr int set = decltype(SET)::value;
+        if constexpr (AKC) {
+            const half_t * as = &As[buf][(wm0 + l32) * LDK + 8 * lh];
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+                    fa[set][kk][i] = *reinterpret_cast<const f16x8 *>(as + i * 32 * LDK + kk * 16);
         }
+        else {
+            const half_t * as = &As[buf][(8 * lh + trRow) * LDA + wm0 + trCol];
 #pragma unroll
-        for (int s = 0; s < NB; s++) {
-            if (BKC)
-                *reinterpret_cast<f16x8 *>(&Bs[buf][bMN[s] * LDK + bK[s]]) = rb[s];
-            else {
+            for (int kk = 0; kk < KS; kk++)
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    Bs[buf][(bMN[s] + e) * LDK + bK[s]] = rb[s][e];
-            }
+                for (int i = 0; i < TI; i++) {
+                    f16x4 lo = lds_read_tr16(as + (kk * 16) * LDA + i * 32);
+                    f16x4 hi = lds_read_tr16(as + (kk * 16 + 4) * LDA + i * 32);
+                    fa[set][kk][i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+        }
+        if constexpr (BKC) {
+            const half_t * bs = &Bs[buf][(wn0 + l32) * LDK + 8 * lh];
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    fb[set][kk][j] = *reinterpret_cast<const f16x8 *>(bs + j * 32 * LDK + kk * 16);
+        }
+        else {
+            const half_t * bs = &Bs[buf][(8 * lh + trRow) * LDB + wn0 + trCol];
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    f16x4 lo = lds_read_tr16(bs + (kk * 16) * LDB + j * 32);
+                    f16x4 hi = lds_read_tr16(bs + (kk * 16 + 4) * LDB + j * 32);
+                    fb[set][kk][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
         }
     };
 
@@ -186,66 +312,139 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.f;
 
-    const int nk = (K + BKT - 1) / BKT;
-    if (nk > 0) {
-        load_global(0);
-        store_lds(0);
-    }
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk)
-            load_global((kt + 1) * BKT);
-
-        const half_t * as = &As[buf][(wm0 + l32) * LDK + 8 * lh];
-        const half_t * bs = &Bs[buf][(wn0 + l32) * LDK + 8 * lh];
+    /* MFMAs number first .. last-1 of the slab, in (k step, i, j) order */
+    auto mfma_range = [&](auto SET, int first, int last) {
+        constexpr int set = decltype(SET)::value;
 #pragma unroll
-        for (int kk = 0; kk < BKT / 16; kk++) {
-            f16x8 af[TI], bf[TJ];
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-                af[i] = *reinterpret_cast<const f16x8 *>(as + i * 32 * LDK + kk * 16);
-#pragma unroll
-            for (int j = 0; j < TJ; j++)
-                bf[j] = *reinterpret_cast<const f16x8 *>(bs + j * 32 * LDK + kk * 16);
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int t = first; t < last; t++) {
+            const int kk = t / (TI * TJ), i = (t / TJ) % TI, j = t % TJ;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][kk][i], fb[set][kk][j], acc[i][j], 0, 0, 0);
         }
+    };
 
-        if (kt + 1 < nk)
-            store_lds(buf ^ 1);
+    const int nk = (K + BKT - 1) / BKT;
+
+    /* One slab: fragments of slab kt are in register set SET and came from LDS stage SET.
+       FULL: slabs kt+1 and kt+2 exist and are complete, so the slab is straight-line code. */
+    auto slab = [&](auto SET, auto FULL, int kt) {
+        constexpr int set = decltype(SET)::value;
+        constexpr bool full = decltype(FULL)::value != 0;
+        if (full || kt + 1 < nk)
+            store_lds(set ^ 1);                  /* slab kt+1, fetched during slab kt-1 */
+        mfma_range(SET, 0, PRE);
+        if constexpr (full) {
+#pragma unroll
+            for (int g = 0; g < PRE; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* one MFMA */
+                __builtin_amdgcn_sched_group_barrier(0x200, (NA + NB + PREG - 1) / PREG, 0);   /* LDS writes */
+                __builtin_amdgcn_sched_group_barrier(0x006, 2, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();                         /* stage set^1 complete; stage set no longer read by anyone */
+        __builtin_amdgcn_sched_barrier(0);
+        if (full)
+            load_global(IntC<0>(), (kt + 2) * BKT);
+        else if (kt + 2 < nk)
+            load_global(IntC<1>(), (kt + 2) * BKT);
+        if (full || kt + 1 < nk)
+            read_frags(IntC<set ^ 1>(), set ^ 1);
+        mfma_range(SET, PRE, NMFMA);
+        if constexpr (full) {
+            constexpr int REST = NMFMA - PRE;
+            constexpr int NREAD = (AKC ? 1 : 2) * KS * TI + (BKC ? 1 : 2) * KS * TJ;
+#pragma unroll
+            for (int g = 0; g < REST; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* one MFMA */
+                __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + REST - 1) / REST, 0);   /* LDS reads */
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                            /* one global read */
+                __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    if (nk > 0) {
+        load_global(IntC<1>(), 0);
+        store_lds(0);
+        if (nk > 1)
+            load_global(IntC<1>(), BKT);
         __syncthreads();
+        read_frags(IntC<0>(), 0);
+        const int nkFull = K / BKT;
+        int kt = 0;
+        for (; kt + 3 < nkFull; kt += 2) {
+            slab(IntC<0>(), IntC<1>(), kt);
+            slab(IntC<1>(), IntC<1>(), kt + 1);
+        }
+        for (; kt < nk; kt += 2) {
+            slab(IntC<0>(), IntC<0>(), kt);
+            if (kt + 1 < nk)
+                slab(IntC<1>(), IntC<0>(), kt + 1);
+        }
     }
 
+    /* ---- epilogue: accumulator register r of lane l is element
+       (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block ------------------------ */
     const float alpha = p.alpha, beta = p.beta;
     const OutT * __restrict__ bias = static_cast<const OutT *>(p.bias);
+    const int biasMode = p.biasMode;
+
+    if constexpr (VEC) {
+        /* the wave's rows of c as one buffer that ends where c ends: rows past M drop off
+           its end, columns past N are sent out of range. Row-indexed bias is not handled here. */
+        if (m0 + wm0 >= M)
+            return;
+        OutT * cw = C + (size_t)(m0 + wm0) * p.ldc;
+        __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * (long long)sizeof(OutT));
+        const unsigned rowPitch = (unsigned)p.ldc * (unsigned)sizeof(OutT);
 #pragma unroll
-    for (int j = 0; j < TJ; j++) {
-        const int col = n0 + wn0 + j * 32 + l32;
-        if (col >= N)
-            continue;
-        float bcol = 0.f;
-        if (p.biasMode == BIAS_COL)
-            bcol = (float)bias[col];
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + col) * (unsigned)sizeof(OutT)
+                                          : (unsigned)NTSAMD_OOB_OFFSET;
+            float bcol = 0.f;
+            if (biasMode == BIAS_COL && col < N)
+                bcol = (float)bias[col];
 #pragma unroll
-        for (int i = 0; i < TI; i++) {
+            for (int i = 0; i < TI; i++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (row < M) {
-                    OutT * cp = C + (size_t)row * p.ldc + col;
-                    float v = alpha * acc[i][j][r];
+                for (int r = 0; r < 16; r++) {
+                    const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    float v = alpha * acc[i][j][r] + bcol;
                     if (beta != 0.f)
-                        v += beta * (float)(*cp);
-                    if (p.biasMode == BIAS_ROW)
-                        v += (float)bias[(row / p.biasRowDiv) % p.biasLen];
-                    else
-                        v += bcol;
-                    *cp = (OutT)v;
+                        v += beta * buffer_load_out<OutT>(cr, (int)off);
+                    buffer_store_out<OutT>((OutT)v, cr, (int)off);
+                }
+            }
+        }
+    }
+    else {
+        /* generic path: plain pointers, per-element bounds, every bias mode */
+#pragma unroll
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col >= N)
+                continue;
+            float bcol = 0.f;
+            if (biasMode == BIAS_COL)
+                bcol = (float)bias[col];
+#pragma unroll
+            for (int i = 0; i < TI; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                    if (row < M) {
+                        OutT * cp = C + (size_t)row * p.ldc + col;
+                        float v = alpha * acc[i][j][r];
+                        if (beta != 0.f)
+                            v += beta * (float)(*cp);
+                        if (biasMode == BIAS_ROW)
+                            v += (float)bias[(row / p.biasRowDiv) % p.biasLen];
+                        else
+                            v += bcol;
+                        *cp = (OutT)v;
+                    }
                 }
             }
         }
@@ -260,29 +459,9 @@ static int launch_f16_one(const GemmParams & p0, const PT & tab, hipStream_t str
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, AKC, BKC, VEC, PT>),
+    hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, S::MINW16, AKC, BKC, VEC, PT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();
-}
-
-template <bool AKC, bool BKC>
-static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, bool vec, bool outF32, int cfg,
-                            hipStream_t stream)
-{
-    NoPtrs none = {0};
-    if (ptrs) {
-        if (outF32)
-            return launch_f16_one<float, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
-        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
-    }
-    /* half inputs with a float result are outside the main path: one generic instantiation */
-    if (outF32)
-        return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
-    if (!vec)
-        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
-    if (cfg == CFG_128x128)
-        return launch_f16_one<half_t, CFG_128x128, AKC, BKC, true, NoPtrs>(p, none, stream);
-    return launch_f16_one<half_t, CFG_64x64, AKC, BKC, true, NoPtrs>(p, none, stream);
 }
 
 }  // namespace ntsamd

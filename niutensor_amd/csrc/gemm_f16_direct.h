@@ -1,0 +1,417 @@
+/*
+ * fp16 GEMM for gfx950, main path: global memory -> LDS without passing through
+ * registers (buffer_load_dwordx4 ... lds), four LDS stages, fp32 accumulation.
+ * Used for 16-byte aligned operands with a half result; everything else goes
+ * through the register-staged kernel in gemm_f16.h. Same arithmetic, same
+ * fragment layouts (see that file for what v_mfma_f32_32x32x16_f16 and
+ * ds_read_b64_tr_b16 expect).
+ *
+ * An LDS-direct load writes the 64 lanes' 16 bytes to 1 KB of consecutive LDS, at
+ * an address the whole wave shares; WHICH 16 bytes of global memory a lane fetches
+ * is free. That freedom is what keeps the fragment reads free of bank conflicts
+ * without padding inside a chunk:
+ *   K-contiguous operand (rows of mn, 32 halves = 64 bytes of k per row): a chunk
+ *       is 16 rows. The four 16-byte columns of row r are stored permuted,
+ *       column c at position c ^ ((r >> 1) & 3); eight consecutive rows reading
+ *       the same logical column then hit eight different 16-byte bank groups.
+ *   MN-contiguous operand (rows of k): a chunk holds rows k, k + NCH, k + 2 NCH ...
+ *       (NCH chunks per slab), and chunks are 1 KB + 32 bytes apart, so the four
+ *       consecutive k rows of one transposing read sit in four different chunks,
+ *       32 bytes apart modulo 128.
+ *
+ * Pipeline: loads for slab t+3 are issued while slab t is multiplied (about 2.5
+ * slabs = 2500 cycles of cover for the global latency). A slab is two MFMA k
+ * steps; its fragments are double-buffered per k step. The one barrier of a slab
+ * sits between the two steps: by then the wave has waited for its own loads of
+ * slab t+1 (vmcnt) and for its own last reads of slab t (lgkmcnt), so after the
+ * barrier every wave may read slab t+1 and, one step later, overwrite the stage
+ * of slab t-1... and the MFMAs of the second step are ready to issue the moment
+ * the barrier opens, because their fragments were read before it.
+ */
+#pragma once
+#include "gemm_common.h"
+#include "gemm_f16.h"
+
+namespace ntsamd {
+
+/* s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt in bits 3:0 and 15:14) */
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+__device__ __forceinline__ void wait_lgkmcnt0()
+{
+    __builtin_amdgcn_s_waitcnt(0xC07F);     /* lgkmcnt = 0, vmcnt and expcnt left at their maxima */
+}
+
+/* A raw buffer descriptor as four scalars (base low, base high, bytes, format word), for
+   the loads below that the compiler must not see as memory operations of its own. */
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ i32x4 make_desc(const void * base, long long bytes)
+{
+    const unsigned long long b = reinterpret_cast<unsigned long long>(base);
+    i32x4 d;
+    d[0] = (int)(unsigned)b;
+    d[1] = (int)((b >> 32) & 0xffffu);
+    d[2] = (unsigned long long)bytes >> 31 ? 0x7fffffff : (int)bytes;
+    d[3] = 0x00020000;
+    return d;
+}
+
+/* Global memory -> LDS, 16 bytes per lane: lane l's data lands at ldsAddr + 16 l (ldsAddr is the
+   same for the whole wave and travels in M0). Written as inline assembly on purpose: as a
+   compiler builtin, every later LDS read is made to wait for ALL outstanding loads (the compiler
+   cannot tell which LDS bytes a load in flight will write), which would serialise the
+   pipeline. The waits are placed by hand instead (wait_vmcnt below). */
+__device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byteOffset)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(ldsAddr), "v"(byteOffset), "s"(desc)
+                 : "memory");
+}
+
+template <int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC>
+__global__ void __launch_bounds__(WGM * WGN * 64, MINW)
+gemm_f16_direct_kernel(const GemmParams p)
+{
+    constexpr int BKT = 32, KS = 2, NSTAGE = 4;
+    constexpr int NW = WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TI = WM / 32, TJ = WN / 32;
+    /* per-operand LDS geometry, bytes */
+    constexpr int A_RPC = AKC ? 16 : 512 / BM;             /* rows per chunk */
+    constexpr int B_RPC = BKC ? 16 : 512 / BN;
+    constexpr int A_NCH = AKC ? BM / 16 : BKT / A_RPC;     /* chunks per slab */
+    constexpr int B_NCH = BKC ? BN / 16 : BKT / B_RPC;
+    constexpr int A_CP = AKC ? 1024 : 1056;                /* chunk pitch */
+    constexpr int B_CP = BKC ? 1024 : 1056;
+    constexpr int A_BYTES = A_NCH * A_CP;
+    constexpr int B_BYTES = B_NCH * B_CP;
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    constexpr int NLA = A_NCH / NW, NLB = B_NCH / NW;      /* load instructions per wave and slab */
+    constexpr int NL = NLA + NLB;
+    static_assert(A_NCH % NW == 0 && B_NCH % NW == 0, "chunks must divide among the waves");
+    static_assert(AKC || A_NCH >= 4, "transposing reads need four chunks");
+    static_assert(BKC || B_NCH >= 4, "transposing reads need four chunks");
+
+    __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
+
+    const TileCoord tc = tile_of_workgroup(p);
+    const half_t * __restrict__ A = static_cast<const half_t *>(p.a) + (long long)tc.batch * p.strideA;
+    const half_t * __restrict__ B = static_cast<const half_t *>(p.b) + (long long)tc.batch * p.strideB;
+    half_t * __restrict__ C = static_cast<half_t *>(p.c) + (long long)tc.batch * p.strideC;
+
+    const int M = p.M, N = p.N, K = p.K;
+    const int m0 = tc.tm * BM, n0 = tc.tn * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    /* ---- what each lane fetches for each of its wave's chunks -------------------- */
+    int aOff[NLA], bOff[NLB];      /* byte offset from the slab base */
+    int aKc[NLA], bKc[NLB];        /* K-contiguous: first k of the lane's 16 bytes inside the slab */
+#pragma unroll
+    for (int q = 0; q < NLA; q++) {
+        const int ch = wave * NLA + q;
+        if (AKC) {
+            int row = ch * 16 + (lane >> 2);
+            int col = (lane & 3) ^ ((row >> 1) & 3);
+            aKc[q] = col * 8;
+            int r = m0 + row < M - 1 ? row : M - 1 - m0;
+            aOff[q] = (r * p.lda + col * 8) * 2;
+        }
+        else {
+            constexpr int LPR = 64 / A_RPC;                  /* lanes per row */
+            int krow = ch + A_NCH * (lane / LPR);
+            int c = (lane % LPR) * 8;
+            c = m0 + c < M - 8 ? c : M - 8 - m0;
+            aKc[q] = 0;
+            aOff[q] = (krow * p.lda + c) * 2;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NLB; q++) {
+        const int ch = wave * NLB + q;
+        if (BKC) {
+            int row = ch * 16 + (lane >> 2);
+            int col = (lane & 3) ^ ((row >> 1) & 3);
+            bKc[q] = col * 8;
+            int r = n0 + row < N - 1 ? row : N - 1 - n0;
+            bOff[q] = (r * p.ldb + col * 8) * 2;
+        }
+        else {
+            constexpr int LPR = 64 / B_RPC;
+            int krow = ch + B_NCH * (lane / LPR);
+            int c = (lane % LPR) * 8;
+            c = n0 + c < N - 8 ? c : N - 8 - n0;
+            bKc[q] = 0;
+            bOff[q] = (krow * p.ldb + c) * 2;
+        }
+    }
+
+    const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
+    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
+    const half_t * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
+    const half_t * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+
+    const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);
+
+    /* issue load number q (0 .. NL-1) of this wave for slab kt */
+    auto issue_load = [&](auto TAIL, int kt, int q) {
+        constexpr bool mayHangOver = decltype(TAIL)::value != 0;
+        const int k0 = kt * BKT;
+        const unsigned stage = ldsBase + (unsigned)((kt % NSTAGE) * STAGE);
+        const bool tail = mayHangOver && k0 + BKT > K;
+        if (q < NLA) {
+            const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
+            int off = aOff[q];
+            if (AKC && tail && k0 + aKc[q] >= K)
+                off = NTSAMD_OOB_OFFSET;
+            lds_dma16(make_desc(ab, (long long)(aEnd - ab) * 2), stage + (unsigned)((wave * NLA + q) * A_CP), off);
+        }
+        else {
+            const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
+            int off = bOff[q - NLA];
+            if (BKC && tail && k0 + bKc[q - NLA] >= K)
+                off = NTSAMD_OOB_OFFSET;
+            lds_dma16(make_desc(bb, (long long)(bEnd - bb) * 2), stage + (unsigned)(A_BYTES + (wave * NLB + (q - NLA)) * B_CP), off);
+        }
+    };
+
+    auto issue_loads = [&](auto TAIL, int kt) {
+#pragma unroll
+        for (int q = 0; q < NL; q++)
+            issue_load(TAIL, kt, q);
+    };
+
+    /* ---- fragment addresses (byte offsets inside a stage) ---------------------------- */
+    const int trRow = (lane & 15) >> 2;
+    const int trCol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    int aFrag[KS], bFrag[KS];      /* K-contiguous: offset for k step kk, block 0 */
+    int aTr[KS][2], bTr[KS][2];    /* MN-contiguous: offset for k step kk, half h, block 0 */
+#pragma unroll
+    for (int kk = 0; kk < KS; kk++) {
+        const int sw = (l32 >> 1) & 3;
+        aFrag[kk] = (wm0 + l32) * 64 + ((kk * 2 + lh) ^ sw) * 16;
+        bFrag[kk] = A_BYTES + (wn0 + l32) * 64 + ((kk * 2 + lh) ^ sw) * 16;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int kr = 16 * kk + 8 * lh + 4 * h + trRow;
+            aTr[kk][h] = (kr % A_NCH) * A_CP + (kr / A_NCH) * (BM * 2) + (wm0 + trCol) * 2;
+            bTr[kk][h] = A_BYTES + (kr % B_NCH) * B_CP + (kr / B_NCH) * (BN * 2) + (wn0 + trCol) * 2;
+        }
+    }
+
+    f16x8 fa[2][TI], fb[2][TJ];
+
+    /* fragment number f (a blocks first, then b blocks) of k step KK of the slab in `stage` */
+    auto read_frag = [&](auto KKC, const char * stage, int f) {
+        constexpr int kk = decltype(KKC)::value;
+        if (f < TI) {
+            const int i = f;
+            if constexpr (AKC)
+                fa[kk][i] = *reinterpret_cast<const f16x8 *>(stage + aFrag[kk] + i * 32 * 64);
+            else {
+                f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][0] + i * 64));
+                f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][1] + i * 64));
+                fa[kk][i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+        else {
+            const int j = f - TI;
+            if constexpr (BKC)
+                fb[kk][j] = *reinterpret_cast<const f16x8 *>(stage + bFrag[kk] + j * 32 * 64);
+            else {
+                f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][0] + j * 64));
+                f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][1] + j * 64));
+                fb[kk][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+    };
+
+    auto read_frags = [&](auto KKC, const char * stage) {
+#pragma unroll
+        for (int f = 0; f < TI + TJ; f++)
+            read_frag(KKC, stage, f);
+    };
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.f;
+
+    constexpr int NM = TI * TJ;                                       /* MFMAs per k step */
+    constexpr int NF = TI + TJ;                                       /* fragments per k step */
+    constexpr int RPF = (AKC ? 1 : 2);                                /* LDS reads per a fragment */
+
+    const int nk = (K + BKT - 1) / BKT;
+
+    /* One k step: its NM MFMAs, with the reads of the OTHER register set (from `src`, if
+       READ) and this wave's loads of slab `loadKt` (if LOAD) dealt out between them, in
+       program order AND pinned there: an MFMA holds the matrix pipe for 32 cycles but
+       takes one issue slot, so the other instructions ride in its shadow. */
+    auto k_step = [&](auto KKC, auto READC, auto LOADC, auto TAILC, const char * src, int loadKt) {
+        constexpr int kk = decltype(KKC)::value;
+        constexpr bool doRead = decltype(READC)::value != 0;
+        constexpr bool doLoad = decltype(LOADC)::value != 0;
+#pragma unroll
+        for (int g = 0; g < NM; g++) {
+            const int i = g / TJ, j = g % TJ;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+            if (doRead) {
+                /* fragments f with f * NM / NF == g: spread evenly over the MFMAs */
+#pragma unroll
+                for (int f = 0; f < NF; f++)
+                    if (f * NM / NF == g)
+                        read_frag(IntC<kk ^ 1>(), src, f);
+            }
+            if (doLoad) {
+#pragma unroll
+                for (int q = 0; q < NL; q++)
+                    if (q * NM / NL == g)
+                        issue_load(TAILC, loadKt, q);
+            }
+        }
+    };
+
+    /* One slab. AHEAD = how many later slabs exist (capped at 3): decides which loads are
+       issued and how many may still be in flight at the barrier. */
+    auto slab = [&](auto AHEADC, auto TAILC, int kt) {
+        constexpr int ahead = decltype(AHEADC)::value;
+        const char * stage = lds + (kt % NSTAGE) * STAGE;
+        const char * next = lds + ((kt + 1) % NSTAGE) * STAGE;
+
+        /* k step 0: multiply it, fetch step 1 of this slab, start the loads of slab kt+3 */
+        k_step(IntC<0>(), IntC<1>(), IntC<(ahead >= 3)>(), TAILC, stage, kt + 3);
+        __builtin_amdgcn_sched_barrier(0);
+
+        /* slab kt+1 must have landed: at most the loads of slabs kt+2 and kt+3 stay in flight */
+        if constexpr (ahead >= 3)
+            wait_vmcnt<2 * NL>();
+        else if constexpr (ahead == 2)
+            wait_vmcnt<NL>();
+        else
+            wait_vmcnt<0>();
+        wait_lgkmcnt0();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+
+        /* k step 1: multiply it, fetch step 0 of the next slab */
+        k_step(IntC<1>(), IntC<(ahead >= 1)>(), IntC<0>(), TAILC, next, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (nk > 0) {
+        /* prologue: three slabs in flight, then wait for the first */
+        issue_loads(IntC<1>(), 0);
+        if (nk > 1)
+            issue_loads(IntC<1>(), 1);
+        if (nk > 2)
+            issue_loads(IntC<1>(), 2);
+        if (nk > 2)
+            wait_vmcnt<2 * NL>();
+        else if (nk > 1)
+            wait_vmcnt<NL>();
+        else
+            wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(IntC<0>(), lds);
+
+        const int nkFull = K / BKT;              /* slabs entirely inside K */
+        int kt = 0;
+        for (; kt + 3 < nkFull; kt++)
+            slab(IntC<3>(), IntC<0>(), kt);      /* slab kt+3 is complete: no tail handling */
+        for (; kt + 3 < nk; kt++)
+            slab(IntC<3>(), IntC<1>(), kt);
+        if (kt + 2 < nk) {
+            slab(IntC<2>(), IntC<0>(), kt);
+            kt++;
+        }
+        if (kt + 1 < nk) {
+            slab(IntC<1>(), IntC<0>(), kt);
+            kt++;
+        }
+        if (kt < nk)
+            slab(IntC<0>(), IntC<0>(), kt);
+    }
+
+    /* ---- epilogue: accumulator register r of lane l is element
+       (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block. The wave's rows of c are one
+       buffer that ends where c ends: rows past M drop off it, columns past N are sent
+       out of range. ------------------------------------------------------------------- */
+    if (m0 + wm0 >= M)
+        return;
+    const float alpha = p.alpha, beta = p.beta;
+    const half_t * __restrict__ bias = static_cast<const half_t *>(p.bias);
+    const int biasMode = p.biasMode;
+    half_t * cw = C + (size_t)(m0 + wm0) * p.ldc;
+    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
+    const unsigned rowPitch = (unsigned)p.ldc * 2u;
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+        const int col = n0 + wn0 + j * 32 + l32;
+        const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+        float bcol = 0.f;
+        if (biasMode == BIAS_COL && col < N)
+            bcol = (float)bias[col];
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                float v = alpha * acc[i][j][r] + bcol;
+                if (beta != 0.f)
+                    v += beta * buffer_load_out<half_t>(cr, (int)off);
+                buffer_store_out<half_t>((half_t)v, cr, (int)off);
+            }
+        }
+    }
+}
+
+template <int CFG, bool AKC, bool BKC>
+static int launch_f16_direct(const GemmParams & p0, hipStream_t stream)
+{
+    typedef TileShape<CFG> S;
+    GemmParams p = p0;
+    p.tilesM = (p.M + S::BM - 1) / S::BM;
+    p.tilesN = (p.N + S::BN - 1) / S::BN;
+    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC>),
+                       grid, dim3(S::WGM * S::WGN * 64), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+template <bool AKC, bool BKC>
+static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, bool vec, bool outF32, int cfg,
+                            hipStream_t stream)
+{
+    NoPtrs none = {0};
+    if (ptrs) {
+        if (outF32)
+            return launch_f16_one<float, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
+        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
+    }
+    /* half inputs with a float result are outside the main path: one generic instantiation */
+    if (outF32)
+        return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
+    if (!vec)
+        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
+    if (cfg == CFG_256x256)
+        return launch_f16_direct<CFG_256x256, AKC, BKC>(p, stream);
+    if (cfg == CFG_128x128)
+        return launch_f16_direct<CFG_128x128, AKC, BKC>(p, stream);
+    return launch_f16_direct<CFG_64x64, AKC, BKC>(p, stream);
+}
+
+}  // namespace ntsamd

@@ -137,15 +137,22 @@ bool aligned16(const void * p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
-/* NTSAMD_TILE_CFG=0|1 forces a tile shape (for measurements); otherwise big
-   tiles once they alone fill most of the 256 CUs */
-int choose_cfg(int M, int N, int count)
+/* NTSAMD_TILE_CFG=0|1|2 forces a tile shape (128x128, 64x64, 256x256 for half; for
+   measurements); otherwise the biggest tile that alone fills most of the 256 CUs */
+int choose_cfg(int M, int N, int count, bool half)
 {
     const char * e = getenv("NTSAMD_TILE_CFG");
-    if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0)
-        return e[0] - '0';
-    long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128) * count;
-    return tiles >= 192 ? CFG_128x128 : CFG_64x64;
+    if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
+        int cfg = e[0] - '0';
+        if (cfg == CFG_256x256 && !half)
+            cfg = CFG_128x128;
+        return cfg;
+    }
+    long long tiles128 = (long long)((M + 127) / 128) * ((N + 127) / 128) * count;
+    long long tiles256 = (long long)((M + 255) / 256) * ((N + 255) / 256) * count;
+    if (half && tiles256 >= 192)
+        return CFG_256x256;
+    return tiles128 >= 192 ? CFG_128x128 : CFG_64x64;
 }
 
 int run(int devID, void * stream, Kind kind, const Shape & s,
@@ -198,7 +205,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                strideA % vecElems == 0 && strideB % vecElems == 0 &&
                lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) &&
                biasMode != NTSAMD_BIAS_ROW;
-    int cfg = choose_cfg(s.M, s.N, count);
+    int cfg = choose_cfg(s.M, s.N, count, kind != KIND_F32);
     hipStream_t hs = static_cast<hipStream_t>(stream);
 
     int rc;
