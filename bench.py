@@ -130,8 +130,9 @@ def cpu_baseline(idx, budget_s=12.0):
     o = Oracle(native=True)
     cfg = configs()[idx]
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
-    # measured rates of this path: ~0.8 GFLOP/s when b is walked by column (NN), ~3 GFLOP/s when both are rows
-    rate = {1: 0.8e9, 2: 0.8e9, 3: 1.5e9, 4: 0.4e9, 5: 2.5e9}[idx]
+    # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
+    # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
+    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -171,6 +172,15 @@ def cpu_baseline(idx, budget_s=12.0):
             "sample": sample + " (%.1f s; %.2f GFLOP/s, -O3 -march=native)" % (dt, fl / dt / 1e9)}
 
 
+def measured_traffic(idx):
+    """HBM-side bytes per step from the committed rocprofv3 counter runs (profiles/hbm_traffic.json), or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f).get(str(idx))
+    except (OSError, ValueError):
+        return None
+
+
 def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     import torch
     wl = Workload(idx, dev, oracle)
@@ -191,6 +201,15 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     kt = min(ev.time(wl.run, stream, reps) for _ in range(5))
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
+    # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
+    if idx == 3:
+        roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
+                "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
+    else:
+        roof = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4)}
+    roof.update({"traffic": measured_traffic(idx), "kernel_us": round(kt / wl.launches * 1e6, 2),
+                 "mfma_tflops": round(achieved, 3), "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)})
     out = {
         "metric": "TFLOP/s & % of dense matrix peak for MatrixMul/Batched (fp32, fp16), 1 GPU",
         "value": round(wl.flops / wall / 1e12, 3),
@@ -208,10 +227,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
                    "launches_per_step": wl.launches, "inputs": "resident in HBM", "flops_per_step": wl.flops,
                    "algorithmic_bytes_per_step": wl.bytes},
         "pct_of_peak": round(100.0 * wl.flops / wall / 1e12 / peak, 2),
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel_us": round(kt / wl.launches * 1e6, 2),
-                     "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)},
+        "roofline": roof,
     }
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline(idx)
@@ -226,6 +242,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="configuration 1-5 (default 2, the MulAndShift linear layer)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain device copy of known size (scale for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path has no multi-GPU part (each product is independent); "
@@ -238,6 +256,15 @@ def main():
         raise SystemExit("bench.py needs a gfx950 GPU")
     nt.load()
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        # 256 MiB read + 256 MiB written per copy: what a profiler's HBM counters should show
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "copies": args.steps}))
+        return
     oracle = Oracle()
     if args.all:
         for idx in (1, 3, 4, 5):

@@ -449,7 +449,7 @@ static int launch_f32_one(const GemmParams & p0, const PT & tab, hipStream_t str
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, 16, S::WGM, S::WGN, AKC, BKC, VEC, PT>),
+    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, S::BKT32, S::WGM, S::WGN, AKC, BKC, VEC, PT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();
 }

@@ -137,8 +137,20 @@ bool aligned16(const void * p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+/* Relative run time of a product under a tile shape: rounds of workgroups (256 CUs x the
+   workgroups a CU holds at once) times the work of one tile, divided by how fast the shape
+   runs relative to the best one on a product that fits it (measured: small tiles re-read
+   operands from LDS more often per MFMA, which costs fp16 far more than fp32). */
+double tile_cost(int M, int N, int count, int bm, int bn, int perCU, double quality)
+{
+    long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count;
+    long long slots = 256LL * perCU;
+    long long rounds = (tiles + slots - 1) / slots;
+    return (double)rounds * bm * bn / quality;
+}
+
 /* NTSAMD_TILE_CFG=0|1|2 forces a tile shape (128x128, 64x64, 256x256 for half; for
-   measurements); otherwise the biggest tile that alone fills most of the 256 CUs */
+   measurements); otherwise the shape with the lowest estimated run time */
 int choose_cfg(int M, int N, int count, bool half)
 {
     const char * e = getenv("NTSAMD_TILE_CFG");
@@ -148,11 +160,19 @@ int choose_cfg(int M, int N, int count, bool half)
             cfg = CFG_128x128;
         return cfg;
     }
-    long long tiles128 = (long long)((M + 127) / 128) * ((N + 127) / 128) * count;
-    long long tiles256 = (long long)((M + 255) / 256) * ((N + 255) / 256) * count;
-    if (half && tiles256 >= 192)
-        return CFG_256x256;
-    return tiles128 >= 192 ? CFG_128x128 : CFG_64x64;
+    int best = CFG_64x64;
+    double bestCost = tile_cost(M, N, count, 64, 64, 2, half ? 0.2 : 0.8);
+    double c128 = tile_cost(M, N, count, 128, 128, 2, half ? 0.45 : 1.0);
+    if (c128 <= bestCost) {
+        best = CFG_128x128;
+        bestCost = c128;
+    }
+    if (half) {
+        double c256 = tile_cost(M, N, count, 256, 256, 1, 1.0);
+        if (c256 <= bestCost)
+            best = CFG_256x256;
+    }
+    return best;
 }
 
 int run(int devID, void * stream, Kind kind, const Shape & s,
