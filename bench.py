@@ -173,32 +173,37 @@ def cpu_baseline(idx, budget_s=12.0):
 
 
 def measured_traffic(idx):
-    """HBM-side bytes per step from the committed rocprofv3 counter runs (profiles/hbm_traffic.json), or None."""
+    """HBM-side bytes per step from the committed rocprofv3 counter runs: the table in
+    profiles/hbm_traffic_per_step.md (rows "| configuration | bytes |"), or None."""
+    import re
     try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            return json.load(f).get(str(idx))
-    except (OSError, ValueError):
-        return None
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic_per_step.md")) as f:
+            for line in f:
+                m = re.match(r"\|\s*(\d+)\s*\|\s*(\d+)\s*\|", line)
+                if m and int(m.group(1)) == idx:
+                    return int(m.group(2))
+    except OSError:
+        pass
+    return None
 
 
 def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     import torch
     wl = Workload(idx, dev, oracle)
     cfg = wl.cfg
+    ev = HipEvents()
+    stream = torch.cuda.current_stream(dev).cuda_stream
     for _ in range(warmup):
         wl.run()
     torch.cuda.synchronize()
+    # the timed region: wall clock around it, and HIP events on the stream the launches go to inside it
     t0 = time.perf_counter()
-    for _ in range(steps):
-        wl.run()
+    kt = ev.time(wl.run, stream, steps)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-
-    # the kernel alone: HIP events on the stream the launches go to, best of 5 groups
-    ev = HipEvents()
-    stream = torch.cuda.current_stream(dev).cuda_stream
+    # shortest of five more groups of launches, reported beside the average (clock and power state move it by a few %)
     reps = max(10, min(200, steps))
-    kt = min(ev.time(wl.run, stream, reps) for _ in range(5))
+    kt_best = min(ev.time(wl.run, stream, reps) for _ in range(5))
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
     # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
@@ -209,6 +214,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
         roof = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4)}
     roof.update({"traffic": measured_traffic(idx), "kernel_us": round(kt / wl.launches * 1e6, 2),
+                 "kernel_us_best": round(kt_best / wl.launches * 1e6, 2),
                  "mfma_tflops": round(achieved, 3), "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)})
     out = {
         "metric": "TFLOP/s & % of dense matrix peak for MatrixMul/Batched (fp32, fp16), 1 GPU",

@@ -350,33 +350,105 @@ gemm_f16_direct_kernel(const GemmParams p)
        (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block. The wave's rows of c are one
        buffer that ends where c ends: rows past M drop off it, columns past N are sent
        out of range. ------------------------------------------------------------------- */
-    if (m0 + wm0 >= M)
-        return;
     const float alpha = p.alpha, beta = p.beta;
     const half_t * __restrict__ bias = static_cast<const half_t *>(p.bias);
     const int biasMode = p.biasMode;
     half_t * cw = C + (size_t)(m0 + wm0) * p.ldc;
-    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
     const unsigned rowPitch = (unsigned)p.ldc * 2u;
+
+    /* Wide path (beta == 0, rows of c 16-byte aligned): a lane owns one COLUMN of each block,
+       so storing straight from the accumulators means 2-byte stores, 64 contiguous bytes per
+       row and instruction, and the store instruction count (16 per block) bounds the epilogue.
+       Instead each wave turns 32 rows at a time through its own piece of LDS (the stages are
+       free by now) and writes 16 bytes per lane: whole rows of the wave's tile, whole cache
+       lines, an eighth of the instructions. */
+    const bool wide = beta == 0.f && (p.ldc & 7) == 0 && (N & 7) == 0 && (reinterpret_cast<size_t>(C) & 15) == 0;
+    if (wide) {
+        constexpr int PITCH = TJ * 64 + 16;          /* bytes; 4 rows apart = 64 bytes apart modulo 128 */
+        constexpr int LPR = TJ * 4;                  /* lanes that cover one row of the wave's tile */
+        constexpr int RPI = 64 / LPR;                /* rows per 16-byte store instruction */
+        constexpr int GROUP = 32 * PITCH;
+        static_assert(2 * GROUP * NW <= NSTAGE * STAGE, "epilogue staging must fit the stages");
+        __syncthreads();                             /* every wave has read its last fragments */
+        if (m0 + wm0 >= M)
+            return;
+        char * mine = lds + wave * 2 * GROUP;
+        __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
+        float bcol[TJ];
 #pragma unroll
-    for (int j = 0; j < TJ; j++) {
-        const int col = n0 + wn0 + j * 32 + l32;
-        const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
-        float bcol = 0.f;
-        if (biasMode == BIAS_COL && col < N)
-            bcol = (float)bias[col];
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            bcol[j] = biasMode == BIAS_COL && col < N ? (float)bias[col] : 0.f;
+        }
+        const int rdRow = lane / LPR, rdChunk = lane % LPR;
+        const int colW = n0 + wn0 + rdChunk * 8;
+        const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
 #pragma unroll
         for (int i = 0; i < TI; i++) {
+            char * buf = mine + (i & 1) * GROUP;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
-                float v = alpha * acc[i][j][r] + bcol;
-                if (beta != 0.f)
-                    v += beta * buffer_load_out<half_t>(cr, (int)off);
-                buffer_store_out<half_t>((half_t)v, cr, (int)off);
+            for (int j = 0; j < TJ; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = 8 * (r / 4) + 4 * lh + (r % 4);
+                    *reinterpret_cast<half_t *>(buf + row * PITCH + (j * 32 + l32) * 2) = (half_t)(alpha * acc[i][j][r] + bcol[j]);
+                }
+            /* the wave's own lanes exchange data through LDS: LDS executes one wave's
+               instructions in order, the fences only keep the compiler from reordering */
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int q = 0; q < 32 / RPI; q++) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(buf + (q * RPI + rdRow) * PITCH + rdChunk * 16);
+                const unsigned off = cOffW + (unsigned)(i * 32 + q * RPI) * rowPitch;
+                __builtin_amdgcn_raw_buffer_store_b128(v, cr, (int)off, 0, 0);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
+
+    if (m0 + wm0 >= M)
+        return;
+    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
+    /* beta is tested outside the loops: inside them every load of c would sit in a block of
+       its own, one memory round trip after the other */
+    auto narrow = [&](auto BETAC) {
+        constexpr bool useOld = decltype(BETAC)::value != 0;
+#pragma unroll
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+            float bcol = 0.f;
+            if (biasMode == BIAS_COL && col < N)
+                bcol = (float)bias[col];
+            float old[TI][16];
+            if constexpr (useOld) {
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        old[i][r] = buffer_load_out<half_t>(cr, (int)(cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch));
+            }
+#pragma unroll
+            for (int i = 0; i < TI; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    float v = alpha * acc[i][j][r] + bcol;
+                    if constexpr (useOld)
+                        v += beta * (float)old[i][r];
+                    buffer_store_out<half_t>((half_t)v, cr, (int)off);
+                }
             }
         }
-    }
+    };
+    if (beta != 0.f)
+        narrow(IntC<1>());
+    else
+        narrow(IntC<0>());
 }
 
 template <int CFG, bool AKC, bool BKC>

@@ -386,25 +386,49 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         float * cw = C + (size_t)(m0 + wm0) * p.ldc;
         __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 4);
         const unsigned rowPitch = (unsigned)p.ldc * 4u;
+        unsigned cOff[TJ];
+        float bcol[TJ];
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = n0 + wn0 + j * 32 + l32;
-            const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + (n0 + wn0 + j * 32 + l32)) * 4u
-                                          : (unsigned)NTSAMD_OOB_OFFSET;
-            float bcol = 0.f;
-            if (biasMode == BIAS_COL && col < N)
-                bcol = bias[col];
+            cOff[j] = col < N ? (unsigned)(4 * lh * p.ldc + col) * 4u : (unsigned)NTSAMD_OOB_OFFSET;
+            bcol[j] = biasMode == BIAS_COL && col < N ? bias[col] : 0.f;
+        }
+        /* beta is tested once, outside the loops: inside them the test would fence every
+           load of c off in a block of its own, one memory round trip after the other */
+        if (beta != 0.f) {
+            float old[TI][TJ][16];
 #pragma unroll
-            for (int i = 0; i < TI; i++) {
+            for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
-                    float v = alpha * acc[i][j][r] + bcol;
-                    if (beta != 0.f)
-                        v += beta * __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
-                }
-            }
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                        old[i][j][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
+                    }
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                        const float v = alpha * acc[i][j][r] + bcol[j] + beta * old[i][j][r];
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
+                    }
+        }
+        else {
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                        const float v = alpha * acc[i][j][r] + bcol[j];
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
+                    }
         }
     }
     else {
