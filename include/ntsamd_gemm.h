@@ -101,6 +101,40 @@ int ntsamd_matrix_mul_bias(int devID, void * stream,
                            const void * bias, int biasMode, int biasLen, int biasRowDiv);
 
 /*
+ * One product that also returns the column sums of op(b), gathered from the
+ * operand on its way through the kernel:
+ *   c = alpha * op(a) * op(b) + beta * c
+ *   colSum[j] = colSumBeta * colSum[j] + sum_k op(b)[k][j],   j < mc.
+ * This is the weight-gradient step of a linear layer: for c = x * w + bias the
+ * reference's GradMulAndShift (source/network/XBackwardMath.cpp:1774-1884)
+ * computes dE/dw = x^T * dE/dc with _MatrixMul (:635-637 via :1857-1879) and
+ * dE/dbias = column sums of dE/dc with _ReduceSum + _Sum into the gradient
+ * (:1805-1810), two passes over dE/dc. Here op(b) = dE/dc is read once.
+ * colSum has the data type of c and mc elements and must not overlap c.
+ * (X_FLOAT16, X_FLOAT16, X_FLOAT) is not accepted here.
+ */
+int ntsamd_matrix_mul_colsum(int devID, void * stream,
+                             const void * a, int transposedA, int dataTypeA,
+                             const void * b, int transposedB, int dataTypeB,
+                             void * c, int dataTypeC,
+                             int na, int ma, int nb, int mb, int nc, int mc,
+                             float alpha, float beta,
+                             void * colSum, float colSumBeta);
+
+/*
+ * out[j] = beta * out[j] + sum_i sum_k in[i][j][k] over a dense [x][y][z]
+ * tensor (z == 1: the column sums of an x by y matrix). Replaces what
+ * GradMulAndShift does for the bias gradient when it is not a by-product of
+ * the weight gradient (source/network/XBackwardMath.cpp:1793-1846):
+ * _CudaReduceSum over the last dimension into a temporary, _CudaReduceSum
+ * over the first into a second temporary, _CudaSum into the gradient
+ * (source/tensor/core/reduce/ReduceSum.cu, core/arithmetic/Sum.cu). No
+ * temporaries here. dataType is X_FLOAT or X_FLOAT16 for both tensors.
+ */
+int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType,
+                         int x, int y, int z, void * out, float beta);
+
+/*
  * `count` products over equally spaced matrices; strides are in ELEMENTS and
  * a stride of 0 shares one a or b among all products. Replaces
  *   _CudaBLASMatrixMULBatchedStrided(handle, a, transposedA, dataTypeA, strideA, ...)

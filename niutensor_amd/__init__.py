@@ -26,6 +26,8 @@ EXPORTS = (
     "ntsamd_matrix_mul_bias",
     "ntsamd_matrix_mul_batched_strided",
     "ntsamd_matrix_mul_batched",
+    "ntsamd_matrix_mul_colsum",
+    "ntsamd_reduce_sum_xz",
 )
 
 
@@ -60,6 +62,8 @@ def load():
                                                     ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_batched.argtypes = [ci, vp, C.POINTER(vp), ci, ci, C.POINTER(vp), ci, ci, C.POINTER(vp), ci,
                                             ci] + [ci] * 6 + [cf, cf]
+    L.ntsamd_matrix_mul_colsum.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, cf]
+    L.ntsamd_reduce_sum_xz.argtypes = [ci, vp, vp, ci, ci, ci, ci, vp, cf]
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
     _lib = L
@@ -140,3 +144,27 @@ def matrix_mul_batched(a_list, transA, b_list, transB, c_list, alpha=1.0, beta=0
                                      n, na, ma, nb, mb, nc, mc, alpha, beta)
     _check(rc)
     return c_list
+
+
+def matrix_mul_colsum(a, transA, b, transB, c, col_sum, alpha=1.0, beta=0.0, col_sum_beta=0.0):
+    """c = alpha * op(a) op(b) + beta * c and col_sum = col_sum_beta * col_sum + column sums of op(b)."""
+    L = load()
+    na, ma = _mat(a)
+    nb, mb = _mat(b)
+    nc, mc = _mat(c)
+    rc = L.ntsamd_matrix_mul_colsum(a.device.index, _stream_ptr(a), a.data_ptr(), transA, _dtype_code(a),
+                                    b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
+                                    na, ma, nb, mb, nc, mc, alpha, beta, col_sum.data_ptr(), col_sum_beta)
+    _check(rc)
+    return c, col_sum
+
+
+def reduce_sum_xz(t, out, beta=0.0):
+    """out[y] = beta * out[y] + sum over x and z of a dense [x][y][z] device tensor."""
+    L = load()
+    assert t.is_contiguous() and t.dim() == 3
+    x, y, z = (int(v) for v in t.shape)
+    rc = L.ntsamd_reduce_sum_xz(t.device.index, _stream_ptr(t), t.data_ptr(), _dtype_code(t), x, y, z,
+                                out.data_ptr(), beta)
+    _check(rc)
+    return out

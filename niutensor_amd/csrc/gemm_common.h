@@ -48,6 +48,14 @@ struct GemmParams {
     int tilesM, tilesN;
     int batch;
     int groupM;                            /* tile rows that share a pass over the tile columns */
+    /* column sums of op(b) in the same pass: colSum[j] = colSumBeta * colSum[j] + sum_k op(b)[k][j]
+       (NULL = none); written by the workgroups of the first tile row */
+    void * colSum;
+    float colSumBeta;
+    /* fp32 only: the k range is cut into `splits` pieces of kPerSplit (a multiple of every slab
+       depth), one workgroup each, which ADD alpha * (their partial product) to c with atomics;
+       the caller has already applied beta to c. 1 = one workgroup per tile, plain stores. */
+    int splits, kPerSplit;
 };
 
 /* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and
@@ -62,15 +70,17 @@ __device__ __forceinline__ int xcd_contiguous_id(int id, int total)
 }
 
 struct TileCoord {
-    int batch, tm, tn;
+    int batch, tm, tn, split;
 };
 
 __device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
 {
-    int total = p.tilesM * p.tilesN * p.batch;
-    int id = xcd_contiguous_id((int)blockIdx.x, total);
     int perBatch = p.tilesM * p.tilesN;
+    int perSplit = perBatch * p.batch;
+    int id = xcd_contiguous_id((int)blockIdx.x, perSplit * p.splits);
     TileCoord t;
+    t.split = id / perSplit;
+    id -= t.split * perSplit;
     t.batch = id / perBatch;
     int r = id - t.batch * perBatch;
     int perGroup = p.groupM * p.tilesN;

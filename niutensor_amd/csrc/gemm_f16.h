@@ -458,6 +458,7 @@ static int launch_f16_one(const GemmParams & p0, const PT & tab, hipStream_t str
     GemmParams p = p0;
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
+    p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
     hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, S::MINW16, AKC, BKC, VEC, PT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);

@@ -31,6 +31,7 @@
 #pragma once
 #include "gemm_common.h"
 #include "gemm_f16.h"
+#include <type_traits>
 
 namespace ntsamd {
 
@@ -75,7 +76,7 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
                  : "memory");
 }
 
-template <int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC>
+template <int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
@@ -250,6 +251,14 @@ gemm_f16_direct_kernel(const GemmParams p)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.f;
 
+    /* CS: column sums of op(b), gathered from the b fragments on their way to the MFMAs
+       (v_dot2_f32_f16 against ones: exact products, fp32 sums). Lane (l32, lh) sees, for each
+       of its columns, the k values its half of the wave feeds in; the halves meet at the end. */
+    float colSum[CS ? TJ : 1];
+#pragma unroll
+    for (int j = 0; j < (CS ? TJ : 1); j++)
+        colSum[j] = 0.f;
+
     constexpr int NM = TI * TJ;                                       /* MFMAs per k step */
     constexpr int NF = TI + TJ;                                       /* fragments per k step */
     constexpr int RPF = (AKC ? 1 : 2);                                /* LDS reads per a fragment */
@@ -268,6 +277,17 @@ gemm_f16_direct_kernel(const GemmParams p)
         for (int g = 0; g < NM; g++) {
             const int i = g / TJ, j = g % TJ;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+            if constexpr (CS) {
+                if (i == 0) {
+                    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                    const h2 ones = {(_Float16)1, (_Float16)1};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const h2 pr = {fb[kk][j][2 * e], fb[kk][j][2 * e + 1]};
+                        colSum[j] = __builtin_amdgcn_fdot2(pr, ones, colSum[j], false);
+                    }
+                }
+            }
             if (doRead) {
                 /* fragments f with f * NM / NF == g: spread evenly over the MFMAs */
 #pragma unroll
@@ -350,96 +370,148 @@ gemm_f16_direct_kernel(const GemmParams p)
        (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block. The wave's rows of c are one
        buffer that ends where c ends: rows past M drop off it, columns past N are sent
        out of range. ------------------------------------------------------------------- */
+    /* the lane number again, from the hardware rather than from threadIdx: a value that
+       would otherwise have to stay in a register (or be spilled) across the whole main loop */
+    const int laneE = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int l32E = laneE & 31, lhE = laneE >> 5;
     const float alpha = p.alpha, beta = p.beta;
     const half_t * __restrict__ bias = static_cast<const half_t *>(p.bias);
     const int biasMode = p.biasMode;
     half_t * cw = C + (size_t)(m0 + wm0) * p.ldc;
     const unsigned rowPitch = (unsigned)p.ldc * 2u;
 
-    /* Wide path (beta == 0, rows of c 16-byte aligned): a lane owns one COLUMN of each block,
-       so storing straight from the accumulators means 2-byte stores, 64 contiguous bytes per
-       row and instruction, and the store instruction count (16 per block) bounds the epilogue.
+    if constexpr (CS) {
+        /* the first tile row's first wave row has seen every k of its columns */
+        if (tc.tm == 0 && wm0 == 0) {
+            half_t * cs = static_cast<half_t *>(p.colSum);
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const float v = colSum[j] + __shfl_xor(colSum[j], 32);
+                const int col = n0 + wn0 + j * 32 + l32E;
+                if (lhE == 0 && col < N)
+                    cs[col] = (half_t)(p.colSumBeta != 0.f ? p.colSumBeta * (float)cs[col] + v : v);
+            }
+        }
+    }
+
+    /* Wide path (rows of c 16-byte aligned): a lane owns one COLUMN of each block, so storing
+       straight from the accumulators means 2-byte stores, 64 contiguous bytes per row and
+       instruction, and the store instruction count (16 per block) bounds the epilogue.
        Instead each wave turns 32 rows at a time through its own piece of LDS (the stages are
-       free by now) and writes 16 bytes per lane: whole rows of the wave's tile, whole cache
-       lines, an eighth of the instructions. */
-    const bool wide = beta == 0.f && (p.ldc & 7) == 0 && (N & 7) == 0 && (reinterpret_cast<size_t>(C) & 15) == 0;
+       free by now) and moves 16 bytes per lane: whole rows of the wave's tile, whole cache
+       lines, an eighth of the instructions. With beta == 0 the values cross LDS as halves;
+       with beta != 0 they cross as fp32 and meet the old c (one 16-byte load per lane) on the
+       far side, so the result is still rounded once. */
+    const bool wide = (p.ldc & 7) == 0 && (N & 7) == 0 && (reinterpret_cast<size_t>(C) & 15) == 0;
     if (wide) {
-        constexpr int PITCH = TJ * 64 + 16;          /* bytes; 4 rows apart = 64 bytes apart modulo 128 */
         constexpr int LPR = TJ * 4;                  /* lanes that cover one row of the wave's tile */
         constexpr int RPI = 64 / LPR;                /* rows per 16-byte store instruction */
-        constexpr int GROUP = 32 * PITCH;
-        static_assert(2 * GROUP * NW <= NSTAGE * STAGE, "epilogue staging must fit the stages");
         __syncthreads();                             /* every wave has read its last fragments */
         if (m0 + wm0 >= M)
             return;
-        char * mine = lds + wave * 2 * GROUP;
         __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
         float bcol[TJ];
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const int col = n0 + wn0 + j * 32 + l32;
+            const int col = n0 + wn0 + j * 32 + l32E;
             bcol[j] = biasMode == BIAS_COL && col < N ? (float)bias[col] : 0.f;
         }
-        const int rdRow = lane / LPR, rdChunk = lane % LPR;
+        const int rdRow = laneE / LPR, rdChunk = laneE % LPR;
         const int colW = n0 + wn0 + rdChunk * 8;
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+
+        auto turn = [&](auto BETAC) {
+            constexpr bool useOld = decltype(BETAC)::value != 0;
+            typedef typename std::conditional<useOld, float, half_t>::type StageT;
+            /* row pitch: the two half-waves write rows 4 apart; keep them in different banks */
+            constexpr int PITCH = TJ * 32 * (int)sizeof(StageT) + (useOld ? 32 : 16);
+            constexpr int GROUP = 32 * PITCH;
+            constexpr int NBUF = useOld ? 1 : 2;
+            static_assert(NBUF * GROUP * NW <= NSTAGE * STAGE, "epilogue staging must fit the stages");
+            char * mine = lds + wave * NBUF * GROUP;
 #pragma unroll
-        for (int i = 0; i < TI; i++) {
-            char * buf = mine + (i & 1) * GROUP;
+            for (int i = 0; i < TI; i++) {
+                char * buf = mine + (i % NBUF) * GROUP;
+                f32x4 old[32 / RPI];
+                if constexpr (useOld) {
 #pragma unroll
-            for (int j = 0; j < TJ; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = 8 * (r / 4) + 4 * lh + (r % 4);
-                    *reinterpret_cast<half_t *>(buf + row * PITCH + (j * 32 + l32) * 2) = (half_t)(alpha * acc[i][j][r] + bcol[j]);
+                    for (int q = 0; q < 32 / RPI; q++)
+                        old[q] = buffer_load_f32x4(cr, (int)(cOffW + (unsigned)(i * 32 + q * RPI) * rowPitch));
                 }
-            /* the wave's own lanes exchange data through LDS: LDS executes one wave's
-               instructions in order, the fences only keep the compiler from reordering */
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int q = 0; q < 32 / RPI; q++) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(buf + (q * RPI + rdRow) * PITCH + rdChunk * 16);
-                const unsigned off = cOffW + (unsigned)(i * 32 + q * RPI) * rowPitch;
-                __builtin_amdgcn_raw_buffer_store_b128(v, cr, (int)off, 0, 0);
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int row = 8 * (r / 4) + 4 * lhE + (r % 4);
+                        *reinterpret_cast<StageT *>(buf + row * PITCH + (j * 32 + l32E) * (int)sizeof(StageT)) =
+                            (StageT)(alpha * acc[i][j][r] + bcol[j]);
+                    }
+                /* the wave's own lanes exchange data through LDS: LDS executes one wave's
+                   instructions in order, the fences only keep the compiler from reordering */
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int q = 0; q < 32 / RPI; q++) {
+                    const char * src = buf + (q * RPI + rdRow) * PITCH + rdChunk * 8 * (int)sizeof(StageT);
+                    const unsigned off = cOffW + (unsigned)(i * 32 + q * RPI) * rowPitch;
+                    if constexpr (useOld) {
+                        const f32x4 lo = *reinterpret_cast<const f32x4 *>(src);
+                        const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + 16);
+                        const f16x8 o = __builtin_bit_cast(f16x8, old[q]);
+                        f16x8 v;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            v[e] = (half_t)(lo[e] + beta * (float)o[e]);
+                            v[4 + e] = (half_t)(hi[e] + beta * (float)o[4 + e]);
+                        }
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(f32x4, v), cr, (int)off, 0, 0);
+                    }
+                    else {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(src);
+                        __builtin_amdgcn_raw_buffer_store_b128(v, cr, (int)off, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-        }
+        };
+        if (beta != 0.f)
+            turn(IntC<1>());
+        else
+            turn(IntC<0>());
         return;
     }
 
+    /* Narrow path: 2-byte stores straight from the accumulators, any alignment of c. beta is
+       tested outside the loops: inside them every load of c would sit in a block of its own,
+       one memory round trip after the other. */
     if (m0 + wm0 >= M)
         return;
     __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
-    /* beta is tested outside the loops: inside them every load of c would sit in a block of
-       its own, one memory round trip after the other */
     auto narrow = [&](auto BETAC) {
         constexpr bool useOld = decltype(BETAC)::value != 0;
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const int col = n0 + wn0 + j * 32 + l32;
-            const unsigned cOff = col < N ? (unsigned)(4 * lh * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+            const int col = n0 + wn0 + j * 32 + l32E;
+            const unsigned cOff = col < N ? (unsigned)(4 * lhE * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
             float bcol = 0.f;
             if (biasMode == BIAS_COL && col < N)
                 bcol = (float)bias[col];
-            float old[TI][16];
-            if constexpr (useOld) {
-#pragma unroll
-                for (int i = 0; i < TI; i++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        old[i][r] = buffer_load_out<half_t>(cr, (int)(cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch));
-            }
 #pragma unroll
             for (int i = 0; i < TI; i++) {
+                float old[16];
+                if constexpr (useOld) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        old[r] = buffer_load_out<half_t>(cr, (int)(cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch));
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const unsigned off = cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
                     float v = alpha * acc[i][j][r] + bcol;
                     if constexpr (useOld)
-                        v += beta * (float)old[i][r];
+                        v += beta * old[r];
                     buffer_store_out<half_t>((half_t)v, cr, (int)off);
                 }
             }
@@ -451,15 +523,16 @@ gemm_f16_direct_kernel(const GemmParams p)
         narrow(IntC<0>());
 }
 
-template <int CFG, bool AKC, bool BKC>
+template <int CFG, bool AKC, bool BKC, bool CS>
 static int launch_f16_direct(const GemmParams & p0, hipStream_t stream)
 {
     typedef TileShape<CFG> S;
     GemmParams p = p0;
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
+    p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC>),
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -479,11 +552,18 @@ static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
         return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
     if (!vec)
         return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
+    /* column sums: the 256x256 tile has no registers to spare, and products that want column
+       sums (weight gradients) are too small for it anyway */
+    if (p.colSum != NULL) {
+        if (cfg == CFG_64x64)
+            return launch_f16_direct<CFG_64x64, AKC, BKC, true>(p, stream);
+        return launch_f16_direct<CFG_128x128, AKC, BKC, true>(p, stream);
+    }
     if (cfg == CFG_256x256)
-        return launch_f16_direct<CFG_256x256, AKC, BKC>(p, stream);
+        return launch_f16_direct<CFG_256x256, AKC, BKC, false>(p, stream);
     if (cfg == CFG_128x128)
-        return launch_f16_direct<CFG_128x128, AKC, BKC>(p, stream);
-    return launch_f16_direct<CFG_64x64, AKC, BKC>(p, stream);
+        return launch_f16_direct<CFG_128x128, AKC, BKC, false>(p, stream);
+    return launch_f16_direct<CFG_64x64, AKC, BKC, false>(p, stream);
 }
 
 }  // namespace ntsamd

@@ -59,7 +59,7 @@ __device__ __forceinline__ f32x4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t rsrc, 
     return __builtin_bit_cast(f32x4, v);
 }
 
-template <int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, typename PT>
+template <int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, bool CS, typename PT>
 __global__ void __launch_bounds__(WGM * WGN * 64, 2)
 gemm_f32_kernel(const GemmParams p, const PT tab)
 {
@@ -289,6 +289,14 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.f;
 
+    /* CS: every lane also adds up the op(b) values that pass through its fragments: lane
+       (l32, lh) of a wave sees, for each of its columns, every k of the slab that its half
+       of the wave feeds to the MFMAs; the two halves are added at the end */
+    float colSum[CS ? TJ : 1];
+#pragma unroll
+    for (int j = 0; j < (CS ? TJ : 1); j++)
+        colSum[j] = 0.f;
+
     auto mfma_steps = [&](auto SET, int first, int last) {
         constexpr int set = decltype(SET)::value;
 #pragma unroll
@@ -300,10 +308,16 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                     float av = AKC ? fa4[set][t / 4][i][t % 4] : fa1[set][t][i];
                     float bv = BKC ? fb4[set][t / 4][j][t % 4] : fb1[set][t][j];
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                    if constexpr (CS)
+                        if (i == 0)
+                            colSum[j] += bv;
                 }
     };
 
-    const int nk = (K + BKT - 1) / BKT;
+    /* this workgroup's k range: all of K, or one of p.splits pieces */
+    const int kBeg = tc.split * p.kPerSplit;
+    const int kLen = (p.splits > 1 && kBeg + p.kPerSplit < K ? p.kPerSplit : K - kBeg);
+    const int nk = (kLen + BKT - 1) / BKT;
 
     /* One slab: fragments of slab kt are in register set SET and came from LDS stage SET.
        FULL: slabs kt+1 and kt+2 exist and are complete, so nothing is conditional and the
@@ -314,9 +328,9 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         if (full || kt + 1 < nk)
             store_lds(set ^ 1);                  /* slab kt+1, fetched during slab kt-1 */
         if (full)
-            load_global(IntC<0>(), (kt + 2) * BKT);
+            load_global(IntC<0>(), kBeg + (kt + 2) * BKT);
         else if (kt + 2 < nk)
-            load_global(IntC<1>(), (kt + 2) * BKT);
+            load_global(IntC<1>(), kBeg + (kt + 2) * BKT);
         mfma_steps(SET, 0, KK / 2);
         if constexpr (full) {
             /* An MFMA keeps the matrix pipe busy for 64 cycles but takes one issue slot:
@@ -351,13 +365,13 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     };
 
     if (nk > 0) {
-        load_global(IntC<1>(), 0);
+        load_global(IntC<1>(), kBeg);
         store_lds(0);
         if (nk > 1)
-            load_global(IntC<1>(), BKT);
+            load_global(IntC<1>(), kBeg + BKT);
         __syncthreads();
         read_frags(IntC<0>(), 0);
-        const int nkFull = K / BKT;              /* slabs that lie entirely inside K */
+        const int nkFull = kLen / BKT;           /* slabs that lie entirely inside the k range */
         int kt = 0;
         for (; kt + 3 < nkFull; kt += 2) {
             slab(IntC<0>(), IntC<1>(), kt);
@@ -393,6 +407,38 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             const int col = n0 + wn0 + j * 32 + l32;
             cOff[j] = col < N ? (unsigned)(4 * lh * p.ldc + col) * 4u : (unsigned)NTSAMD_OOB_OFFSET;
             bcol[j] = biasMode == BIAS_COL && col < N ? bias[col] : 0.f;
+        }
+        if constexpr (CS) {
+            /* the first tile row's first wave row has seen every k of its columns */
+            if (tc.tm == 0 && wm0 == 0) {
+                float * cs = static_cast<float *>(p.colSum);
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    const float v = colSum[j] + __shfl_xor(colSum[j], 32);
+                    const int col = n0 + wn0 + j * 32 + l32;
+                    if (lh == 0 && col < N) {
+                        if (p.splits > 1)
+                            unsafeAtomicAdd(cs + col, v);      /* the caller has applied colSumBeta */
+                        else
+                            cs[col] = p.colSumBeta != 0.f ? p.colSumBeta * cs[col] + v : v;
+                    }
+                }
+            }
+        }
+        if (p.splits > 1) {
+            /* one of several workgroups that share this tile: add the partial product to c,
+               which already holds beta * c; the bias rides on the first piece */
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                        const float v = alpha * acc[i][j][r] + (tc.split == 0 ? bcol[j] : 0.f);
+                        (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, cr, (int)off, 0, 0);
+                    }
+            return;
         }
         /* beta is tested once, outside the loops: inside them the test would fence every
            load of c off in a block of its own, one memory round trip after the other */
@@ -465,15 +511,17 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     }
 }
 
-template <int CFG, bool AKC, bool BKC, bool VEC, typename PT>
+template <int CFG, bool AKC, bool BKC, bool VEC, bool CS, typename PT>
 static int launch_f32_one(const GemmParams & p0, const PT & tab, hipStream_t stream)
 {
     typedef TileShape<CFG> S;
     GemmParams p = p0;
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
-    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, S::BKT32, S::WGM, S::WGN, AKC, BKC, VEC, PT>),
+    if (p.splits < 1 || !VEC)
+        p.splits = 1;
+    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
+    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, S::BKT32, S::WGM, S::WGN, AKC, BKC, VEC, CS, PT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();
 }
@@ -484,13 +532,19 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
     NoPtrs none = {0};
     if (ptrs) {
         /* pointer lists are the rare path: one instantiation, element-wise loads */
-        return launch_f32_one<CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
+        return launch_f32_one<CFG_64x64, AKC, BKC, false, false, PtrBatch>(p, *ptrs, stream);
     }
     if (!vec)
-        return launch_f32_one<CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
+        return launch_f32_one<CFG_64x64, AKC, BKC, false, false, NoPtrs>(p, none, stream);
+    /* column sums and split k ranges exist on the 16-byte path only; the caller checks that */
+    if (p.colSum != NULL) {
+        if (cfg == CFG_128x128)
+            return launch_f32_one<CFG_128x128, AKC, BKC, true, true, NoPtrs>(p, none, stream);
+        return launch_f32_one<CFG_64x64, AKC, BKC, true, true, NoPtrs>(p, none, stream);
+    }
     if (cfg == CFG_128x128)
-        return launch_f32_one<CFG_128x128, AKC, BKC, true, NoPtrs>(p, none, stream);
-    return launch_f32_one<CFG_64x64, AKC, BKC, true, NoPtrs>(p, none, stream);
+        return launch_f32_one<CFG_128x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
+    return launch_f32_one<CFG_64x64, AKC, BKC, true, false, NoPtrs>(p, none, stream);
 }
 
 }  // namespace ntsamd

@@ -22,6 +22,8 @@ int launch_f16_nn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStre
 int launch_f16_nt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
 int launch_f16_tn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
 int launch_f16_tt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
+int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
+int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -137,40 +139,67 @@ bool aligned16(const void * p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
-/* Relative run time of a product under a tile shape: rounds of workgroups (256 CUs x the
-   workgroups a CU holds at once) times the work of one tile, divided by how fast the shape
-   runs relative to the best one on a product that fits it (measured: small tiles re-read
-   operands from LDS more often per MFMA, which costs fp16 far more than fp32). */
-double tile_cost(int M, int N, int count, int bm, int bn, int perCU, double quality)
+/* Relative run time of a product under a tile shape and a number of k pieces: rounds of
+   workgroups (256 CUs x the workgroups a CU holds at once) times the work of one workgroup
+   (tile area x its k range plus a fixed cost per workgroup, in units of k: fetching the first
+   slabs, storing the tile), divided by how fast the shape runs relative to the best one on a
+   product that fits it (measured: small tiles re-read operands from LDS more often per MFMA,
+   which costs fp16 far more than fp32). */
+double tile_cost(int M, int N, int K, int count, int bm, int bn, int perCU, double quality, int splits)
 {
-    long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count;
+    long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
     long long slots = 256LL * perCU;
     long long rounds = (tiles + slots - 1) / slots;
-    return (double)rounds * bm * bn / quality;
+    double kFixed = splits > 1 ? 192.0 : 96.0;       /* atomics cost more than stores */
+    return (double)rounds * bm * bn * ((double)((K + splits - 1) / splits) + kFixed) / quality;
 }
 
-/* NTSAMD_TILE_CFG=0|1|2 forces a tile shape (128x128, 64x64, 256x256 for half; for
-   measurements); otherwise the shape with the lowest estimated run time */
-int choose_cfg(int M, int N, int count, bool half)
+struct Plan {
+    int cfg;
+    int splits;
+};
+
+/* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
+   estimated run time. NTSAMD_TILE_CFG=0|1|2 forces a shape (128x128, 64x64, 256x256 for
+   half) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
+Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit)
 {
+    static const int bms[CFG_COUNT] = {128, 64, 256};
+    static const int perCU[CFG_COUNT] = {2, 2, 1};
+    static const double q32[CFG_COUNT] = {1.0, 0.8, 0.0};
+    static const double q16[CFG_COUNT] = {0.45, 0.2, 1.0};
+    int forcedCfg = -1, forcedSplits = -1;
     const char * e = getenv("NTSAMD_TILE_CFG");
     if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
-        int cfg = e[0] - '0';
-        if (cfg == CFG_256x256 && !half)
-            cfg = CFG_128x128;
-        return cfg;
+        forcedCfg = e[0] - '0';
+        if (forcedCfg == CFG_256x256 && !half)
+            forcedCfg = CFG_128x128;
     }
-    int best = CFG_64x64;
-    double bestCost = tile_cost(M, N, count, 64, 64, 2, half ? 0.2 : 0.8);
-    double c128 = tile_cost(M, N, count, 128, 128, 2, half ? 0.45 : 1.0);
-    if (c128 <= bestCost) {
-        best = CFG_128x128;
-        bestCost = c128;
-    }
-    if (half) {
-        double c256 = tile_cost(M, N, count, 256, 256, 1, 1.0);
-        if (c256 <= bestCost)
-            best = CFG_256x256;
+    e = getenv("NTSAMD_SPLIT_K");
+    if (e && atoi(e) >= 1)
+        forcedSplits = atoi(e);
+    if (forcedSplits != 1 && forcedSplits != 2 && forcedSplits != 4 && forcedSplits != 8 && forcedSplits != 16)
+        forcedSplits = -1;
+    if (forcedSplits > 1 && (!maySplit || K / forcedSplits < 256))
+        forcedSplits = 1;
+    Plan best = {CFG_64x64, 1};
+    double bestCost = -1.0;
+    for (int cfg = 0; cfg < CFG_COUNT; cfg++) {
+        const double q = half ? q16[cfg] : q32[cfg];
+        if (q <= 0.0 || (forcedCfg >= 0 && cfg != forcedCfg))
+            continue;
+        for (int splits = 1; splits <= 16; splits *= 2) {
+            if (splits > 1 && (!maySplit || K / splits < 256))
+                break;
+            if (forcedSplits >= 1 && splits != forcedSplits)
+                continue;
+            double c = tile_cost(M, N, K, count, bms[cfg], bms[cfg], perCU[cfg], q, splits);
+            if (bestCost < 0.0 || c < bestCost) {
+                bestCost = c;
+                best.cfg = cfg;
+                best.splits = splits;
+            }
+        }
     }
     return best;
 }
@@ -181,7 +210,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         long long strideA, long long strideB, long long strideC, int count,
         const PtrBatch * ptrs,
         float alpha, float beta,
-        const void * bias, int biasMode, int biasLen, int biasRowDiv)
+        const void * bias, int biasMode, int biasLen, int biasRowDiv,
+        void * colSum = NULL, float colSumBeta = 0.f)
 {
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
@@ -225,10 +255,48 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                strideA % vecElems == 0 && strideB % vecElems == 0 &&
                lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) &&
                biasMode != NTSAMD_BIAS_ROW;
-    int cfg = choose_cfg(s.M, s.N, count, kind != KIND_F32);
     hipStream_t hs = static_cast<hipStream_t>(stream);
+    const bool half = kind != KIND_F32;
+    /* cutting k into pieces pays when the result has few tiles and k is long (weight
+       gradients); the pieces add to c with fp32 atomics, so c gets its beta first.
+       SWITCHED OFF: a product cut this way ended in a GPU memory fault whose cause has not
+       been found yet, so every product runs as one piece per tile until it has. */
+    const bool splitKEnabled = false;
+    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, splitKEnabled && kind == KIND_F32 && vec);
+    const int cfg = plan.cfg;
+    int rc = 0;
+    p.splits = 1;
+    if (plan.splits > 1) {
+        p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 31) / 32 * 32;
+        p.splits = (s.K + p.kPerSplit - 1) / p.kPerSplit;
+    }
+    if (p.splits > 1 && beta != 1.f) {
+        /* c is dense: count matrices of M x N, strideC apart */
+        if (count == 1 || strideC == (long long)s.M * s.N)
+            rc = launch_scale(false, c, (long long)s.M * s.N * count, beta, hs);
+        else
+            for (int i = 0; i < count && rc == 0; i++)
+                rc = launch_scale(false, static_cast<float *>(c) + i * strideC, (long long)s.M * s.N, beta, hs);
+        if (rc != 0)
+            return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    }
+    if (colSum != NULL) {
+        if (vec && count == 1) {
+            /* by-product of the product kernel */
+            p.colSum = colSum;
+            p.colSumBeta = colSumBeta;
+            if (p.splits > 1)
+                rc = launch_scale(false, colSum, s.N, colSumBeta, hs);
+        }
+        else {
+            /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS */
+            rc = s.bKContig ? launch_reduce_sum_xz(half, b, 1, s.N, s.K, colSum, colSumBeta, hs)
+                            : launch_reduce_sum_xz(half, b, s.K, s.N, 1, colSum, colSumBeta, hs);
+        }
+        if (rc != 0)
+            return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    }
 
-    int rc;
     if (kind == KIND_F32) {
         if (s.aKContig)
             rc = s.bKContig ? launch_f32_nt(p, ptrs, vec, cfg, hs) : launch_f32_nn(p, ptrs, vec, cfg, hs);
@@ -311,6 +379,74 @@ int ntsamd_matrix_mul_bias(int devID, void * stream,
     }
     return run(devID, stream, kind, s, a, b, c, ma, mb, mc, 0, 0, 0, 1, NULL, alpha, beta,
                biasMode == NTSAMD_BIAS_NONE ? NULL : bias, biasMode, biasLen, biasRowDiv);
+}
+
+int ntsamd_matrix_mul_colsum(int devID, void * stream,
+                             const void * a, int transposedA, int dataTypeA,
+                             const void * b, int transposedB, int dataTypeB,
+                             void * c, int dataTypeC,
+                             int na, int ma, int nb, int mb, int nc, int mc,
+                             float alpha, float beta,
+                             void * colSum, float colSumBeta)
+{
+    Kind kind;
+    Shape s;
+    int st = check_types(dataTypeA, dataTypeB, dataTypeC, kind);
+    if (st == NTSAMD_OK)
+        st = check_shape(transposedA, transposedB, na, ma, nb, mb, nc, mc, s);
+    if (st != NTSAMD_OK)
+        return st;
+    if (kind == KIND_F16_F32OUT)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");   /* the sums have the type of b and of c */
+    if (s.N == 0)
+        return NTSAMD_OK;
+    if (!colSum)
+        return fail(NTSAMD_ERR_ARGUMENT, "column sums requested but empty");
+    if (!b || (s.M > 0 && (!a || !c)))
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty matrices in multiplication!");
+    if (s.M == 0) {
+        /* no product to ride on: only the sums */
+        st = check_device(devID);
+        if (st != NTSAMD_OK)
+            return st;
+        DeviceScope scope(devID);
+        if (scope.status != NTSAMD_OK)
+            return scope.status;
+        hipStream_t hs = static_cast<hipStream_t>(stream);
+        int rc = s.bKContig ? launch_reduce_sum_xz(kind != KIND_F32, b, 1, s.N, s.K, colSum, colSumBeta, hs)
+                            : launch_reduce_sum_xz(kind != KIND_F32, b, s.K, s.N, 1, colSum, colSumBeta, hs);
+        if (rc != 0)
+            return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+        return NTSAMD_OK;
+    }
+    return run(devID, stream, kind, s, a, b, c, ma, mb, mc, 0, 0, 0, 1, NULL, alpha, beta,
+               NULL, NTSAMD_BIAS_NONE, 0, 1, colSum, colSumBeta);
+}
+
+int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType,
+                         int x, int y, int z, void * out, float beta)
+{
+    if (dataType != NTSAMD_X_FLOAT && dataType != NTSAMD_X_FLOAT16)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
+    if (x < 0 || y < 0 || z < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
+    if (y == 0)
+        return NTSAMD_OK;
+    if (!out || (!in && x > 0 && z > 0))
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty input or output tensors!");
+    if ((long long)x * y * z > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
+    int st = check_device(devID);
+    if (st != NTSAMD_OK)
+        return st;
+    DeviceScope scope(devID);
+    if (scope.status != NTSAMD_OK)
+        return scope.status;
+    int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,
+                                  static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return NTSAMD_OK;
 }
 
 int ntsamd_matrix_mul(int devID, void * stream,

@@ -1,0 +1,152 @@
+/*
+ * Sums over the outer and inner dimensions of a dense [X][Y][Z] tensor:
+ *     out[y] = beta * out[y] + sum_x sum_z in[x][y][z]
+ * which is what the bias gradient of MulAndShift needs
+ * (source/network/XBackwardMath.cpp:1793-1846: _ReduceSum over the last
+ * dimension, _ReduceSum over the first, _Sum into the gradient). With Z == 1
+ * it is the column sum of an [X][Y] matrix. The matrix-multiplication kernels
+ * produce the same column sums as a by-product when they can; these kernels
+ * serve the shapes and layouts where they cannot. Also here: the scaling pass
+ * that applies beta ahead of kernels that add to their result with atomics.
+ * Memory-bound, fp32 accumulation for both data types.
+ */
+#include "gemm_common.h"
+#include "gemm_f16.h"       /* half_t */
+
+namespace ntsamd {
+
+/* Z == 1. A workgroup owns 64 columns and one piece of the rows: 16 threads side by side
+   read 4 columns each (256 contiguous bytes of a row for fp32), 16 such rows per step. */
+template <typename T, bool ATOMIC>
+__global__ void __launch_bounds__(256)
+column_sum_kernel(const T * __restrict__ in, int X, int Y, int rowsPerPiece, T * __restrict__ out, float beta)
+{
+    __shared__ float part[16][64];
+    const int cg = threadIdx.x & 15, rl = threadIdx.x >> 4;
+    const int col0 = blockIdx.x * 64 + cg * 4;
+    const int xBeg = blockIdx.y * rowsPerPiece;
+    const int xEnd = xBeg + rowsPerPiece < X ? xBeg + rowsPerPiece : X;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (col0 + 3 < Y) {
+#pragma unroll 4
+        for (int x = xBeg + rl; x < xEnd; x += 16) {
+            const T * rp = in + (size_t)x * Y + col0;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                s[e] += (float)rp[e];
+        }
+    }
+    else {
+        for (int x = xBeg + rl; x < xEnd; x += 16) {
+            const T * rp = in + (size_t)x * Y + col0;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (col0 + e < Y)
+                    s[e] += (float)rp[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        part[rl][cg * 4 + e] = s[e];
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float v = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            v += part[r][threadIdx.x];
+        const int col = blockIdx.x * 64 + threadIdx.x;
+        if (col < Y) {
+            if constexpr (ATOMIC)
+                unsafeAtomicAdd(reinterpret_cast<float *>(out) + col, v);     /* beta already applied */
+            else
+                out[col] = (T)(beta != 0.f ? beta * (float)out[col] + v : v);
+        }
+    }
+}
+
+/* any Z: one workgroup per y, its threads stride over the (x, z) pairs */
+template <typename T>
+__global__ void __launch_bounds__(256)
+outer_inner_sum_kernel(const T * __restrict__ in, int X, int Y, int Z, T * __restrict__ out, float beta)
+{
+    __shared__ float part[256];
+    const int y = blockIdx.x;
+    const long long total = (long long)X * Z;
+    float s = 0.f;
+    for (long long e = threadIdx.x; e < total; e += 256) {
+        const long long x = e / Z, z = e - x * Z;
+        s += (float)in[(x * Y + y) * Z + z];
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w)
+            part[threadIdx.x] += part[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0)
+        out[y] = (T)(beta != 0.f ? beta * (float)out[y] + part[0] : part[0]);
+}
+
+/* v[i] = beta * v[i] (beta == 0 stores zeros whatever v held) */
+template <typename T>
+__global__ void __launch_bounds__(256)
+scale_kernel(T * __restrict__ v, long long n, float beta)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n)
+        v[i] = (T)(beta != 0.f ? beta * (float)v[i] : 0.f);
+}
+
+int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream)
+{
+    if (n <= 0 || beta == 1.f)
+        return 0;
+    dim3 grid((unsigned)((n + 255) / 256));
+    if (half)
+        hipLaunchKernelGGL(scale_kernel<half_t>, grid, dim3(256), 0, stream, static_cast<half_t *>(v), n, beta);
+    else
+        hipLaunchKernelGGL(scale_kernel<float>, grid, dim3(256), 0, stream, static_cast<float *>(v), n, beta);
+    return (int)hipGetLastError();
+}
+
+int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream)
+{
+    if (Y <= 0)
+        return 0;
+    if (Z != 1) {
+        if (half)
+            hipLaunchKernelGGL(outer_inner_sum_kernel<half_t>, dim3((unsigned)Y), dim3(256), 0, stream,
+                               static_cast<const half_t *>(in), X, Y, Z, static_cast<half_t *>(out), beta);
+        else
+            hipLaunchKernelGGL(outer_inner_sum_kernel<float>, dim3((unsigned)Y), dim3(256), 0, stream,
+                               static_cast<const float *>(in), X, Y, Z, static_cast<float *>(out), beta);
+        return (int)hipGetLastError();
+    }
+    const int colGroups = (Y + 63) / 64;
+    if (half) {
+        /* one piece: half sums are rounded once, from the fp32 total */
+        hipLaunchKernelGGL((column_sum_kernel<half_t, false>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
+                           static_cast<const half_t *>(in), X, Y, X > 0 ? X : 1, static_cast<half_t *>(out), beta);
+        return (int)hipGetLastError();
+    }
+    /* enough pieces to give every CU a few workgroups, at least 64 rows each */
+    int pieces = (1024 + colGroups - 1) / colGroups;
+    if (pieces > (X + 63) / 64)
+        pieces = (X + 63) / 64;
+    if (pieces <= 1) {
+        hipLaunchKernelGGL((column_sum_kernel<float, false>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
+                           static_cast<const float *>(in), X, Y, X > 0 ? X : 1, static_cast<float *>(out), beta);
+        return (int)hipGetLastError();
+    }
+    int rc = launch_scale(false, out, Y, beta, stream);
+    if (rc != 0)
+        return rc;
+    const int rowsPerPiece = (X + pieces - 1) / pieces;
+    pieces = (X + rowsPerPiece - 1) / rowsPerPiece;
+    hipLaunchKernelGGL((column_sum_kernel<float, true>), dim3((unsigned)colGroups, (unsigned)pieces), dim3(256), 0, stream,
+                       static_cast<const float *>(in), X, Y, rowsPerPiece, static_cast<float *>(out), 1.f);
+    return (int)hipGetLastError();
+}
+
+}  // namespace ntsamd

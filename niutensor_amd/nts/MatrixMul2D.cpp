@@ -71,6 +71,32 @@ void _AmdMatrixMul2DBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const
     }
 }
 
+void _AmdMatrixMul2DColSum(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
+                           XTensor * c, DTYPE alpha, DTYPE beta, XTensor * colSum, DTYPE colSumBeta)
+{
+    CheckNTErrors((a && b && c && colSum), "Empty matrices in multiplication!");
+    CheckNTErrors((a->order == 2 && b->order == 2 && c->order == 2), "Input tensors must have a order = 2!");
+
+    int an = transposedA == X_TRANS ? a->dimSize[1] : a->dimSize[0];
+    int am = transposedA == X_TRANS ? a->dimSize[0] : a->dimSize[1];
+    int bn = transposedB == X_TRANS ? b->dimSize[1] : b->dimSize[0];
+    int bm = transposedB == X_TRANS ? b->dimSize[0] : b->dimSize[1];
+
+    CheckNTErrors((am == bn && an == c->dimSize[0] && bm == c->dimSize[1]), "Unmatched matrices in multiplication!");
+    CheckNTErrors((colSum->unitNum == bm), "Wrong tensor size!");
+    CheckNTErrors((a->devID >= 0), "Cuda version matrix mutiplication must be run on GPUs.");
+    CheckNTErrors(a->devID == b->devID && a->devID == c->devID && a->devID == colSum->devID,
+                  "Matrices used in multiplication are not on the same GPU.");
+    CheckNTErrors((a->dataType == b->dataType && a->dataType == c->dataType && a->dataType == colSum->dataType),
+                  "Input tensors should have the same data type!");
+    CheckNTErrors((a->dataType == X_FLOAT || a->dataType == X_FLOAT16), "TODO!");
+
+    _AmdMatrixMULColSum(a->devID, a->data, transposedA, a->dataType, b->data, transposedB, b->dataType,
+                        c->data, c->dataType,
+                        a->dimSize[0], a->dimSize[1], b->dimSize[0], b->dimSize[1], c->dimSize[0], c->dimSize[1],
+                        alpha, beta, colSum->data, colSumBeta);
+}
+
 void _AmdMatrixMul2D(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
                      XTensor * c, DTYPE alpha, DTYPE beta)
 {

@@ -25,5 +25,10 @@ struct BiasSpec {
 void _AmdMatrixMul2DBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
                          XTensor * c, DTYPE alpha, DTYPE beta, const BiasSpec * bias);
 
+/* _AmdMatrixMul2D that also adds the column sums of op(b) to colSum (an order-1 tensor,
+   or any tensor with as many elements as c has columns): colSum = colSum * colSumBeta + sums */
+void _AmdMatrixMul2DColSum(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
+                           XTensor * c, DTYPE alpha, DTYPE beta, XTensor * colSum, DTYPE colSumBeta);
+
 }  // namespace nts
 #endif

@@ -145,6 +145,23 @@ void XLink::AddParamToHeadTrans(XTensor * h, MATRIX_TRANS_TYPE param)
     AddParamToHeadInt(h, (int)param);
 }
 
+DTYPE XLink::GetParam(int i) const
+{
+    CheckNTErrors(i >= 0 && i < paramNum, "parameter array cannot be empty!");
+    return params[i].f;
+}
+
+int XLink::GetParamInt(int i) const
+{
+    CheckNTErrors(i >= 0 && i < paramNum, "parameter array cannot be empty!");
+    return params[i].i;
+}
+
+MATRIX_TRANS_TYPE XLink::GetParamTrans(int i) const
+{
+    return (MATRIX_TRANS_TYPE)GetParamInt(i);
+}
+
 /* ---- XTensor -------------------------------------------------------------- */
 
 void XTensor::Init()
@@ -164,6 +181,8 @@ void XTensor::Init()
     isInit = false;
     isTmp = false;
     enableGrad = false;
+    grad = NULL;
+    isGrad = false;
     income.Reset();
 }
 
@@ -241,6 +260,8 @@ XTensor & XTensor::operator=(const XTensor & reference)
 XTensor::~XTensor()
 {
     DestroyData();
+    if (grad != NULL)
+        delete grad;
 }
 
 void XTensor::DestroyData()
@@ -332,6 +353,25 @@ int XTensor::GetDim(int dim) const
     return dimSize[d];
 }
 
+void XTensor::Reshape(const int myOrder, const int * myDimSize)
+{
+    CheckNTErrors(myOrder >= 0 && myOrder <= MAX_TENSOR_DIM_NUM, "Illegal tensor order!");
+    int num = 1;
+    for (int i = 0; i < myOrder; i++)
+        num *= myDimSize[i];
+    CheckNTErrors(abs(num) == unitNum, "Wrong size for reshape!");
+    order = myOrder;
+    memset(dimSize, 0, sizeof(dimSize));
+    for (int i = 0; i < myOrder; i++)
+        dimSize[i] = abs(myDimSize[i]);
+}
+
+void XTensor::Reshape(const int rowNum, const int colNum)
+{
+    int dims[2] = {rowNum, colNum};
+    Reshape(2, dims);
+}
+
 /* ---- creation helpers ----------------------------------------------------- */
 
 void InitTensorV2(XTensor * tensor, const int myOrder, const int * myDimSize,
@@ -372,6 +412,16 @@ XTensor * NewTensorBufV2(const int myOrder, const int * myDimSize, const TENSOR_
                          const float myDenseRatio, const int myDevID, XMem * myMem)
 {
     return NewTensorV2(myOrder, myDimSize, myDataType, myDenseRatio, myDevID, myMem);
+}
+
+XTensor * NewTensor(const XTensor * a, bool isFilledData)
+{
+    CheckNTErrors(a != NULL, "Empty input!");
+    int dims[MAX_TENSOR_DIM_NUM];
+    memcpy(dims, a->dimSize, sizeof(int) * MAX_TENSOR_DIM_NUM);
+    if (!isFilledData && a->order > 0)
+        dims[0] = -dims[0];
+    return new XTensor(a->order, dims, a->dataType, a->denseRatio, a->devID, a->mem);
 }
 
 void DelTensorBuf(XTensor * tensor)

@@ -3,8 +3,8 @@
  *
  * It keeps the names and meaning of the fields the path reads in the reference
  * (source/tensor/XTensor.h:62-200): data, devID, order, dimSize, dataType,
- * unitSize, unitNum, isSparse, denseRatio, mem, isInit, isTmp, enableGrad and
- * the `income` edge used by autograd. It is not a re-implementation of the
+ * unitSize, unitNum, isSparse, denseRatio, mem, isInit, isTmp, enableGrad, grad,
+ * isGrad and the `income` edge used by autograd. It is not a re-implementation of the
  * reference's tensor class: memory pools, sparse storage, naming, gradients
  * and the 300-odd other members are outside this library. In an integration
  * the reference's own XTensor is used and only XTensorBLAS changes.
@@ -58,6 +58,11 @@ struct XLink {
     static void AddParamToHead(XTensor * h, DTYPE param);
     static void AddParamToHeadInt(XTensor * h, int param);
     static void AddParamToHeadTrans(XTensor * h, MATRIX_TRANS_TYPE param);
+
+    /* parameter i as recorded (source/tensor/XLink.cpp:287-328) */
+    DTYPE GetParam(int i) const;
+    int GetParamInt(int i) const;
+    MATRIX_TRANS_TYPE GetParamTrans(int i) const;
 };
 
 struct XTensor {
@@ -76,6 +81,10 @@ struct XTensor {
     bool isInit;
     bool isTmp;
     bool enableGrad;
+    /* dE/d(this tensor), owned by the tensor (source/tensor/XTensor.h:163-166); isGrad: the
+       tensor wants its gradient kept when the backward pass runs in its "efficient" mode */
+    XTensor * grad;
+    bool isGrad;
     XLink income;
 
     XTensor();
@@ -100,6 +109,9 @@ struct XTensor {
     void SetTMPFlag(bool myIsTmp = true);
     void DestroyData();
     int GetDim(int dim) const;
+    /* a new shape over the same elements (source/tensor/XTensor.cpp:618-650) */
+    void Reshape(const int myOrder, const int * myDimSize);
+    void Reshape(const int rowNum, const int colNum);
 
 private:
     void Init();
@@ -118,6 +130,8 @@ XTensor * NewTensor2DV2(const int rowNum, const int colNum, const TENSOR_DATA_TY
 XTensor * NewTensorBufV2(const int myOrder, const int * myDimSize, const TENSOR_DATA_TYPE myDataType = X_FLOAT,
                          const float myDenseRatio = 1.0F, const int myDevID = -1, XMem * myMem = NULL);
 void DelTensorBuf(XTensor * tensor);
+/* a tensor shaped like `a` on the same device (source/tensor/XCall.cpp:770-790) */
+XTensor * NewTensor(const XTensor * a, bool isFilledData = true);
 
 /* source/tensor/core/shape/IsSameShaped.cpp:32-58 */
 bool _IsSameShaped(const XTensor * a, const XTensor * b);

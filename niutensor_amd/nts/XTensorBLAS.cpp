@@ -68,6 +68,23 @@ void _AmdMatrixMULBias(int devID,
                                  na, ma, nb, mb, nc, mc, alpha, beta, bias, biasMode, biasLen, biasRowDiv));
 }
 
+void _AmdMatrixMULColSum(int devID,
+                         const void * a, MATRIX_TRANS_TYPE transposedA, TENSOR_DATA_TYPE dataTypeA,
+                         const void * b, MATRIX_TRANS_TYPE transposedB, TENSOR_DATA_TYPE dataTypeB,
+                         void * c, TENSOR_DATA_TYPE dataTypeC,
+                         int na, int ma, int nb, int mb, int nc, int mc, DTYPE alpha, DTYPE beta,
+                         void * colSum, DTYPE colSumBeta)
+{
+    Check(ntsamd_matrix_mul_colsum(devID, NULL, a, transposedA, dataTypeA, b, transposedB, dataTypeB, c, dataTypeC,
+                                   na, ma, nb, mb, nc, mc, alpha, beta, colSum, colSumBeta));
+}
+
+void _AmdReduceSumXZ(int devID, const void * in, TENSOR_DATA_TYPE dataType, int x, int y, int z,
+                     void * out, DTYPE beta)
+{
+    Check(ntsamd_reduce_sum_xz(devID, NULL, in, dataType, x, y, z, out, beta));
+}
+
 void _AmdMatrixMULBatched(int devID,
                           const void ** a, MATRIX_TRANS_TYPE transposedA, TENSOR_DATA_TYPE dataTypeA,
                           const void ** b, MATRIX_TRANS_TYPE transposedB, TENSOR_DATA_TYPE dataTypeB,

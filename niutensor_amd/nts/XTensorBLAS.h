@@ -57,5 +57,20 @@ void _AmdMatrixMULBias(int devID,
                        int na, int ma, int nb, int mb, int nc, int mc, DTYPE alpha, DTYPE beta,
                        const void * bias, int biasMode, int biasLen, int biasRowDiv);
 
+/* one product that also returns the column sums of op(b):
+   colSum[j] = colSumBeta * colSum[j] + sum_k op(b)[k][j]; for the backward step of MulAndShift,
+   where the reference runs _CudaBLASMatrixMUL, _CudaReduceSum and _CudaSum one after the other
+   (source/network/XBackwardMath.cpp:1805-1810, 1857-1879) */
+void _AmdMatrixMULColSum(int devID,
+                         const void * a, MATRIX_TRANS_TYPE transposedA, TENSOR_DATA_TYPE dataTypeA,
+                         const void * b, MATRIX_TRANS_TYPE transposedB, TENSOR_DATA_TYPE dataTypeB,
+                         void * c, TENSOR_DATA_TYPE dataTypeC,
+                         int na, int ma, int nb, int mb, int nc, int mc, DTYPE alpha, DTYPE beta,
+                         void * colSum, DTYPE colSumBeta);
+
+/* out[j] = beta * out[j] + sum_i sum_k in[i][j][k] over a dense [x][y][z] tensor */
+void _AmdReduceSumXZ(int devID, const void * in, TENSOR_DATA_TYPE dataType, int x, int y, int z,
+                     void * out, DTYPE beta);
+
 }  // namespace nts
 #endif

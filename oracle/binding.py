@@ -71,6 +71,15 @@ class Oracle:
         L.oracle_mulandshift.argtypes = [_fp, C.c_int, _ip, C.c_int, _fp, C.c_int, _ip, C.c_int,
                                          _fp, _ip, C.c_int, _fp, _ip, _ip, C.c_float]
         L.oracle_mulandshift.restype = C.c_int
+        L.oracle_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.oracle_reduce_sum.restype = C.c_int
+        L.oracle_grad_matmul.argtypes = [_fp, _fp, C.c_int, _ip, C.c_int, _fp, _fp, C.c_int, _ip, C.c_int, _fp, C.c_float]
+        L.oracle_grad_matmul.restype = C.c_int
+        L.oracle_grad_matmul_batched.argtypes = [_fp, _fp, C.c_int, _ip, _fp, _fp, C.c_int, _ip, _fp, _ip, C.c_int, C.c_float]
+        L.oracle_grad_matmul_batched.restype = C.c_int
+        L.oracle_grad_mulandshift.argtypes = [_fp, _fp, C.c_int, _ip, C.c_int, _fp, _fp, C.c_int, _ip, C.c_int,
+                                              _fp, C.c_int, _fp, _ip, C.c_int, C.c_int, C.c_float]
+        L.oracle_grad_mulandshift.restype = C.c_int
         L.oracle_is_float_equal.argtypes = [C.c_float] * 4
         L.oracle_is_float_equal.restype = C.c_int
         L.oracle_check_data.argtypes = [_fp, _fp, C.c_int, C.c_float]
@@ -141,6 +150,43 @@ class Oracle:
         return c, n
 
     # -- helpers ----------------------------------------------------------
+    # -- backward ---------------------------------------------------------
+    def reduce_sum(self, x, dim):
+        out = np.zeros(x.shape[:dim] + x.shape[dim + 1:], np.float32)
+        if self.lib.oracle_reduce_sum(_f(x), _dims(x.shape), x.ndim, dim, _f(out)) != 0:
+            raise ValueError("Illegal dimension to reduce!")
+        return out
+
+    @staticmethod
+    def _opt(g):
+        return _f(g) if g is not None else None
+
+    def grad_matmul(self, a, transA, b, transB, dedc, alpha=1.0, deda=None, dedb=None):
+        """deda, dedb: starting values of the gradients (updated in place and returned); None = not wanted."""
+        r = self.lib.oracle_grad_matmul(_f(a), self._opt(deda), transA, _dims(a.shape), a.ndim,
+                                        _f(b), self._opt(dedb), transB, _dims(b.shape), b.ndim, _f(dedc), alpha)
+        if r != 0:
+            raise ValueError("TODO!" if r == -2 else "Unmatched tensors in multiplication!")
+        return deda, dedb
+
+    def grad_matmul_batched(self, a, transA, b, transB, dedc, alpha=1.0, deda=None, dedb=None):
+        r = self.lib.oracle_grad_matmul_batched(_f(a), self._opt(deda), transA, _dims(a.shape),
+                                                _f(b), self._opt(dedb), transB, _dims(b.shape),
+                                                _f(dedc), _dims(dedc.shape), a.ndim, alpha)
+        if r != 0:
+            raise ValueError("Unmatched tensors in multiplication!")
+        return deda, dedb
+
+    def grad_mulandshift(self, x, w, dedc, n, alpha=1.0, dedx=None, dedw=None, dedbias=None,
+                         transX=X_NOTRANS, transW=X_NOTRANS):
+        r = self.lib.oracle_grad_mulandshift(_f(x), self._opt(dedx), transX, _dims(x.shape), x.ndim,
+                                             _f(w), self._opt(dedw), transW, _dims(w.shape), w.ndim,
+                                             self._opt(dedbias), 0 if dedbias is None else dedbias.size,
+                                             _f(dedc), _dims(dedc.shape), dedc.ndim, n, alpha)
+        if r != 0:
+            raise ValueError("TODO!" if r == -2 else "Wrong tensor size!")
+        return dedx, dedw, dedbias
+
     def is_float_equal(self, a, b, abs_err, rel_err=1e-4):
         return bool(self.lib.oracle_is_float_equal(a, b, abs_err, rel_err))
 
@@ -194,6 +240,9 @@ class Reference:
         L.ref_mulandshift.argtypes = [C.c_int, _fp, C.c_int, _ip, C.c_int, _fp, C.c_int, _ip, C.c_int,
                                       _fp, _ip, C.c_int, _fp, _ip, C.c_float]
         L.ref_enum_values.argtypes = [_ip]
+        L.ref_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.ref_grad.argtypes = [C.c_int, _fp, _ip, C.c_int, C.c_int, _fp, _ip, C.c_int, C.c_int,
+                               _fp, _ip, C.c_int, C.c_float, _fp, _fp, _fp, _fp]
 
     def matmul2d(self, a, transA, b, transB, c=None, alpha=1.0, beta=0.0):
         na, ma = a.shape
@@ -244,6 +293,20 @@ class Reference:
                                          _f(bias), _dims(bias.shape), bias.ndim, _f(c), cd, alpha)
         assert tuple(cd[i] for i in range(order)) == shape
         return c
+
+    def reduce_sum(self, x, dim):
+        out = np.zeros(x.shape[:dim] + x.shape[dim + 1:], np.float32)
+        self.lib.ref_reduce_sum(_f(x), _dims(x.shape), x.ndim, dim, _f(out))
+        return out
+
+    def grad(self, kind, a, transA, b, transB, dedc, alpha, deda, dedb, bias=None, dedbias=None):
+        """Forward with the reference's operator (0 MatrixMul, 1 MatrixMulBatched, 2 MulAndShift), then
+        its autograd step on the recorded edge; the gradients are updated in place."""
+        self.lib.ref_grad(kind, _f(a), _dims(a.shape), a.ndim, transA, _f(b), _dims(b.shape), b.ndim, transB,
+                          _f(bias) if bias is not None else None,
+                          _dims(bias.shape) if bias is not None else None, 0 if bias is None else bias.ndim,
+                          alpha, _f(dedc), _f(deda), _f(dedb), _f(dedbias) if dedbias is not None else None)
+        return deda, dedb, dedbias
 
     def run_matmul_tests(self):
         return self.lib.ref_run_matmul_tests()

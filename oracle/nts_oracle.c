@@ -370,6 +370,207 @@ int oracle_mulandshift(const float *x, int transX, const int *xDims, int xOrder,
     return n;
 }
 
+/* ---- backward: the products and sums the autograd issues for this path ------ */
+
+int oracle_reduce_sum(const float *in, const int *dims, int order, int dim, float *out)
+{
+    /* ReduceSum.cpp:47-80 */
+    if (order < 1 || dim < 0 || dim >= order)
+        return -1;
+    int stride = 1, strideNum = dims[dim], blockNum = 1;
+    for (int i = 0; i < order; i++) {
+        if (i < dim)
+            blockNum *= dims[i];
+        else if (i > dim)
+            stride *= dims[i];
+    }
+    long blockSize = (long)stride * strideNum;
+    int last = dims[order - 1];
+
+    if (last % 32 == 0 && last >= 32 && dim == order - 1) {
+        /* ReduceSum.cpp:83-116: 32 running sums (four buffers of eight lanes) over the
+           contiguous items, folded as (b0 + b1) + (b2 + b3) and then lane by lane from 0 */
+        for (int i = 0; i < blockNum; i++) {
+            const float *ip = in + blockSize * i;
+            float buf[4][8];
+            for (int k = 0; k < 4; k++)
+                for (int l = 0; l < 8; l++)
+                    buf[k][l] = ip[k * 8 + l] - 0.0F;
+            for (int j = 1; j < strideNum / 32; j++)
+                for (int k = 0; k < 4; k++)
+                    for (int l = 0; l < 8; l++)
+                        buf[k][l] = (ip[j * 32 + k * 8 + l] - 0.0F) + buf[k][l];
+            float sum = 0.0F;
+            for (int l = 0; l < 8; l++) {
+                /* operator+ computes a[i] + this[i]: the right operand comes first */
+                float b01 = buf[1][l] + buf[0][l];
+                float b23 = buf[3][l] + buf[2][l];
+                sum = sum + (b23 + b01);
+            }
+            out[i] = sum;
+        }
+        return 0;
+    }
+    /* ReduceSum.cpp:117-143 (buffers over columns) and :146-228 (scalar loop) both add the
+       items of one output element one after the other, in ascending position along dim;
+       the first starts from the first item, the second from 0 */
+    int vector = last % 32 == 0 && last >= 32;
+    for (int k = 0; k < blockNum; k++) {
+        const float *ip = in + blockSize * k;
+        float *op = out + (long)stride * k;
+        for (int i = 0; i < stride; i++) {
+            float sum;
+            int first;
+            if (vector) {
+                sum = ip[i] - 0.0F;
+                first = 1;
+            }
+            else {
+                sum = 0;
+                first = 0;
+            }
+            for (int j = first; j < strideNum; j++) {
+                if (vector)
+                    sum = (ip[(long)j * stride + i] - 0.0F) + sum;
+                else
+                    sum += ip[(long)j * stride + i];
+            }
+            op[i] = sum;
+        }
+    }
+    return 0;
+}
+
+int oracle_grad_matmul2d(const float *a, float *deda, int transA,
+                         const float *b, float *dedb, int transB,
+                         const float *dedc, int na, int ma, int nb, int mb, float alpha)
+{
+    /* shape of c as _MatrixMul2D sees it (MatrixMul2D.cpp:56-67) */
+    int cn = transA == ORACLE_X_TRANS ? ma : na;
+    int cm = transB == ORACLE_X_TRANS ? nb : mb;
+    int r = 0;
+    const int T = ORACLE_X_TRANS, NT = ORACLE_X_NOTRANS;
+    /* XBackwardMath.cpp:636-696: every gradient is ADDED to what the tensor holds (beta = 1) */
+    if (transA == NT && transB == NT) {
+        if (deda)
+            r |= oracle_matmul2d(dedc, NT, b, T, deda, cn, cm, nb, mb, na, ma, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul2d(a, T, dedc, NT, dedb, na, ma, cn, cm, nb, mb, alpha, 1.0F);
+    }
+    else if (transA == T && transB == NT) {
+        if (deda)
+            r |= oracle_matmul2d(b, NT, dedc, T, deda, nb, mb, cn, cm, na, ma, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul2d(a, NT, dedc, NT, dedb, na, ma, cn, cm, nb, mb, alpha, 1.0F);
+    }
+    else if (transA == NT && transB == T) {
+        if (deda)
+            r |= oracle_matmul2d(dedc, NT, b, NT, deda, cn, cm, nb, mb, na, ma, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul2d(dedc, T, a, NT, dedb, cn, cm, na, ma, nb, mb, alpha, 1.0F);
+    }
+    else {
+        if (deda)
+            r |= oracle_matmul2d(b, T, dedc, T, deda, nb, mb, cn, cm, na, ma, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul2d(dedc, T, a, T, dedb, cn, cm, na, ma, nb, mb, alpha, 1.0F);
+    }
+    return r;
+}
+
+int oracle_grad_matmul(const float *a, float *deda, int transA, const int *aDims, int aOrder,
+                       const float *b, float *dedb, int transB, const int *bDims, int bOrder,
+                       const float *dedc, float alpha)
+{
+    /* XBackwardMath.cpp:608-633 */
+    if (aOrder == 2 && bOrder == 2)
+        return oracle_grad_matmul2d(a, deda, transA, b, dedb, transB, dedc,
+                                    aDims[0], aDims[1], bDims[0], bDims[1], alpha);
+    if (transA == ORACLE_X_NOTRANS && aOrder > 2 && bOrder == 2) {
+        int ncolA = aDims[aOrder - 1];
+        return oracle_grad_matmul2d(a, deda, transA, b, dedb, transB, dedc,
+                                    (int)(unit_num(aDims, aOrder) / ncolA), ncolA, bDims[0], bDims[1], alpha);
+    }
+    return -2;      /* ShowNTErrors("TODO!") */
+}
+
+int oracle_grad_matmul_batched(const float *a, float *deda, int transA, const int *aDims,
+                               const float *b, float *dedb, int transB, const int *bDims,
+                               const float *dedc, const int *cDims, int order, float alpha)
+{
+    const int T = ORACLE_X_TRANS, NT = ORACLE_X_NOTRANS;
+    int r = 0;
+    /* XBackwardMath.cpp:731-786: the same eight products, batched */
+    if (transA == NT && transB == NT) {
+        if (deda)
+            r |= oracle_matmul_batched(dedc, NT, cDims, b, T, bDims, deda, aDims, order, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul_batched(a, T, aDims, dedc, NT, cDims, dedb, bDims, order, alpha, 1.0F);
+    }
+    else if (transA == T && transB == NT) {
+        if (deda)
+            r |= oracle_matmul_batched(b, NT, bDims, dedc, T, cDims, deda, aDims, order, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul_batched(a, NT, aDims, dedc, NT, cDims, dedb, bDims, order, alpha, 1.0F);
+    }
+    else if (transA == NT && transB == T) {
+        if (deda)
+            r |= oracle_matmul_batched(dedc, NT, cDims, b, NT, bDims, deda, aDims, order, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul_batched(dedc, T, cDims, a, NT, aDims, dedb, bDims, order, alpha, 1.0F);
+    }
+    else {
+        if (deda)
+            r |= oracle_matmul_batched(b, T, bDims, dedc, T, cDims, deda, aDims, order, alpha, 1.0F);
+        if (dedb)
+            r |= oracle_matmul_batched(dedc, T, cDims, a, T, aDims, dedb, bDims, order, alpha, 1.0F);
+    }
+    return r;
+}
+
+int oracle_grad_mulandshift(const float *x, float *dedx, int transX, const int *xDims, int xOrder,
+                            const float *w, float *dedw, int transW, const int *wDims, int wOrder,
+                            float *dedbias, int biasNum,
+                            const float *dedc, const int *cDims, int cOrder, int n, float alpha)
+{
+    long num = unit_num(cDims, cOrder);
+    if (dedbias) {
+        float *tmp = (float *)malloc(sizeof(float) * (size_t)(biasNum > 0 ? biasNum : 1));
+        if (!tmp)
+            return -1;
+        if (n == cOrder - 1) {
+            /* XBackwardMath.cpp:1797-1814: dE/dc as a matrix with |b| columns, summed over its
+               rows into a temporary, which _Sum then adds to the gradient (c = a + b * 1) */
+            int d2[2] = {(int)(num / cDims[cOrder - 1]), cDims[cOrder - 1]};
+            if (d2[1] != biasNum || oracle_reduce_sum(dedc, d2, 2, 0, tmp) != 0) {
+                free(tmp);
+                return -1;
+            }
+        }
+        else {
+            /* :1816-1846: dE/dc as (x, |b|, z), summed over z, then over x */
+            int d3[3] = {1, cDims[n], 1};
+            for (int i = 0; i < n; i++)
+                d3[0] *= cDims[i];
+            d3[2] = (int)(num / ((long)d3[0] * d3[1]));
+            float *inter = (float *)malloc(sizeof(float) * (size_t)d3[0] * d3[1]);
+            if (!inter || d3[1] != biasNum) {
+                free(inter);
+                free(tmp);
+                return -1;
+            }
+            oracle_reduce_sum(dedc, d3, 3, 2, inter);
+            oracle_reduce_sum(inter, d3, 2, 0, tmp);
+            free(inter);
+        }
+        for (int i = 0; i < biasNum; i++)
+            dedbias[i] = tmp[i] + dedbias[i];
+        free(tmp);
+    }
+    /* :1857-1879: the products of GradMatrixMul on x and w */
+    return oracle_grad_matmul(x, dedx, transX, xDims, xOrder, w, dedw, transW, wDims, wOrder, dedc, alpha);
+}
+
 /* ---- comparator ---------------------------------------------------------- */
 
 int oracle_is_float_equal(float a, float b, float absError, float relError)

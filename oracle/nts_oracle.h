@@ -60,6 +60,37 @@ int oracle_mulandshift(const float *x, int transX, const int *xDims, int xOrder,
                        const float *bias, const int *bDims, int bOrder,
                        float *c, int *cDims, int *cOrder, float alpha);
 
+/* out = sum of `in` along dimension dim; the CPU branch of ReduceSum.cpp:47-232 with
+   power 1, no shift, no exp (how GradMulAndShift calls it), including the order in which
+   its 32-lane buffers fold when the reduced dimension is the last one. */
+int oracle_reduce_sum(const float *in, const int *dims, int order, int dim, float *out);
+
+/* The products XMathGrad::GradMatrixMul issues for c = op(a) op(b) alpha on 2-D tensors
+   (source/network/XBackwardMath.cpp:636-696): deda += ..., dedb += ... (beta = 1); a NULL
+   gradient is skipped, as for a tensor that needs none. dedc is [rows of op(a)] x [cols of op(b)]. */
+int oracle_grad_matmul2d(const float *a, float *deda, int transA,
+                         const float *b, float *dedb, int transB,
+                         const float *dedc, int na, int ma, int nb, int mb, float alpha);
+
+/* XMathGrad::GradMatrixMul(node) (XBackwardMath.cpp:584-633): 2-D x 2-D, or the flatten
+   rule for an untransposed N-D a; -2 where the reference aborts with "TODO!". */
+int oracle_grad_matmul(const float *a, float *deda, int transA, const int *aDims, int aOrder,
+                       const float *b, float *dedb, int transB, const int *bDims, int bOrder,
+                       const float *dedc, float alpha);
+
+/* XMathGrad::GradMatrixMulBatched (XBackwardMath.cpp:709-786) */
+int oracle_grad_matmul_batched(const float *a, float *deda, int transA, const int *aDims,
+                               const float *b, float *dedb, int transB, const int *bDims,
+                               const float *dedc, const int *cDims, int order, float alpha);
+
+/* XMathGrad::GradMulAndShift (XBackwardMath.cpp:1774-1884) for c = alpha op(x) op(w) + bias with
+   the bias broadcast along dimension n of c: dedbias += sums of dedc, then GradMatrixMul.
+   transX / transW are the flags as that function holds them in its local variables. */
+int oracle_grad_mulandshift(const float *x, float *dedx, int transX, const int *xDims, int xOrder,
+                            const float *w, float *dedw, int transW, const int *wDims, int wOrder,
+                            float *dedbias, int biasNum,
+                            const float *dedc, const int *cDims, int cOrder, int n, float alpha);
+
 /* comparator of the reference tests, CheckData.cpp:29-39 */
 int oracle_is_float_equal(float a, float b, float absError, float relError);
 /* CheckData.cpp:78-97 with its fixed relative bound 1e-4 */

@@ -6,7 +6,9 @@
  * resulting library is only used to validate the C restatement in
  * nts_oracle.c and, optionally, as the CPU baseline. Every tensor here lives
  * on the host (devID = -1), so the reference takes its naive CPU path
- * (_MatrixMul2DParallel; no BLAS is linked).
+ * (_MatrixMul2DParallel; no BLAS is linked). The backward entry points run the
+ * reference's own autograd step (source/network/XBackwardMath.cpp) on the edge
+ * that its forward operator recorded.
  */
 #include "XTensor.h"
 #include "XCall.h"
@@ -16,6 +18,7 @@
 #include "test/TMatrixMul2DParallel.h"
 #include "test/TMatrixMulBatched.h"
 #include "test/TSumDim.h"
+#include "../network/XBackwardMath.h"
 
 #include <string.h>
 
@@ -128,6 +131,71 @@ int ref_mulandshift(int overload,
     memcpy(c, tc.data, sizeof(float) * (size_t)tc.unitNum);
     int order = tc.order;
     delete tx; delete tw; delete tb;
+    return order;
+}
+
+int ref_reduce_sum(const float * in, const int * dims, int order, int dim, float * out)
+{
+    XTensor * ti = Make(dims, order, in);
+    int od[MAX_TENSOR_DIM_NUM];
+    int n = 0;
+    for (int i = 0; i < order; i++)
+        if (i != dim)
+            od[n++] = dims[i];
+    XTensor * to = Make(od, order - 1, NULL);
+    _ReduceSum(ti, to, dim);
+    memcpy(out, to->data, sizeof(float) * (size_t)to->unitNum);
+    delete ti; delete to;
+    return 0;
+}
+
+/* Forward with the reference's operator (kind 0: MatrixMul, 1: MatrixMulBatched,
+   2: MulAndShift(x, w, b, alpha)) with gradients enabled, so that the result carries the
+   edge; then dE/dc is set and XMathGrad::MakeGrad runs the backward step for that edge.
+   deda / dedb / dedbias hold the gradients' starting values on entry (the step adds to
+   them) and the results on return. Returns the order of c. */
+int ref_grad(int kind,
+             const float * a, const int * aDims, int aOrder, int transA,
+             const float * b, const int * bDims, int bOrder, int transB,
+             const float * bias, const int * biasDims, int biasOrder,
+             float alpha, const float * dedc,
+             float * deda, float * dedb, float * dedbias)
+{
+    bool backup = X_ENABLE_GRAD;
+    X_ENABLE_GRAD = true;
+    XTensor * ta = Make(aDims, aOrder, a);
+    XTensor * tb = Make(bDims, bOrder, b);
+    XTensor * tbias = kind == 2 ? Make(biasDims, biasOrder, bias) : NULL;
+    int order;
+    {
+        XTensor tc;
+        if (kind == 0)
+            tc = MatrixMul(*ta, (MATRIX_TRANS_TYPE)transA, *tb, (MATRIX_TRANS_TYPE)transB, alpha);
+        else if (kind == 1)
+            tc = MatrixMulBatched(*ta, (MATRIX_TRANS_TYPE)transA, *tb, (MATRIX_TRANS_TYPE)transB, alpha);
+        else
+            tc = MulAndShift(*ta, *tb, *tbias, alpha);
+        order = tc.order;
+        tc.grad = NewTensor(&tc);
+        tc.grad->SetData(dedc, tc.unitNum);
+        ta->grad = NewTensor(ta);
+        ta->grad->SetData(deda, ta->unitNum);
+        tb->grad = NewTensor(tb);
+        tb->grad->SetData(dedb, tb->unitNum);
+        if (tbias != NULL) {
+            tbias->grad = NewTensor(tbias);
+            tbias->grad->SetData(dedbias, tbias->unitNum);
+        }
+        XMathGrad::MakeGrad(&tc, false);
+        memcpy(deda, ta->grad->data, sizeof(float) * (size_t)ta->unitNum);
+        memcpy(dedb, tb->grad->data, sizeof(float) * (size_t)tb->unitNum);
+        if (tbias != NULL)
+            memcpy(dedbias, tbias->grad->data, sizeof(float) * (size_t)tbias->unitNum);
+    }
+    delete ta; delete tb;
+    if (tbias != NULL)
+        delete tbias;
+    X_ENABLE_GRAD = backup;
     return order;
 }
 

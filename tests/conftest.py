@@ -40,8 +40,8 @@ def known_answers():
 class Generated:
     """tests/golden/ref_generated.npz: outputs of the compiled reference (see make_fixtures.py)."""
 
-    def __init__(self):
-        self.z = np.load(os.path.join(GOLDEN, "ref_generated.npz"), allow_pickle=False)
+    def __init__(self, file="ref_generated.npz"):
+        self.z = np.load(os.path.join(GOLDEN, file), allow_pickle=False)
         self.names = [str(n) for n in self.z["index"]]
 
     def case(self, name):
@@ -55,6 +55,12 @@ class Generated:
 @pytest.fixture(scope="session")
 def generated():
     return Generated()
+
+
+@pytest.fixture(scope="session")
+def generated_backward():
+    """tests/golden/ref_generated_backward.npz: gradients left by the compiled reference's autograd step."""
+    return Generated("ref_generated_backward.npz")
 
 
 @pytest.fixture(scope="session")

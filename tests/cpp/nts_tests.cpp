@@ -5,7 +5,7 @@
  * known answer through the reference's comparator (abs 1e-4 or rel 1e-4,
  * core/utilities/CheckData.cpp:29-39). The GPU halves of those tests are what is
  * reproduced here; cases the reference does not have (NT/TT, alpha/beta, fp16,
- * MulAndShift, lists) are checked against the CPU oracle on seeded inputs.
+ * MulAndShift, lists, the backward step) are checked against the CPU oracle on seeded inputs.
  *
  *   nts_tests                run everything on device 0, exit 0 if all passed
  *   nts_tests --abort NAME   provoke one fatal error (no GPU needed): the process
@@ -16,6 +16,7 @@
 #include "../../niutensor_amd/nts/MatrixMul2D.h"
 #include "../../niutensor_amd/nts/MatrixMulBatched.h"
 #include "../../niutensor_amd/nts/MulAndShift.h"
+#include "../../niutensor_amd/nts/XBackwardMath.h"
 #include "../../oracle/nts_oracle.h"
 
 #include <math.h>
@@ -422,6 +423,191 @@ static bool TestBetaZeroIgnoresOldContents()
     return ok;
 }
 
+/* ---- backward: XMathGrad on the edges the forward operators record ------------ */
+
+static std::vector<float> Filled(int n, uint64_t seed)
+{
+    std::vector<float> v(n);
+    oracle_fill_uniform(v.data(), n, seed, -1, 1);
+    return v;
+}
+
+static void SetGrad(XTensor * t, const std::vector<float> & g)
+{
+    t->grad = NewTensor(t);
+    t->grad->SetData(g.data(), t->unitNum);
+}
+
+static float GradErr(const XTensor * t, const std::vector<float> & ref)
+{
+    std::vector<float> got(ref.size());
+    t->grad->GetData(got.data());
+    return MaxRelErr(got, ref);
+}
+
+/* MatrixMul, 2-D, every transpose pair; gradients start non-zero: the step must ADD */
+static bool TestGradMatrixMul()
+{
+    bool ok = true;
+    const int M = 70, K = 45, N = 52;
+    for (int ta = 0; ta < 2; ta++)
+        for (int tb = 0; tb < 2; tb++) {
+            int da[2] = {ta == X_TRANS ? K : M, ta == X_TRANS ? M : K};
+            int db[2] = {tb == X_TRANS ? N : K, tb == X_TRANS ? K : N};
+            std::vector<float> a = Filled(M * K, 1), b = Filled(K * N, 2), dedc = Filled(M * N, 3);
+            std::vector<float> deda = Filled(M * K, 4), dedb = Filled(K * N, 5);
+            XTensor * ga = NewGPU(2, da, a.data());
+            XTensor * gb = NewGPU(2, db, b.data());
+            ga->enableGrad = gb->enableGrad = true;
+            SetGrad(ga, deda);
+            SetGrad(gb, dedb);
+            {
+                XTensor c = MatrixMul(*ga, (MATRIX_TRANS_TYPE)ta, *gb, (MATRIX_TRANS_TYPE)tb, 0.75F);
+                SetGrad(&c, dedc);
+                ok = ok && XMathGrad::IsMathOP(&c);
+                XMathGrad::MakeGrad(&c, false);
+            }
+            oracle_grad_matmul(a.data(), deda.data(), ta, da, 2, b.data(), dedb.data(), tb, db, 2, dedc.data(), 0.75F);
+            float ea = GradErr(ga, deda), eb = GradErr(gb, dedb);
+            if (!(ea < 8e-5F && eb < 8e-5F)) {
+                fprintf(stderr, "grad matmul ta=%d tb=%d: %g %g\n", ta, tb, ea, eb);
+                ok = false;
+            }
+            delete ga; delete gb;
+        }
+    return ok;
+}
+
+/* the flatten rule (an untransposed a of order 3 against a matrix), and the "efficient" mode:
+   only tensors with isGrad set receive a gradient */
+static bool TestGradMatrixMulFlattenAndEfficient()
+{
+    int da[3] = {5, 9, 20}, db[2] = {20, 16};
+    std::vector<float> a = Filled(900, 11), b = Filled(320, 12), dedc = Filled(5 * 9 * 16, 13);
+    std::vector<float> deda(900, 0.f), dedb(320, 0.f);
+    XTensor * ga = NewGPU(3, da, a.data());
+    XTensor * gb = NewGPU(2, db, b.data());
+    ga->enableGrad = gb->enableGrad = true;
+    gb->isGrad = true;                       /* a does not want a gradient */
+    bool ok = true;
+    {
+        XTensor c = MatrixMul(*ga, X_NOTRANS, *gb, X_NOTRANS);
+        SetGrad(&c, dedc);
+        XMathGrad::MakeGrad(&c, true);
+        ok = ok && c.order == 3 && c.grad->order == 3 && ga->order == 3;     /* shapes restored */
+    }
+    ok = ok && ga->grad == NULL && gb->grad != NULL;
+    oracle_grad_matmul(a.data(), NULL, X_NOTRANS, da, 3, b.data(), dedb.data(), X_NOTRANS, db, 2, dedc.data(), 1.0F);
+    ok = ok && GradErr(gb, dedb) < 8e-5F;
+    /* the full mode gives a its gradient too */
+    {
+        XTensor c = MatrixMul(*ga, X_NOTRANS, *gb, X_NOTRANS);
+        SetGrad(&c, dedc);
+        XMathGrad::MakeGrad(&c, false);
+    }
+    oracle_grad_matmul(a.data(), deda.data(), X_NOTRANS, da, 3, b.data(), dedb.data(), X_NOTRANS, db, 2, dedc.data(), 1.0F);
+    ok = ok && ga->grad != NULL && ga->grad->order == 3 && GradErr(ga, deda) < 8e-5F && GradErr(gb, dedb) < 8e-5F;
+    delete ga; delete gb;
+    return ok;
+}
+
+static bool TestGradMatrixMulBatched()
+{
+    bool ok = true;
+    const int B = 6, M = 40, K = 24, N = 50;
+    for (int ta = 0; ta < 2; ta++)
+        for (int tb = 0; tb < 2; tb++) {
+            int da[3] = {B, ta == X_TRANS ? K : M, ta == X_TRANS ? M : K};
+            int db[3] = {B, tb == X_TRANS ? N : K, tb == X_TRANS ? K : N};
+            int dc[3] = {B, M, N};
+            std::vector<float> a = Filled(B * M * K, 21), b = Filled(B * K * N, 22), dedc = Filled(B * M * N, 23);
+            std::vector<float> deda = Filled(B * M * K, 24), dedb = Filled(B * K * N, 25);
+            XTensor * ga = NewGPU(3, da, a.data());
+            XTensor * gb = NewGPU(3, db, b.data());
+            ga->enableGrad = gb->enableGrad = true;
+            SetGrad(ga, deda);
+            SetGrad(gb, dedb);
+            {
+                XTensor c = MatrixMulBatched(*ga, (MATRIX_TRANS_TYPE)ta, *gb, (MATRIX_TRANS_TYPE)tb, 0.125F);
+                SetGrad(&c, dedc);
+                XMathGrad::MakeGrad(&c, false);
+            }
+            oracle_grad_matmul_batched(a.data(), deda.data(), ta, da, b.data(), dedb.data(), tb, db, dedc.data(), dc, 3, 0.125F);
+            float ea = GradErr(ga, deda), eb = GradErr(gb, dedb);
+            if (!(ea < 8e-5F && eb < 8e-5F)) {
+                fprintf(stderr, "grad batched ta=%d tb=%d: %g %g\n", ta, tb, ea, eb);
+                ok = false;
+            }
+            delete ga; delete gb;
+        }
+    return ok;
+}
+
+/* MulAndShift: bias along the last dimension (its gradient rides on the dE/dw product), along a
+   middle one and along the first (a reduction of its own); fp32 and fp16 */
+static bool TestGradMulAndShift()
+{
+    bool ok = true;
+    int dx[3] = {4, 6, 40}, dw[2] = {40, 32};
+    int biasShapes[3][3] = {{32, 0, 0}, {6, 0, 0}, {4, 1, 1}};
+    int biasOrders[3] = {1, 1, 3};
+    for (int half = 0; half < 2; half++)
+        for (int i = 0; i < 3; i++) {
+            const TENSOR_DATA_TYPE type = half ? X_FLOAT16 : X_FLOAT;
+            const int nb = Prod(biasShapes[i], biasOrders[i]);
+            std::vector<float> x = Filled(960, 31), w = Filled(1280, 32), bias = Filled(nb, 33), dedc = Filled(4 * 6 * 32, 34);
+            std::vector<float> dedx = Filled(960, 35), dedw = Filled(1280, 36), dedb = Filled(nb, 37);
+            std::vector<float> * all[7] = {&x, &w, &bias, &dedc, &dedx, &dedw, &dedb};
+            if (half)
+                for (int k = 0; k < 7; k++) {           /* the checker works on the values the GPU holds */
+                    std::vector<uint16_t> h(all[k]->size());
+                    oracle_f32_to_f16_array(all[k]->data(), h.data(), (long)h.size());
+                    oracle_f16_to_f32_array(h.data(), all[k]->data(), (long)h.size());
+                }
+            XTensor * gx = NewGPU(3, dx, x.data(), type);
+            XTensor * gw = NewGPU(2, dw, w.data(), type);
+            XTensor * gb = NewGPU(biasOrders[i], biasShapes[i], bias.data(), type);
+            gx->enableGrad = gw->enableGrad = gb->enableGrad = true;
+            gx->grad = NewGPU(3, dx, dedx.data(), type);
+            gw->grad = NewGPU(2, dw, dedw.data(), type);
+            gb->grad = NewGPU(biasOrders[i], biasShapes[i], dedb.data(), type);
+            int n;
+            {
+                XTensor c = MulAndShift(*gx, *gw, *gb, 0.5F);
+                n = c.income.GetParamInt(0);
+                int dc[3] = {4, 6, 32};
+                c.grad = NewGPU(3, dc, dedc.data(), type);
+                XMathGrad::MakeGrad(&c, false);
+                ok = ok && c.grad->order == 3 && gx->grad->order == 3;
+            }
+            int dc[3] = {4, 6, 32};
+            oracle_grad_mulandshift(x.data(), dedx.data(), X_NOTRANS, dx, 3, w.data(), dedw.data(), X_NOTRANS, dw, 2,
+                                    dedb.data(), nb, dedc.data(), dc, 3, n, 0.5F);
+            std::vector<float> got;
+            float errs[3];
+            XTensor * grads[3] = {gx->grad, gw->grad, gb->grad};
+            std::vector<float> * refs[3] = {&dedx, &dedw, &dedb};
+            for (int k = 0; k < 3; k++) {
+                got.resize(refs[k]->size());
+                if (half) {
+                    std::vector<uint16_t> h(got.size());
+                    grads[k]->GetData(h.data());
+                    oracle_f16_to_f32_array(h.data(), got.data(), (long)h.size());
+                }
+                else
+                    grads[k]->GetData(got.data());
+                errs[k] = MaxRelErr(got, *refs[k]);
+            }
+            const float lim = half ? 1e-2F : 8e-5F;
+            if (!(errs[0] < lim && errs[1] < lim && errs[2] < lim)) {
+                fprintf(stderr, "grad mulandshift half=%d bias %d (n=%d): %g %g %g\n", half, i, n, errs[0], errs[1], errs[2]);
+                ok = false;
+            }
+            delete gx; delete gw; delete gb;
+        }
+    return ok;
+}
+
 /* ---- fatal errors: same message, same ending as the reference ---------------- */
 
 static int Provoke(const char * name)
@@ -444,6 +630,22 @@ static int Provoke(const char * name)
         _MatrixMul(NULL, X_NOTRANS, &b, X_NOTRANS, &c);
     else if (!strcmp(name, "host"))
         _MatrixMul2D(&host, X_NOTRANS, &host, X_NOTRANS, &host);
+    else if (!strcmp(name, "nograd")) {
+        /* a node without dE/dc cannot be differentiated (XBackwardMath.cpp:34-36) */
+        XLink::MakeLink(&a, &b, &c, MATH_MATRIXMUL);
+        XMathGrad::MakeGrad(&c, false);
+    }
+    else if (!strcmp(name, "gradtodo")) {
+        /* a transposed a of order 3 has no backward in the reference either (:631-633) */
+        XTensor cc(3, d223, X_FLOAT, 1.0F, 0, NULL);
+        XLink::MakeLink(&t3, &b, &cc, MATH_MATRIXMUL);
+        XLink::AddParamToHeadTrans(&cc, X_TRANS);
+        XLink::AddParamToHeadTrans(&cc, X_NOTRANS);
+        XLink::AddParamToHead(&cc, 1.0F);
+        t3.isGrad = false;
+        cc.grad = new XTensor(3, d223, X_FLOAT, 1.0F, 0, NULL);
+        XMathGrad::MakeGrad(&cc, true);
+    }
     else if (!strcmp(name, "biasshape")) {
         XTensor bias(2, d22, X_FLOAT, 1.0F, 0, NULL);
         MulAndShift(a, b, bias);
@@ -473,6 +675,10 @@ int main(int argc, char ** argv)
     RUN(TestMatrixMulHalf);
     RUN(TestMatrixMulLinkAndReuse);
     RUN(TestBetaZeroIgnoresOldContents);
+    RUN(TestGradMatrixMul);
+    RUN(TestGradMatrixMulFlattenAndEfficient);
+    RUN(TestGradMatrixMulBatched);
+    RUN(TestGradMulAndShift);
     printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
     return all ? 0 : 1;
 }

@@ -20,7 +20,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
-from oracle.binding import Oracle, Reference, X_TRANS, X_NOTRANS  # noqa: E402
+from oracle.binding import Oracle, Reference, X_TRANS, X_NOTRANS, mm_shape, bmm_shape  # noqa: E402
 
 
 def main():
@@ -126,5 +126,80 @@ def main():
     print("wrote", path, len(index), "cases", os.path.getsize(path), "bytes")
 
 
+def backward():
+    o = Oracle()
+    r = Reference()
+    out = {}
+    index = []
+
+    def put(name, **arrays):
+        index.append(name)
+        for k, v in arrays.items():
+            out["%s/%s" % (name, k)] = np.asarray(v)
+
+    seed = 5000
+
+    # _ReduceSum: scalar loop, column buffers, and the 32-lane fold over a contiguous last dimension
+    for i, (shape, dim) in enumerate([((7, 5), 0), ((9, 64), 0), ((5, 96), 1), ((6, 160), 1), ((4, 6, 32), 2),
+                                      ((4, 6, 33), 2), ((3, 5, 7), 1), ((70, 128), 0), ((4, 6, 32), 0)]):
+        seed += 1
+        x = o.uniform(shape, seed)
+        put("reduce_%d" % i, kind="reduce_sum", x=x, y=r.reduce_sum(x, dim), params=[dim])
+
+    # GradMatrixMul: 2-D, all transposes; flatten rule
+    mm = [((9, 7), (7, 5)), ((33, 20), (20, 17))]
+    for i, (sa, sb) in enumerate(mm):
+        for ta, tb in itertools.product((X_NOTRANS, X_TRANS), repeat=2):
+            seed += 6
+            M, K = sa
+            N = sb[1]
+            a = o.uniform((K, M) if ta == X_TRANS else (M, K), seed)
+            b = o.uniform((N, K) if tb == X_TRANS else (K, N), seed + 1)
+            dedc = o.uniform((M, N), seed + 2)
+            deda0, dedb0 = o.uniform(a.shape, seed + 3), o.uniform(b.shape, seed + 4)
+            deda, dedb, _ = r.grad(0, a, ta, b, tb, dedc, 0.75, deda0.copy(), dedb0.copy())
+            put("gmm_%d_%d%d" % (i, ta, tb), kind="grad_matmul", a=a, b=b, dedc=dedc, deda0=deda0, dedb0=dedb0,
+                deda=deda, dedb=dedb, params=[ta, tb], scal=[0.75])
+    for i, (sa, sb, tb) in enumerate([((3, 4, 6), (6, 5), X_NOTRANS), ((2, 3, 4, 6), (5, 6), X_TRANS)]):
+        seed += 6
+        a, b = o.uniform(sa, seed), o.uniform(sb, seed + 1)
+        dedc = o.uniform(mm_shape(sa, X_NOTRANS, sb, tb), seed + 2)
+        deda0, dedb0 = o.uniform(sa, seed + 3), o.uniform(sb, seed + 4)
+        deda, dedb, _ = r.grad(0, a, X_NOTRANS, b, tb, dedc, 1.0, deda0.copy(), dedb0.copy())
+        put("gmm_flat_%d" % i, kind="grad_matmul", a=a, b=b, dedc=dedc, deda0=deda0, dedb0=dedb0,
+            deda=deda, dedb=dedb, params=[X_NOTRANS, tb], scal=[1.0])
+
+    # GradMatrixMulBatched
+    for ta, tb in itertools.product((X_NOTRANS, X_TRANS), repeat=2):
+        seed += 6
+        M, K, N = 6, 9, 5
+        a = o.uniform((4, K, M) if ta == X_TRANS else (4, M, K), seed)
+        b = o.uniform((4, N, K) if tb == X_TRANS else (4, K, N), seed + 1)
+        dedc = o.uniform(bmm_shape(a.shape, ta, b.shape, tb), seed + 2)
+        deda0, dedb0 = o.uniform(a.shape, seed + 3), o.uniform(b.shape, seed + 4)
+        deda, dedb, _ = r.grad(1, a, ta, b, tb, dedc, 0.125, deda0.copy(), dedb0.copy())
+        put("gbmm_%d%d" % (ta, tb), kind="grad_matmul_batched", a=a, b=b, dedc=dedc, deda0=deda0, dedb0=dedb0,
+            deda=deda, dedb=dedb, params=[ta, tb], scal=[0.125])
+
+    # GradMulAndShift (first overload): bias on the last dimension (with and without the 32-lane
+    # buffers), on a middle one and on the first
+    for i, (sx, sw, sb) in enumerate([((4, 6, 8), (8, 64), (64,)), ((4, 6, 8), (8, 5), (5,)), ((12, 8), (8, 32), (32,)),
+                                      ((5, 6, 8), (8, 7), (6,)), ((4, 32, 8), (8, 32), (4,)), ((3, 6, 8), (8, 6), (6,))]):
+        seed += 8
+        x, w, bias = o.uniform(sx, seed), o.normal(sw, seed + 1, 0, 0.5), o.normal(sb, seed + 2, 0, 0.5)
+        cshape = mm_shape(sx, X_NOTRANS, sw, X_NOTRANS)
+        dedc = o.uniform(cshape, seed + 3)
+        dedx0, dedw0, dedb0 = o.uniform(sx, seed + 4), o.uniform(sw, seed + 5), o.uniform(sb, seed + 6)
+        dedx, dedw, dedb = r.grad(2, x, X_NOTRANS, w, X_NOTRANS, dedc, 0.5, dedx0.copy(), dedw0.copy(), bias, dedb0.copy())
+        put("gmas_%d" % i, kind="grad_mulandshift", x=x, w=w, bias=bias, dedc=dedc, dedx0=dedx0, dedw0=dedw0,
+            dedb0=dedb0, dedx=dedx, dedw=dedw, dedb=dedb, params=[r.broadcast_dim_index(cshape, sb)], scal=[0.5])
+
+    out["index"] = np.array(index)
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_generated_backward.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, len(index), "cases", os.path.getsize(path), "bytes")
+
+
 if __name__ == "__main__":
     main()
+    backward()

@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 7
+    assert len(names) == 9
     assert sorted(nt.EXPORTS) == names
     lib = C.CDLL(nt.LIB_PATH)
     for name in names:
@@ -85,6 +85,27 @@ def test_argument_errors_need_no_device():
     assert rc == 1
 
 
+def test_column_sum_and_reduction_argument_errors_need_no_device():
+    L = nt.load()
+    cs = L.ntsamd_matrix_mul_colsum
+    # missing column-sum buffer; half inputs with a float result; shapes that do not multiply
+    assert cs(0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 3, 2, 2, 2, 1.0, 0.0, None, 0.0) == 1
+    assert "column sums" in L.ntsamd_last_error().decode()
+    assert cs(0, None, 0x1000, 1, 3, 0x1000, 1, 3, 0x1000, 2, 2, 3, 3, 2, 2, 2, 1.0, 0.0, 0x1000, 0.0) == 2
+    assert cs(0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 2, 3, 2, 3, 1.0, 0.0, 0x1000, 0.0) == 1
+    assert cs(0, None, None, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 3, 2, 2, 2, 1.0, 0.0, 0x1000, 0.0) == 1
+    # no columns: nothing to do
+    assert cs(0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2, 2, 3, 3, 0, 2, 0, 1.0, 0.0, 0x1000, 0.0) == 0
+    rs = L.ntsamd_reduce_sum_xz
+    assert rs(0, None, 0x1000, 4, 2, 3, 1, 0x1000, 0.0) == 2              # X_DOUBLE
+    assert L.ntsamd_last_error().decode() == "Unsupported data type!"
+    assert rs(0, None, 0x1000, 2, -2, 3, 1, 0x1000, 0.0) == 1
+    assert rs(0, None, None, 2, 2, 3, 1, 0x1000, 0.0) == 1
+    assert rs(0, None, 0x1000, 2, 2, 3, 1, None, 0.0) == 1
+    assert rs(0, None, 0x1000, 2, 70000, 70000, 1, 0x1000, 0.0) == 1
+    assert rs(0, None, 0x1000, 2, 5, 0, 1, 0x1000, 0.0) == 0              # no output elements
+
+
 def test_empty_products_succeed_without_a_device():
     L = nt.load()
     # zero rows, zero columns, zero batch items: nothing to do, no device needed
@@ -111,6 +132,8 @@ def test_invalid_device_is_an_error():
     ("empty", "Empty input tensors!"),
     ("host", "does not replace"),
     ("biasshape", "TODO!"),
+    ("nograd", "No gradient found!"),
+    ("gradtodo", "TODO!"),
 ])
 def test_nts_layer_fatal_errors(case, message):
     """CheckNTErrors / ShowNTErrors of the reference: '[ERROR] ...' on stderr, then std::terminate."""
