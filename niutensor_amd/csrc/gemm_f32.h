@@ -427,17 +427,25 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         }
         if (p.splits > 1) {
             /* one of several workgroups that share this tile: add the partial product to c,
-               which already holds beta * c; the bias rides on the first piece */
+               which already holds beta * c; the bias rides on the first piece. Every add is
+               predicated on its own row and column: an atomic must never be issued out of range
+               (loads and stores past the end of a buffer are dropped by the hardware; this path
+               does not rely on the same for atomics and uses plain global atomics). */
 #pragma unroll
-            for (int i = 0; i < TI; i++)
+            for (int j = 0; j < TJ; j++) {
+                const int col = n0 + wn0 + j * 32 + l32;
+                if (col < N) {
+                    const float bj = tc.split == 0 ? bcol[j] : 0.f;
 #pragma unroll
-                for (int j = 0; j < TJ; j++)
+                    for (int i = 0; i < TI; i++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
-                        const float v = alpha * acc[i][j][r] + (tc.split == 0 ? bcol[j] : 0.f);
-                        (void)__builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, cr, (int)off, 0, 0);
-                    }
+                        for (int r = 0; r < 16; r++) {
+                            const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                            if (row < M)
+                                unsafeAtomicAdd(C + (size_t)row * p.ldc + col, alpha * acc[i][j][r] + bj);
+                        }
+                }
+            }
             return;
         }
         /* beta is tested once, outside the loops: inside them the test would fence every

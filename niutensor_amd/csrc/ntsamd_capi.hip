@@ -258,11 +258,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
-       gradients); the pieces add to c with fp32 atomics, so c gets its beta first.
-       SWITCHED OFF: a product cut this way ended in a GPU memory fault whose cause has not
-       been found yet, so every product runs as one piece per tile until it has. */
-    const bool splitKEnabled = false;
-    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, splitKEnabled && kind == KIND_F32 && vec);
+       gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
+    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec);
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;

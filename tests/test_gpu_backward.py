@@ -50,12 +50,6 @@ def name_the_case(request):
 
 # ---- k cut into pieces ------------------------------------------------------------
 
-SPLIT_K_OFF = ("the split-k path is switched off in the library: a product cut along k ended in a GPU memory fault "
-               "(HSA_STATUS_ERROR_MEMORY_APERTURE_VIOLATION in gemm_f32_kernel<128,128,...>, 4 workgroups) whose cause "
-               "has not been found; the case stays off the GPU until it has")
-
-
-@pytest.mark.skip(reason=SPLIT_K_OFF)
 @pytest.mark.parametrize("ta,tb", TRANS)
 def test_split_k_against_oracle(gpu, oracle, ta, tb):
     """Forced piece counts on both tile shapes, every beta (1: nothing to prepare, 0: c is
@@ -81,7 +75,6 @@ def test_split_k_against_oracle(gpu, oracle, ta, tb):
         assert_fp32(c.cpu().numpy(), ref, K, mag1 + np.abs(c0) + np.abs(bias), what="split bias")
 
 
-@pytest.mark.skip(reason=SPLIT_K_OFF)
 def test_split_k_is_chosen_for_weight_gradient_shapes_and_can_be_turned_off(gpu, oracle):
     """dE/dw of a linear layer: few tiles, long k. The library's own choice (pieces) and the
     forced single piece must agree within the limit; and a batch of such products too."""
@@ -153,7 +146,7 @@ def test_colsum_with_split_k_and_without_a_product(gpu, oracle):
     M, N, K = 128, 256, 4096
     a, b = oracle.uniform((K, M), 1), oracle.uniform((K, N), 2)
     c0, s0 = oracle.uniform((M, N), 3), oracle.uniform((N,), 4)
-    for splits in ("1",):            # "8" as well once the split-k path is back on
+    for splits in ("1", "8"):
         os.environ["NTSAMD_SPLIT_K"] = splits
         for sbeta in (1.0, 0.0, 0.5):
             c, s = dev(c0, gpu), dev(s0, gpu)
