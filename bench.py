@@ -32,13 +32,18 @@ HBM_TBS = 8.0
 
 
 def configs():
-    """The five configurations of the baseline, 1-based."""
+    """The five configurations of the baseline, 1-based, and two backward steps that follow them
+    (the gradient products the reference's autograd issues for configurations 2 and 3)."""
     return {
         1: dict(name="cfg1 fp32 _MatrixMul NN 4096x512 . 512x2048", dtype="f32", M=4096, N=2048, K=512, batch=1),
         2: dict(name="cfg2 fp32 MulAndShift X[32x128x512] . W[512x2048] + b[2048]", dtype="f32", M=4096, N=2048, K=512, batch=1),
         3: dict(name="cfg3 fp32 _MatrixMulBatched Q.K^T/8 then S.V, [256x128x64]", dtype="f32", M=128, N=128, K=64, batch=256),
         4: dict(name="cfg4 fp16 _MatrixMul TN a[1024x8192]^T . b[1024x4096]", dtype="f16", M=8192, N=4096, K=1024, batch=1),
         5: dict(name="cfg5 fp32 _MatrixMul NT H[4096x512] . W[30011x512]^T + C, beta=1", dtype="f32", M=4096, N=30011, K=512, batch=1),
+        6: dict(name="cfg6 fp32 GradMulAndShift of cfg2: dX += dY.W^T (NT), dW += X^T.dY (TN) with db += colsum(dY)",
+                dtype="f32", M=4096, N=2048, K=512, batch=1),
+        7: dict(name="cfg7 fp32 GradMatrixMulBatched of cfg3 step 1: dQ += dS.K/8 (NN), dK += dS^T.Q/8 (TN), [256x128x128]",
+                dtype="f32", M=128, N=128, K=64, batch=256),
     }
 
 
@@ -94,6 +99,38 @@ class Workload:
             self.flops = 2.0 * 4096 * 30011 * 512
             self.bytes = 4.0 * (4096 * 512 + 30011 * 512 + 2 * 4096 * 30011)
             self.launches = 1
+        elif idx == 6:
+            self.x = g(oracle.uniform((4096, 512), 1))
+            self.w = g(oracle.normal((512, 2048), 2, 0, 0.02))
+            self.dy = g(oracle.normal((4096, 2048), 3))
+            self.dx = torch.zeros((4096, 512), device=dev)
+            self.dw = torch.zeros((512, 2048), device=dev)
+            self.db = torch.zeros((2048,), device=dev)
+
+            def run():
+                nt.matrix_mul(self.dy, NT, self.w, T, self.dx, 1.0, 1.0)
+                nt.matrix_mul_colsum(self.x, T, self.dy, NT, self.dw, self.db, 1.0, 1.0, 1.0)
+            self.run = run
+            self.flops = 2 * 2.0 * 4096 * 2048 * 512
+            # dX: dY, W, dX read and written; dW: X, dY, dW read and written (db is 8 KB)
+            self.bytes = 4.0 * ((4096 * 2048 + 512 * 2048 + 2 * 4096 * 512) + (4096 * 512 + 4096 * 2048 + 2 * 512 * 2048))
+            self.launches = 2
+        elif idx == 7:
+            self.q = g(oracle.normal((256, 128, 64), 1))
+            self.k = g(oracle.normal((256, 128, 64), 2))
+            self.ds = g(oracle.normal((256, 128, 128), 3))
+            self.dq = torch.zeros((256, 128, 64), device=dev)
+            self.dk = torch.zeros((256, 128, 64), device=dev)
+
+            def run():
+                nt.matrix_mul_batched_strided(self.ds, NT, self.k, NT, self.dq, 256, 16384, 8192, 8192,
+                                              128, 128, 128, 64, 128, 64, 0.125, 1.0)
+                nt.matrix_mul_batched_strided(self.ds, T, self.q, NT, self.dk, 256, 16384, 8192, 8192,
+                                              128, 128, 128, 64, 128, 64, 0.125, 1.0)
+            self.run = run
+            self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
+            self.bytes = 2 * 4.0 * 256 * (128 * 128 + 128 * 64 + 2 * 128 * 64)
+            self.launches = 2
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
@@ -132,7 +169,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9, 6: 0.75e9, 7: 2e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -142,6 +179,24 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 4.0 * 128 * 128 * 64
         sample = "%d of 256 batch items, both products" % nb
+    elif idx == 7:
+        nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
+        q, k, ds = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 128), 3)
+        dq, dk = np.zeros_like(q), np.zeros_like(k)
+        t0 = time.perf_counter()
+        o.grad_matmul_batched(q, X_NOTRANS, k, X_TRANS, ds, 0.125, dq, dk)
+        dt = time.perf_counter() - t0
+        fl = nb * 4.0 * 128 * 128 * 64
+        sample = "%d of 256 batch items, both gradient products" % nb
+    elif idx == 6:
+        rows = max(8, min(M, int(budget_s * rate / (4.0 * N * K))))
+        x, w, dy = o.uniform((rows, K), 1), o.normal((K, N), 2, 0, 0.02), o.normal((rows, N), 3)
+        dx, dw, db = np.zeros_like(x), np.zeros_like(w), np.zeros((N,), np.float32)
+        t0 = time.perf_counter()
+        o.grad_mulandshift(x, w, dy, 1, 1.0, dx, dw, db)
+        dt = time.perf_counter() - t0
+        fl = 4.0 * rows * N * K
+        sample = "%d of %d rows of x and dE/dc, all of w: both gradient products and the bias sums" % (rows, M)
     else:
         rows = max(8, min(M, int(budget_s * rate / (2.0 * N * K))))
         if idx in (1, 2):
@@ -207,7 +262,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
     # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
-    if idx == 3:
+    if idx in (3, 7):
         roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
                 "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
     else:
@@ -243,9 +298,10 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-5 (default 2, the MulAndShift linear layer)")
+    # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=500)
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-7 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -273,9 +329,10 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5):
+        for idx in (1, 3, 4, 5, 6, 7):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
-            print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else 3, dev, oracle, not args.no_cpu)), flush=True)
+            print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
+                                       not args.no_cpu)), flush=True)
     print(json.dumps(bench_one(args.config, args.steps, args.warmup, dev, oracle, not args.no_cpu)), flush=True)
 
 
