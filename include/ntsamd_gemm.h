@@ -164,6 +164,32 @@ int ntsamd_matrix_mul_batched(int devID, void * stream,
                               int count, int na, int ma, int nb, int mb, int nc, int mc,
                               float alpha, float beta);
 
+/*
+ * Attention for every head in one kernel:
+ *   out[h][b] = softmax(scale * q[h][b] * k[h][b]^T + mask[h][b]) * v[h][b],   softmax over the keys.
+ * Replaces the operator chain of the reference's Attention::MakeAttention in inference
+ * (source/sample/transformer/submodel/Attention.cpp:186-237): Split of q, k and v into
+ * heads (core/shape/Split.cpp), ScaleMe of q (:202-205), BMMul(q, X_NOTRANS, k, X_TRANS)
+ * (:208-211), SumMe with the mask (:217-222), Softmax(att, -1) (:224, function/Softmax.cu),
+ * BMMul(att, v) (:232-235) and Merge of the heads (:239, core/shape/Merge.cpp). The scores
+ * are never written to memory, and the head split and merge are addressing:
+ *   element (h, b, row, col) of q is q[h * strides[0] + b * strides[1] + row * strides[2] + col],
+ *   likewise strides[3..5] for k, [6..8] for v, [9..11] for out (in elements, multiples of 4).
+ * For tensors stored [batch][rows][heads * dh], as before Split and after Merge, the strides
+ * are (dh, rows * heads * dh, heads * dh); for tensors stored [heads][batch][rows][dh], as
+ * after Split, they are (batch * rows * dh, rows * dh, dh).
+ * q and out have lq rows, k and v have lk rows, every row has dh columns (dh a multiple of 4,
+ * at most 128). mask is NULL or a dense X_FLOAT tensor [heads][batch][lq][lk] added to the
+ * scaled scores (the reference's masks hold 0 and -1e9). dataType is X_FLOAT for q, k, v and
+ * out. The training path of the reference applies dropout between the softmax and the second
+ * product (:226-227) and keeps the probabilities for the backward step: it stays on the
+ * batched-product entry points above.
+ */
+int ntsamd_attention(int devID, void * stream,
+                     const void * q, const void * k, const void * v, const void * mask, void * out, int dataType,
+                     int heads, int batch, int lq, int lk, int dh,
+                     const long long * strides, float scale);
+
 #ifdef __cplusplus
 }
 #endif

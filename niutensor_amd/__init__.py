@@ -28,6 +28,7 @@ EXPORTS = (
     "ntsamd_matrix_mul_batched",
     "ntsamd_matrix_mul_colsum",
     "ntsamd_reduce_sum_xz",
+    "ntsamd_attention",
 )
 
 
@@ -64,6 +65,7 @@ def load():
                                             ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_colsum.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, cf]
     L.ntsamd_reduce_sum_xz.argtypes = [ci, vp, vp, ci, ci, ci, ci, vp, cf]
+    L.ntsamd_attention.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
     _lib = L
@@ -166,5 +168,29 @@ def reduce_sum_xz(t, out, beta=0.0):
     x, y, z = (int(v) for v in t.shape)
     rc = L.ntsamd_reduce_sum_xz(t.device.index, _stream_ptr(t), t.data_ptr(), _dtype_code(t), x, y, z,
                                 out.data_ptr(), beta)
+    _check(rc)
+    return out
+
+
+def attention(q, k, v, out, heads, scale, mask=None, split=False):
+    """out = softmax(scale q k^T + mask) v per head. q, k, v, out are [batch][rows][heads*dh] device
+    tensors (split=False: the layout before Split / after Merge) or [heads][batch][rows][dh] (split=True);
+    mask is None or a dense float [heads][batch][lq][lk] tensor."""
+    L = load()
+    if split:
+        _, batch, lq, dh = (int(x) for x in q.shape)
+        lk = int(k.shape[2])
+        st = lambda rows: (batch * rows * dh, rows * dh, dh)
+    else:
+        batch, lq, hd = (int(x) for x in q.shape)
+        lk = int(k.shape[1])
+        dh = hd // heads
+        st = lambda rows: (dh, rows * hd, hd)
+    for t in (q, k, v, out):
+        assert t.is_contiguous()
+    strides = (C.c_longlong * 12)(*(st(lq) + st(lk) + st(lk) + st(lq)))
+    rc = L.ntsamd_attention(q.device.index, _stream_ptr(q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                            mask.data_ptr() if mask is not None else None, out.data_ptr(), _dtype_code(q),
+                            heads, batch, lq, lk, dh, strides, scale)
     _check(rc)
     return out

@@ -24,6 +24,21 @@ int launch_f16_tn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStre
 int launch_f16_tt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
 int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
+struct AttnParams {
+    const float * q;
+    const float * k;
+    const float * v;
+    const float * mask;
+    float * out;
+    int heads, batch, lq, lk, dh;
+    long long qH, qB, qL;
+    long long kH, kB, kL;
+    long long vH, vB, vL;
+    long long oH, oB, oL;
+    float scale;
+    int qTiles;
+};
+int launch_attention_f32(const AttnParams & p, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -441,6 +456,62 @@ int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType
         return scope.status;
     int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,
                                   static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return NTSAMD_OK;
+}
+
+int ntsamd_attention(int devID, void * stream,
+                     const void * q, const void * k, const void * v, const void * mask, void * out, int dataType,
+                     int heads, int batch, int lq, int lk, int dh,
+                     const long long * strides, float scale)
+{
+    if (dataType != NTSAMD_X_FLOAT)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
+    if (heads < 0 || batch < 0 || lq < 0 || lk < 0 || dh < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
+    if (heads == 0 || batch == 0 || lq == 0 || dh == 0)
+        return NTSAMD_OK;
+    if (lk == 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "attention over no keys");
+    if (!q || !k || !v || !out || !strides)
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty input tensors!");
+    if (dh > 128 || dh % 4 != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "head size %d is not served by the fused kernel (a multiple of 4 up to 128 is)", dh);
+    for (int i = 0; i < 12; i++)
+        if (strides[i] < 0 || strides[i] % 4 != 0)
+            return fail(NTSAMD_ERR_ARGUMENT, "strides must be non-negative multiples of 4 elements");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
+        return fail(NTSAMD_ERR_ARGUMENT, "q, k, v and out must be 16-byte aligned");
+    for (int t = 0; t < 4; t++)
+        if (strides[3 * t + 2] < dh)
+            return fail(NTSAMD_ERR_ARGUMENT, "row stride smaller than the head size");
+    if ((long long)heads * batch * ((lq + 127) / 128) > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
+    int st = check_device(devID);
+    if (st != NTSAMD_OK)
+        return st;
+    DeviceScope scope(devID);
+    if (scope.status != NTSAMD_OK)
+        return scope.status;
+    AttnParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = static_cast<const float *>(q);
+    p.k = static_cast<const float *>(k);
+    p.v = static_cast<const float *>(v);
+    p.mask = static_cast<const float *>(mask);
+    p.out = static_cast<float *>(out);
+    p.heads = heads;
+    p.batch = batch;
+    p.lq = lq;
+    p.lk = lk;
+    p.dh = dh;
+    p.qH = strides[0]; p.qB = strides[1]; p.qL = strides[2];
+    p.kH = strides[3]; p.kB = strides[4]; p.kL = strides[5];
+    p.vH = strides[6]; p.vB = strides[7]; p.vL = strides[8];
+    p.oH = strides[9]; p.oB = strides[10]; p.oL = strides[11];
+    p.scale = scale;
+    int rc = launch_attention_f32(p, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

@@ -80,6 +80,10 @@ class Oracle:
         L.oracle_grad_mulandshift.argtypes = [_fp, _fp, C.c_int, _ip, C.c_int, _fp, _fp, C.c_int, _ip, C.c_int,
                                               _fp, C.c_int, _fp, _ip, C.c_int, C.c_int, C.c_float]
         L.oracle_grad_mulandshift.restype = C.c_int
+        L.oracle_softmax.argtypes = [_fp, C.c_long, C.c_int, _fp]
+        L.oracle_softmax.restype = C.c_int
+        L.oracle_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
+        L.oracle_attention.restype = C.c_int
         L.oracle_is_float_equal.argtypes = [C.c_float] * 4
         L.oracle_is_float_equal.restype = C.c_int
         L.oracle_check_data.argtypes = [_fp, _fp, C.c_int, C.c_float]
@@ -187,6 +191,23 @@ class Oracle:
             raise ValueError("TODO!" if r == -2 else "Wrong tensor size!")
         return dedx, dedw, dedbias
 
+    # -- attention ---------------------------------------------------------
+    def softmax(self, x):
+        y = np.empty_like(x)
+        if self.lib.oracle_softmax(_f(x), x.size // x.shape[-1], x.shape[-1], _f(y)) != 0:
+            raise ValueError("empty softmax")
+        return y
+
+    def attention(self, q, k, v, heads, scale, mask=None):
+        """q [batch][lq][hidden], k and v [batch][lk][hidden], mask None or [heads][batch][lq][lk]."""
+        batch, lq, hidden = q.shape
+        out = np.zeros_like(q)
+        r = self.lib.oracle_attention(_f(q), _f(k), _f(v), _f(mask) if mask is not None else None, _f(out),
+                                      batch, lq, k.shape[1], hidden, heads, scale)
+        if r != 0:
+            raise ValueError("Unmatched tensors in attention")
+        return out
+
     def is_float_equal(self, a, b, abs_err, rel_err=1e-4):
         return bool(self.lib.oracle_is_float_equal(a, b, abs_err, rel_err))
 
@@ -241,6 +262,8 @@ class Reference:
                                       _fp, _ip, C.c_int, _fp, _ip, C.c_float]
         L.ref_enum_values.argtypes = [_ip]
         L.ref_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.ref_softmax.argtypes = [_fp, _ip, C.c_int, _fp]
+        L.ref_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.ref_grad.argtypes = [C.c_int, _fp, _ip, C.c_int, C.c_int, _fp, _ip, C.c_int, C.c_int,
                                _fp, _ip, C.c_int, C.c_float, _fp, _fp, _fp, _fp]
 
@@ -307,6 +330,18 @@ class Reference:
                           _dims(bias.shape) if bias is not None else None, 0 if bias is None else bias.ndim,
                           alpha, _f(dedc), _f(deda), _f(dedb), _f(dedbias) if dedbias is not None else None)
         return deda, dedb, dedbias
+
+    def softmax(self, x):
+        y = np.empty_like(x)
+        self.lib.ref_softmax(_f(x), _dims(x.shape), x.ndim, _f(y))
+        return y
+
+    def attention(self, q, k, v, heads, scale, mask=None):
+        batch, lq, hidden = q.shape
+        out = np.zeros_like(q)
+        self.lib.ref_attention(_f(q), _f(k), _f(v), _f(mask) if mask is not None else None, _f(out),
+                               batch, lq, k.shape[1], hidden, heads, scale)
+        return out
 
     def run_matmul_tests(self):
         return self.lib.ref_run_matmul_tests()

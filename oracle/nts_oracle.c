@@ -571,6 +571,120 @@ int oracle_grad_mulandshift(const float *x, float *dedx, int transX, const int *
     return oracle_grad_matmul(x, dedx, transX, xDims, xOrder, w, dedw, transW, wDims, wOrder, dedc, alpha);
 }
 
+/* ---- attention: the operator chain of the transformer sample -------------------- */
+
+int oracle_softmax(const float *x, long rows, int n, float *y)
+{
+    if (n <= 0)
+        return -1;
+    for (long i = 0; i < rows; i++) {
+        const float *ip = x + i * n;
+        float *op = y + i * n;
+        /* _ReduceMax over the row (ReduceMax.cpp): the maximum does not depend on the order */
+        float mx = ip[0];
+        for (int j = 1; j < n; j++)
+            mx = ip[j] > mx ? ip[j] : mx;
+        /* _ReduceSum(x, sum, leadDim, max, 1.0F, true): sum of (DTYPE)exp(x - max), in the
+           order of ReduceSum.cpp. Which exp runs depends on the file: ReduceSum.cpp and Softmax.cpp call
+           exp on a float and get C++'s float overload; VectorBuffer.cpp (the 32-lane path) gets the
+           double one and rounds the result to float (both established against the compiled reference): 32 running sums folded at the end when the row length is a
+           multiple of 32 (:83-116), one running sum from 0 otherwise (:146-228) */
+        float sum;
+        if (n % 32 == 0 && n >= 32) {
+            float buf[4][8];
+            for (int k = 0; k < 4; k++)
+                for (int l = 0; l < 8; l++)
+                    buf[k][l] = (float)exp(ip[k * 8 + l] - mx);
+            for (int j = 1; j < n / 32; j++)
+                for (int k = 0; k < 4; k++)
+                    for (int l = 0; l < 8; l++)
+                        buf[k][l] = (float)exp(ip[j * 32 + k * 8 + l] - mx) + buf[k][l];
+            sum = 0.0F;
+            for (int l = 0; l < 8; l++) {
+                float b01 = buf[1][l] + buf[0][l];
+                float b23 = buf[3][l] + buf[2][l];
+                sum = sum + (b23 + b01);
+            }
+        }
+        else {
+            sum = 0;
+            for (int j = 0; j < n; j++)
+                sum += expf(ip[j] - mx);
+        }
+        /* Softmax.cpp:92-109 */
+        if (sum == 0) {
+            for (int j = 0; j < n; j++)
+                op[j] = 0;
+        }
+        else {
+            for (int j = 0; j < n; j++) {
+                float r = expf(ip[j] - mx) / sum;
+                if (r > 1.0F)
+                    r = 1.0F;
+                else if (r < 0)
+                    r = 0;
+                op[j] = r;
+            }
+        }
+    }
+    return 0;
+}
+
+int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
+                     int batch, int lq, int lk, int hidden, int heads, float scale)
+{
+    if (heads <= 0 || hidden % heads != 0)
+        return -1;
+    const int dh = hidden / heads;
+    const long nq = (long)heads * batch * lq * dh, nk = (long)heads * batch * lk * dh;
+    const long na = (long)heads * batch * lq * lk;
+    float *qh = (float *)malloc(sizeof(float) * (size_t)(nq > 0 ? nq : 1));
+    float *kh = (float *)malloc(sizeof(float) * (size_t)(nk > 0 ? nk : 1));
+    float *vh = (float *)malloc(sizeof(float) * (size_t)(nk > 0 ? nk : 1));
+    float *att = (float *)malloc(sizeof(float) * (size_t)(na > 0 ? na : 1));
+    float *prob = (float *)malloc(sizeof(float) * (size_t)(na > 0 ? na : 1));
+    float *oh = (float *)malloc(sizeof(float) * (size_t)(nq > 0 ? nq : 1));
+    int r = -1;
+    if (qh && kh && vh && att && prob && oh) {
+        /* Attention.cpp:194-198: Split(x, order - 1, nhead): head h takes columns h*dh .. of every row
+           and becomes block h of a [heads][batch][rows][dh] tensor (Split.cpp) */
+        for (int h = 0; h < heads; h++)
+            for (int b = 0; b < batch; b++) {
+                for (int l = 0; l < lq; l++)
+                    for (int j = 0; j < dh; j++)
+                        /* :202-205 Scale / ScaleMe of q: v * scale + 0 (ScaleAndShift.cpp:70-75) */
+                        qh[(((long)h * batch + b) * lq + l) * dh + j] = q[((long)b * lq + l) * hidden + h * dh + j] * scale + 0.0F;
+                for (int l = 0; l < lk; l++)
+                    for (int j = 0; j < dh; j++) {
+                        kh[(((long)h * batch + b) * lk + l) * dh + j] = k[((long)b * lk + l) * hidden + h * dh + j];
+                        vh[(((long)h * batch + b) * lk + l) * dh + j] = v[((long)b * lk + l) * hidden + h * dh + j];
+                    }
+            }
+        int dq[4] = {heads, batch, lq, dh}, dk[4] = {heads, batch, lk, dh}, da[4] = {heads, batch, lq, lk};
+        /* :208-211 BMMul(q, X_NOTRANS, kheads, X_TRANS) */
+        r = oracle_matmul_batched(qh, ORACLE_X_NOTRANS, dq, kh, ORACLE_X_TRANS, dk, att, da, 4, 1.0F, 0.0F);
+        /* :217-222 Sum / SumMe with the mask: c = a + b */
+        if (r == 0 && mask)
+            for (long i = 0; i < na; i++)
+                att[i] = att[i] + mask[i];
+        /* :224 Softmax(att, -1) */
+        if (r == 0)
+            r = oracle_softmax(att, (long)heads * batch * lq, lk, prob);
+        /* :232-235 BMMul(att, vheads) */
+        if (r == 0)
+            r = oracle_matmul_batched(prob, ORACLE_X_NOTRANS, da, vh, ORACLE_X_NOTRANS, dk, oh, dq, 4, 1.0F, 0.0F);
+        /* :239 Merge(att, order - 1): block h goes back to columns h*dh .. (Merge.cpp) */
+        if (r == 0)
+            for (int h = 0; h < heads; h++)
+                for (int b = 0; b < batch; b++)
+                    for (int l = 0; l < lq; l++)
+                        for (int j = 0; j < dh; j++)
+                            out[((long)b * lq + l) * hidden + h * dh + j] = oh[(((long)h * batch + b) * lq + l) * dh + j];
+    }
+    free(qh); free(kh); free(vh); free(att); free(prob); free(oh);
+    return r;
+}
+
 /* ---- comparator ---------------------------------------------------------- */
 
 int oracle_is_float_equal(float a, float b, float absError, float relError)

@@ -91,6 +91,18 @@ int oracle_grad_mulandshift(const float *x, float *dedx, int transX, const int *
                             float *dedbias, int biasNum,
                             const float *dedc, const int *cDims, int cOrder, int n, float alpha);
 
+/* y = softmax over the last dimension of a [rows][n] tensor: the CPU branch of
+   source/tensor/function/Softmax.cpp:38-117 with its _ReduceMax and its
+   _ReduceSum(x, sum, dim, max, 1, true), sums in the reference's order. */
+int oracle_softmax(const float *x, long rows, int n, float *y);
+
+/* The inference path of Attention::MakeAttention (source/sample/transformer/submodel/
+   Attention.cpp:186-239) on q [batch][lq][hidden], k and v [batch][lk][hidden], mask NULL or
+   [heads][batch][lq][lk]: Split into heads, scale q, BMMul(q, k^T), add the mask, Softmax,
+   BMMul with v, Merge. out is [batch][lq][hidden]. */
+int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
+                     int batch, int lq, int lk, int hidden, int heads, float scale);
+
 /* comparator of the reference tests, CheckData.cpp:29-39 */
 int oracle_is_float_equal(float a, float b, float absError, float relError);
 /* CheckData.cpp:78-97 with its fixed relative bound 1e-4 */

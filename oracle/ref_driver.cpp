@@ -19,6 +19,7 @@
 #include "test/TMatrixMulBatched.h"
 #include "test/TSumDim.h"
 #include "../network/XBackwardMath.h"
+#include "function/FHeader.h"
 
 #include <string.h>
 
@@ -197,6 +198,49 @@ int ref_grad(int kind,
         delete tbias;
     X_ENABLE_GRAD = backup;
     return order;
+}
+
+int ref_softmax(const float * x, const int * dims, int order, float * y)
+{
+    XTensor * tx = Make(dims, order, x);
+    XTensor * ty = Make(dims, order, NULL);
+    _Softmax(tx, ty, order - 1);
+    memcpy(y, ty->data, sizeof(float) * (size_t)ty->unitNum);
+    delete tx; delete ty;
+    return 0;
+}
+
+/* the operator chain of Attention::MakeAttention in inference, with the reference's own operators:
+   q [batch][lq][hidden], k, v [batch][lk][hidden], mask NULL or [heads][batch][lq][lk] */
+int ref_attention(const float * q, const float * k, const float * v, const float * mask, float * out,
+                  int batch, int lq, int lk, int hidden, int heads, float scale)
+{
+    int dq[3] = {batch, lq, hidden}, dk[3] = {batch, lk, hidden}, dm[4] = {heads, batch, lq, lk};
+    XTensor * tq = Make(dq, 3, q);
+    XTensor * tk = Make(dk, 3, k);
+    XTensor * tv = Make(dk, 3, v);
+    XTensor * tm = mask != NULL ? Make(dm, 4, mask) : NULL;
+    /* inference: no autograd edges, as the sample's translator runs it (DISABLE_GRAD) */
+    bool backup = X_ENABLE_GRAD;
+    X_ENABLE_GRAD = false;
+    {
+        XTensor qh = Split(*tq, 2, heads);
+        XTensor kh = Split(*tk, 2, heads);
+        XTensor vh = Split(*tv, 2, heads);
+        ScaleAndShiftMe(qh, scale, 0.0F);
+        XTensor att = BMMul(qh, X_NOTRANS, kh, X_TRANS);
+        if (tm != NULL)
+            SumMe(att, *tm);
+        att = Softmax(att, -1);
+        att = BMMul(att, vh);
+        XTensor merged = Merge(att, att.order - 1);
+        memcpy(out, merged.data, sizeof(float) * (size_t)merged.unitNum);
+    }
+    delete tq; delete tk; delete tv;
+    if (tm != NULL)
+        delete tm;
+    X_ENABLE_GRAD = backup;
+    return 0;
 }
 
 /* the reference's own known-answer tests for this path; bit i set = suite i passed */

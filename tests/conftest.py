@@ -64,6 +64,12 @@ def generated_backward():
 
 
 @pytest.fixture(scope="session")
+def generated_attention():
+    """tests/golden/ref_generated_attention.npz: the compiled reference's softmax and attention chain."""
+    return Generated("ref_generated_attention.npz")
+
+
+@pytest.fixture(scope="session")
 def gpu():
     """cuda:0 with the HIP library loaded. No fallback: a missing library is an error."""
     import torch

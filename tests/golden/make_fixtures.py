@@ -200,6 +200,54 @@ def backward():
     print("wrote", path, len(index), "cases", os.path.getsize(path), "bytes")
 
 
+def attention():
+    o = Oracle()
+    r = Reference()
+    out = {}
+    index = []
+
+    def put(name, **arrays):
+        index.append(name)
+        for k, v in arrays.items():
+            out["%s/%s" % (name, k)] = np.asarray(v)
+
+    seed = 9000
+    # _Softmax over the last dimension: scalar sums, 32-lane sums, a constant row, large magnitudes
+    for i, (shape, std) in enumerate([((5, 7), 1.0), ((3, 32), 3.0), ((4, 96), 3.0), ((2, 3, 40), 1.0), ((6, 128), 0.5),
+                                      ((2, 1), 1.0), ((3, 33), 30.0), ((2, 64), 0.0)]):
+        seed += 1
+        x = o.normal(shape, seed, 0.0, std) if std > 0 else np.full(shape, 2.5, np.float32)
+        put("softmax_%d" % i, kind="softmax", x=x, y=r.softmax(x))
+
+    # attention: (batch, lq, lk, hidden, heads, masked)
+    cases = [(2, 5, 7, 8, 2, 0), (2, 9, 9, 16, 4, 1), (3, 33, 64, 32, 2, 1), (1, 40, 32, 24, 3, 0), (2, 64, 100, 128, 2, 1),
+             (1, 130, 200, 64, 1, 1), (2, 16, 300, 96, 1, 0), (1, 1, 1, 4, 1, 0), (2, 20, 50, 256, 2, 2)]
+    for i, (B, lq, lk, H, nh, masked) in enumerate(cases):
+        seed += 4
+        q, k, v = o.normal((B, lq, H), seed), o.normal((B, lk, H), seed + 1), o.normal((B, lk, H), seed + 2)
+        mask = None
+        if masked == 1:
+            # the sample's masks hold 0 and -1e9 (Model.cpp:249-258, 310-337)
+            mask = np.where(o.uniform((nh, B, lq, lk), seed + 3, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+            mask[..., 0] = 0.0                                  # every row keeps one key
+        elif masked == 2:
+            # causal: row i sees keys 0..i
+            mask = np.broadcast_to(np.where(np.arange(lk)[None, :] > np.arange(lq)[:, None], -1e9, 0.0),
+                                   (nh, B, lq, lk)).astype(np.float32).copy()
+        scale = float(np.float32(1.0 / np.sqrt(H / nh)))
+        y = r.attention(q, k, v, nh, scale, mask)
+        arrays = dict(kind="attention", q=q, k=k, v=v, out=y, params=[nh], scal=[scale])
+        if mask is not None:
+            arrays["mask"] = mask
+        put("attention_%d" % i, **arrays)
+
+    out["index"] = np.array(index)
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_generated_attention.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, len(index), "cases", os.path.getsize(path), "bytes")
+
+
 if __name__ == "__main__":
     main()
     backward()
+    attention()

@@ -1,0 +1,140 @@
+"""Parity of the one-kernel attention (ntsamd_attention) with the CPU oracle's restatement of
+the reference's operator chain (Split, Scale, BMMul(q, k^T), Sum with the mask, Softmax,
+BMMul with v, Merge), through the C ABI.
+
+Limit: fp32, normwise error at most 1e-5 sqrt(K) with K = dh + lk (the two contractions a
+result element passes through); the probabilities come from expf on both sides.
+"""
+import numpy as np
+import pytest
+
+import niutensor_amd as nt
+from tolerance import assert_fp32
+
+pytestmark = pytest.mark.gpu
+
+
+def torch_():
+    import torch
+    return torch
+
+
+def dev(x, gpu):
+    return torch_().from_numpy(np.ascontiguousarray(x)).to(gpu)
+
+
+@pytest.fixture(autouse=True)
+def name_the_case(request):
+    print("\n[gpu-case] %s" % request.node.nodeid, flush=True)
+    yield
+
+
+def run(gpu, q, k, v, heads, scale, mask=None):
+    torch = torch_()
+    out = torch.full(q.shape, float("nan"), device=gpu)
+    nt.attention(dev(q, gpu), dev(k, gpu), dev(v, gpu), out, heads, scale, mask=dev(mask, gpu) if mask is not None else None)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def test_fixtures_of_the_compiled_reference(gpu, generated_attention):
+    names = generated_attention.of_kind("attention")
+    assert len(names) == 9
+    for name in names:
+        d = generated_attention.case(name)
+        heads, scale = int(d["params"][0]), float(d["scal"][0])
+        dh = d["q"].shape[2] // heads
+        if dh % 4 != 0 or dh > 128:
+            pytest.fail("fixture %s has a head size the kernel refuses" % name)
+        got = run(gpu, d["q"], d["k"], d["v"], heads, scale, d.get("mask"))
+        assert_fp32(got, d["out"], dh + d["k"].shape[1], what=name)
+
+
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
+    (2, 128, 128, 128, 2, False),      # one key block, head size 64
+    (3, 100, 77, 96, 3, True),         # ragged rows and keys, head size 32
+    (1, 300, 513, 64, 1, True),        # several query tiles and key blocks
+    (2, 40, 260, 256, 2, False),       # head size 128
+    (2, 33, 65, 192, 2, True),         # head size 96 inside the 128 kernel
+    (4, 9, 5, 8, 2, False),            # head size 4
+    (1, 1, 1, 12, 1, False),           # a single score
+])
+def test_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
+    q, k, v = oracle.normal((B, lq, H), 11), oracle.normal((B, lk, H), 12), oracle.normal((B, lk, H), 13)
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 14, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., lk // 2] = 0.0
+    scale = float(np.float32(1.0 / np.sqrt(H // nh)))
+    ref = oracle.attention(q, k, v, nh, scale, mask)
+    got = run(gpu, q, k, v, nh, scale, mask)
+    assert_fp32(got, ref, H // nh + lk, what=str((B, lq, lk, H, nh, masked)))
+
+
+def test_rows_with_every_key_masked_and_large_scores(gpu, oracle):
+    """A row whose mask is -1e9 everywhere comes out as the mean of v (scores below 32 vanish
+    beside -1e9 in fp32, on both sides); scores of a few hundred do not overflow."""
+    B, lq, lk, H, nh = 1, 70, 140, 64, 2
+    q, k, v = oracle.normal((B, lq, H), 21), oracle.normal((B, lk, H), 22), oracle.normal((B, lk, H), 23)
+    mask = np.zeros((nh, B, lq, lk), np.float32)
+    mask[:, :, 3, :] = -1e9
+    mask[:, :, 69, 1:] = -1e9
+    ref = oracle.attention(q, k, v, nh, 0.5, mask)
+    got = run(gpu, q, k, v, nh, 0.5, mask)
+    assert_fp32(got, ref, 32 + lk, what="masked rows")
+    assert np.abs(got[0, 3] - v[0].mean(0)).max() <= 1e-5
+    assert np.array_equal(got[0, 69], v[0, 0])
+    q, k = oracle.normal((B, lq, H), 24, 0.0, 3.0), oracle.normal((B, lk, H), 25, 0.0, 3.0)
+    ref = oracle.attention(q, k, v, nh, 1.0)
+    got = run(gpu, q, k, v, nh, 1.0)
+    assert_fp32(got, ref, 32 + lk, what="large scores")
+
+
+def test_split_layout_and_stream(gpu, oracle):
+    """Tensors stored [heads][batch][rows][dh], as after the reference's Split, on a stream of the
+    caller: same numbers as the merged layout."""
+    torch = torch_()
+    B, lq, lk, H, nh = 3, 50, 70, 64, 4
+    dh = H // nh
+    q, k, v = oracle.normal((B, lq, H), 31), oracle.normal((B, lk, H), 32), oracle.normal((B, lk, H), 33)
+    ref = oracle.attention(q, k, v, nh, 0.25)
+    sp = lambda x: np.ascontiguousarray(x.reshape(x.shape[0], x.shape[1], nh, dh).transpose(2, 0, 1, 3))
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        qd, kd, vd = dev(sp(q), gpu), dev(sp(k), gpu), dev(sp(v), gpu)
+        out = torch.full((nh, B, lq, dh), float("nan"), device=gpu)
+        nt.attention(qd, kd, vd, out, nh, 0.25, split=True)
+    s.synchronize()
+    got = out.cpu().numpy().transpose(1, 2, 0, 3).reshape(B, lq, H)
+    assert_fp32(got, ref, dh + lk, what="split layout")
+
+
+def test_attention_shape_of_the_benchmark(gpu, oracle):
+    """32 sentences x 8 heads, 128 positions, head size 64: against the oracle, and against the
+    two batched products with torch's softmax between them."""
+    torch = torch_()
+    B, L, H, nh = 32, 128, 512, 8
+    q, k, v = oracle.normal((B, L, H), 41), oracle.normal((B, L, H), 42), oracle.normal((B, L, H), 43)
+    ref = oracle.attention(q, k, v, nh, 0.125)
+    got = run(gpu, q, k, v, nh, 0.125)
+    assert_fp32(got, ref, 64 + L, what="benchmark shape")
+    # properties at full size: rows of v all equal -> the output repeats that row exactly enough
+    vc = np.broadcast_to(oracle.normal((B, 1, H), 44), (B, L, H)).copy()
+    got = run(gpu, q, k, vc, nh, 0.125)
+    assert np.abs(got - vc).max() <= 1e-5 * np.abs(vc).max() * 4
+
+
+def test_bad_arguments_are_refused(gpu):
+    torch = torch_()
+    L = nt.load()
+    import ctypes as C
+    t = torch.zeros(4096, device=gpu)
+    st = (C.c_longlong * 12)(*([8, 64, 8] * 4))
+    p = t.data_ptr()
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 3, 1, 1, 8, 8, 8, st, 1.0) == 2           # fp16: not served
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 6, st, 1.0) != 0           # head size 6
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 132, st, 1.0) != 0         # head size 132
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 0, 8, st, 1.0) != 0           # no keys
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 0, 1, 8, 8, 8, st, 1.0) == 0           # nothing to do
+    bad = (C.c_longlong * 12)(*([8, 64, 6] * 4))
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 8, bad, 1.0) != 0          # unaligned rows
