@@ -32,8 +32,9 @@ HBM_TBS = 8.0
 
 
 def configs():
-    """The five configurations of the baseline, 1-based, and two backward steps that follow them
-    (the gradient products the reference's autograd issues for configurations 2 and 3)."""
+    """The five configurations of the baseline, 1-based, two backward steps that follow them
+    (the gradient products the reference's autograd issues for configurations 2 and 3), and the
+    attention of configuration 3 as one kernel."""
     return {
         1: dict(name="cfg1 fp32 _MatrixMul NN 4096x512 . 512x2048", dtype="f32", M=4096, N=2048, K=512, batch=1),
         2: dict(name="cfg2 fp32 MulAndShift X[32x128x512] . W[512x2048] + b[2048]", dtype="f32", M=4096, N=2048, K=512, batch=1),
@@ -43,6 +44,9 @@ def configs():
         6: dict(name="cfg6 fp32 GradMulAndShift of cfg2: dX += dY.W^T (NT), dW += X^T.dY (TN) with db += colsum(dY)",
                 dtype="f32", M=4096, N=2048, K=512, batch=1),
         7: dict(name="cfg7 fp32 GradMatrixMulBatched of cfg3 step 1: dQ += dS.K/8 (NN), dK += dS^T.Q/8 (TN), [256x128x128]",
+                dtype="f32", M=128, N=128, K=64, batch=256),
+        8: dict(name="cfg8 fp32 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v [32x128x512], 8 heads (cfg3 with the "
+                     "softmax between its products and the head split/merge folded in)",
                 dtype="f32", M=128, N=128, K=64, batch=256),
     }
 
@@ -131,6 +135,16 @@ class Workload:
             self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
             self.bytes = 2 * 4.0 * 256 * (128 * 128 + 128 * 64 + 2 * 128 * 64)
             self.launches = 2
+        elif idx == 8:
+            self.q = g(oracle.normal((32, 128, 512), 1))
+            self.k = g(oracle.normal((32, 128, 512), 2))
+            self.v = g(oracle.normal((32, 128, 512), 3))
+            self.o = torch.empty((32, 128, 512), device=dev)
+            self.run = lambda: nt.attention(self.q, self.k, self.v, self.o, 8, 0.125)
+            self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
+            # q, k, v read once, the result written once; the scores never reach memory
+            self.bytes = 4 * 4.0 * 32 * 128 * 512
+            self.launches = 1
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
@@ -169,7 +183,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9, 6: 0.75e9, 7: 2e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -179,6 +193,14 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 4.0 * 128 * 128 * 64
         sample = "%d of 256 batch items, both products" % nb
+    elif idx == 8:
+        nb = max(1, min(32, int(budget_s * rate / (8 * 4.0 * 128 * 128 * 64))))
+        q, k, v = o.normal((nb, 128, 512), 1), o.normal((nb, 128, 512), 2), o.normal((nb, 128, 512), 3)
+        t0 = time.perf_counter()
+        o.attention(q, k, v, 8, 0.125)
+        dt = time.perf_counter() - t0
+        fl = nb * 8 * 4.0 * 128 * 128 * 64
+        sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax, product, merge" % nb
     elif idx == 7:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, ds = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 128), 3)
@@ -301,7 +323,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-7 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-8 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 the one-kernel attention)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -329,7 +351,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7):
+        for idx in (1, 3, 4, 5, 6, 7, 8):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

@@ -1,0 +1,28 @@
+/*
+ * Problem descriptor of the one-kernel attention (attention_f32.hip), shared with
+ * the C ABI (ntsamd_capi.hip).
+ */
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace ntsamd {
+
+struct AttnParams {
+    const float * q;
+    const float * k;
+    const float * v;
+    const float * mask;                 /* NULL, or dense [heads][batch][lq][lk] added to the scaled scores */
+    float * out;
+    int heads, batch, lq, lk, dh;
+    long long qH, qB, qL;               /* element strides: head, batch item, row (columns are contiguous) */
+    long long kH, kB, kL;
+    long long vH, vB, vL;
+    long long oH, oB, oL;
+    float scale;
+    int qTiles;                         /* filled in by the launcher */
+    int maskVec;                        /* filled in by the launcher: 16-byte mask loads are possible */
+};
+
+int launch_attention_f32(const AttnParams & p, hipStream_t stream);
+
+}  // namespace ntsamd

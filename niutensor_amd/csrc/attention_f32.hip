@@ -5,82 +5,74 @@
  * (source/sample/transformer/submodel/Attention.cpp:186-237): Split of q, k, v
  * into heads, Scale of q, BMMul(q, k^T), Sum with the mask, Softmax over the
  * last dimension, BMMul with v, Merge of the heads. Here the head split and
- * merge are strides, and the scores never leave the CU: per workgroup 128 query
- * rows of one (head, batch item), one wave per 32 rows; the keys stream through
- * LDS in blocks; row maxima and sums are carried along and the running result
- * is rescaled when a later block raises a row's maximum, so any number of keys
- * is handled with one pass over k and v.
+ * merge are strides and the scores never leave the registers.
  *
- * MFMA v_mfma_f32_32x32x2_f32 twice per key block:
- *   scores  = Q (rows x dh, fragments held in registers for the whole kernel)
- *             times the key block (K-contiguous rows in LDS),
- *   result += P (the wave's 32 x KB probabilities, turned through the wave's own
- *             piece of LDS from accumulator layout to operand layout) times the
- *             value block (rows of keys in LDS).
- * Accumulator register r of lane l is element (8*(r/4) + 4*(l/32) + r%4, l%32) of a
- * 32x32 block: a lane holds ONE key column of 16 rows, so a row's maximum and sum are
- * a butterfly over the 32 lanes of a half-wave, after which every lane of the half
- * knows them.
+ * Work split: a workgroup of 4 waves takes 64 query rows of one (head, batch
+ * item), 16 rows per wave; two workgroups share a CU, so each SIMD holds two
+ * waves and one wave's softmax arithmetic runs under the other's MFMAs. Keys
+ * and values stream through LDS in blocks of KB keys; row maxima and sums are
+ * carried from block to block and the running result is rescaled when a later
+ * block raises a row's maximum, so any number of keys takes one pass over k, v.
+ *
+ * Both products are computed TRANSPOSED with v_mfma_f32_16x16x4_f32
+ * (D = A B + C, A: lane l holds A[l%16][l/16], B: lane l holds B[l/16][l%16],
+ * D: register r of lane l holds D[4*(l/16) + r][l%16]):
+ *   S^T = K Q^T   A = key block from LDS (one 16-byte read feeds four steps),
+ *                 B = Q fragments, in registers for the whole kernel;
+ *                 lane (m, g) = (l%16, l/16) ends up with the scores of query m
+ *                 against keys 16 j + 4 g + r of every 16-key block j.
+ *   O^T = V^T P^T B = P^T: lane (m, g) must supply, for query m, one key per
+ *                 step out of its group g - which is exactly a score register
+ *                 it already holds (the order in which a sum runs over the keys
+ *                 is free), A = value rows from LDS.
+ * So the probabilities go from accumulator to operand without any exchange, a
+ * query row's maximum and sum are reductions inside a lane plus two cross-lane
+ * steps (lanes m, m+16, m+32, m+48), and every per-row quantity is one register.
  */
 #include "gemm_common.h"
 #include "gemm_f32.h"
+#include "attention.h"
 
 namespace ntsamd {
 
-struct AttnParams {
-    const float * q;
-    const float * k;
-    const float * v;
-    const float * mask;                 /* NULL, or dense [heads][batch][lq][lk] added to the scaled scores */
-    float * out;
-    int heads, batch, lq, lk, dh;
-    long long qH, qB, qL;               /* element strides: head, batch item, row (columns are contiguous) */
-    long long kH, kB, kL;
-    long long vH, vB, vL;
-    long long oH, oB, oL;
-    float scale;
-    int qTiles;
-};
-
-__device__ __forceinline__ float half_wave_max(float x)
+__device__ __forceinline__ float across_groups_max(float x)
 {
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1)
-        x = fmaxf(x, __shfl_xor(x, m));
-    return x;
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
 }
 
-__device__ __forceinline__ float half_wave_sum(float x)
+__device__ __forceinline__ float across_groups_sum(float x)
 {
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1)
-        x += __shfl_xor(x, m);
-    return x;
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
 }
 
-/* DHM: head size the kernel is built for (dh <= DHM, columns past dh are zero);
+/* DHM: head size the kernel is built for (dh <= DHM; columns past dh are zero in LDS and in the
+   q fragments, and are multiplied like the others: the launcher picks the smallest DHM that holds dh);
    KB: keys per block */
 template <int DHM, int KB>
-__global__ void __launch_bounds__(256, 1)
+__global__ void __launch_bounds__(256, 2)
 attention_f32_kernel(const AttnParams p)
 {
-    constexpr int KP = DHM + 4;          /* row pitch of the key and value blocks, floats */
-    constexpr int PP = KB + 4;           /* row pitch of a wave's probabilities */
-    constexpr int NQ = DHM / 8;          /* groups of four MFMA steps over dh */
-    constexpr int NJ = KB / 32;          /* 32-key blocks of scores per wave */
-    constexpr int NO = DHM / 32;         /* 32-column blocks of the result per wave */
+    constexpr int KP = DHM + 4;          /* row pitch of the key and value blocks in floats: 4 mod 64, so the 16-byte
+                                            reads of 16 consecutive rows and the 4-byte reads of rows 4 apart spread
+                                            over all banks */
+    constexpr int NT = DHM / 16;         /* groups of four MFMA steps over dh; also 16-column blocks of the result */
+    constexpr int NJ = KB / 16;          /* 16-key blocks */
     constexpr int LOADS = KB * DHM / 4 / 256;
+    constexpr float LOG2E = 1.4426950408889634f;
 
     __shared__ __attribute__((aligned(16))) float Ks[KB * KP];
     __shared__ __attribute__((aligned(16))) float Vs[KB * KP];
-    __shared__ __attribute__((aligned(16))) float Ps[4 * 32 * PP];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, lh = lane >> 5;
+    const int m = lane & 15, g = lane >> 4;
 
-    const int qt = (int)blockIdx.x % p.qTiles;
-    const int pair = (int)blockIdx.x / p.qTiles;
+    /* workgroups of one (head, batch item) are neighbours on one XCD: they share k and v in its L2 */
+    const int id = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int qt = id % p.qTiles;
+    const int pair = id / p.qTiles;
     const int h = pair / p.batch, b = pair - h * p.batch;
     const int lq = p.lq, lk = p.lk, dh = p.dh;
 
@@ -88,173 +80,202 @@ attention_f32_kernel(const AttnParams p)
     const float * K = p.k + h * p.kH + b * p.kB;
     const float * V = p.v + h * p.vH + b * p.vB;
     float * O = p.out + h * p.oH + b * p.oB;
-    const float * MK = p.mask ? p.mask + ((long long)pair * lq) * lk : nullptr;
 
-    const int row0 = qt * 128 + wave * 32;          /* first query row of this wave */
+    const int row = qt * 64 + wave * 16 + m;              /* this lane's query row */
+    const int rowc = row < lq ? row : lq - 1;             /* rows past the end repeat the last one; never stored */
+    const float * MK = p.mask ? p.mask + ((long long)pair * lq + rowc) * lk : nullptr;
 
-    /* ---- Q fragments: lane (l32, lh) feeds row l32, k = 8 g + 4 lh + e of group g ---- */
-    f32x4 qf[NQ];
-    {
-        int r = row0 + l32;
-        r = r < lq ? r : lq - 1;                    /* rows past the end repeat the last one; never stored */
-        const float * qr = Q + (long long)r * p.qL;
+    /* ---- key / value staging: 16 bytes per thread and step through buffer loads whose descriptor ends
+       with the last key, so keys past lk read as zero; columns past dh get an offset outside every
+       descriptor. A thread's column never changes, its rows are RSTEP apart from step to step. ---- */
+    constexpr int TPR = DHM / 4;         /* threads per row */
+    constexpr int RSTEP = 256 / TPR;     /* rows per step */
+    const int sr0 = tid / TPR, sc = (tid % TPR) * 4;
+    const int sLds = sr0 * KP + sc;
+    const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K, ((long long)(lk - 1) * p.kL + dh) * 4);
+    const __amdgpu_buffer_rsrc_t vRsrc = make_rsrc(V, ((long long)(lk - 1) * p.vL + dh) * 4);
+    const int kL4 = (int)p.kL * 4, vL4 = (int)p.vL * 4;
+    const int kOff0 = sc < dh ? sr0 * kL4 + sc * 4 : NTSAMD_OOB_OFFSET;
+    const int vOff0 = sc < dh ? sr0 * vL4 + sc * 4 : NTSAMD_OOB_OFFSET;
+    f32x4 kreg[LOADS], vreg[LOADS];
+    auto load_k = [&](int kb0) {
 #pragma unroll
-        for (int g = 0; g < NQ; g++) {
-            const int c = 8 * g + 4 * lh;
+        for (int s = 0; s < LOADS; s++)
+            kreg[s] = buffer_load_f32x4(kRsrc, sc < dh ? kOff0 + (kb0 + s * RSTEP) * kL4 : NTSAMD_OOB_OFFSET);
+    };
+    auto load_v = [&](int kb0) {
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            vreg[s] = buffer_load_f32x4(vRsrc, sc < dh ? vOff0 + (kb0 + s * RSTEP) * vL4 : NTSAMD_OOB_OFFSET);
+    };
+    load_k(0);
+
+    /* ---- Q fragments: lane (m, g) feeds query m with columns 16 t + 4 g + e in step e of group t ---- */
+    f32x4 qf[NT];
+    {
+        const float * qr = Q + (long long)rowc * p.qL;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int c = 16 * t + 4 * g;
             f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            qf[g] = c < dh ? *reinterpret_cast<const f32x4 *>(qr + c) : z;
+            qf[t] = c < dh ? *reinterpret_cast<const f32x4 *>(qr + c) : z;
         }
     }
+    load_v(0);
 
-    f32x16 accO[NO];
+    f32x4 accO[NT];
 #pragma unroll
-    for (int j = 0; j < NO; j++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            accO[j][r] = 0.f;
-    float rowMax[16], rowSum[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        rowMax[r] = -INFINITY;
-        rowSum[r] = 0.f;
-    }
-
-    float * myP = Ps + wave * 32 * PP;
+    for (int d = 0; d < NT; d++)
+        accO[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float rowMax = -INFINITY, rowSum = 0.f;              /* in units of log2: the scores are scaled by log2(e) */
+    const float scale2 = p.scale * LOG2E;
 
     for (int kb0 = 0; kb0 < lk; kb0 += KB) {
-        /* ---- key and value block into LDS: 16 bytes per thread and step; rows past lk and
-           columns past dh are zero ------------------------------------------------------ */
-        __syncthreads();                            /* the previous block is no longer read */
-#pragma unroll
-        for (int s = 0; s < LOADS; s++) {
-            const int idx = tid + s * 256;
-            const int row = idx / (DHM / 4), c = (idx % (DHM / 4)) * 4;
-            const int key = kb0 + row;
-            f32x4 kv = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
-            if (key < lk && c < dh) {
-                kv = *reinterpret_cast<const f32x4 *>(K + (long long)key * p.kL + c);
-                vv = *reinterpret_cast<const f32x4 *>(V + (long long)key * p.vL + c);
-            }
-            *reinterpret_cast<f32x4 *>(&Ks[row * KP + c]) = kv;
-            *reinterpret_cast<f32x4 *>(&Vs[row * KP + c]) = vv;
-        }
-        __syncthreads();
+        const bool more = kb0 + KB < lk;
 
-        /* ---- scores of the wave's 32 rows against the block's keys ---------------------- */
-        f32x16 accS[NJ];
+        /* every wave is past the second barrier of the previous block: nobody reads Ks any more */
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            *reinterpret_cast<f32x4 *>(&Ks[sLds + s * RSTEP * KP]) = kreg[s];
+        __syncthreads();                                 /* also: every wave has finished the previous block's Vs */
+        if (more)
+            load_k(kb0 + KB);
+
+        /* ---- S^T = K Q^T ------------------------------------------------------------------------ */
+        f32x4 accS[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; j++)
+            accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        /* fragments of group t + 1 are fetched while group t multiplies; the scheduling fences keep the
+           compiler from fetching every group up front, which costs more registers than there are */
+        f32x4 kf[2][NJ];
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-                accS[j][r] = 0.f;
+        for (int j = 0; j < NJ; j++)
+            kf[0][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 4 * g]);
 #pragma unroll
-        for (int g = 0; g < NQ; g++) {
-            if (8 * g < dh) {
+        for (int t = 0; t < NT; t++) {
+            if (t + 1 < NT) {
 #pragma unroll
-                for (int j = 0; j < NJ; j++) {
-                    const f32x4 kf = *reinterpret_cast<const f32x4 *>(&Ks[(j * 32 + l32) * KP + 8 * g + 4 * lh]);
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        accS[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[g][e], kf[e], accS[j], 0, 0, 0);
-                }
+                for (int j = 0; j < NJ; j++)
+                    kf[(t + 1) & 1][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 16 * (t + 1) + 4 * g]);
             }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+                    accS[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t & 1][j][e], qf[t][e], accS[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
-        /* ---- scale and mask: the mask test sits outside the loops so that the loads are not
-           fenced off one by one; rows and keys past the end read the last valid element ------ */
+        /* ---- scale and mask (tests hoisted so that the loads are not fenced off one by one) ------ */
         if (MK != nullptr) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int row = row0 + 8 * (r / 4) + 4 * lh + (r % 4);
-                row = row < lq ? row : lq - 1;
+            if (p.maskVec) {
 #pragma unroll
                 for (int j = 0; j < NJ; j++) {
-                    int key = kb0 + j * 32 + l32;
-                    key = key < lk ? key : lk - 1;
-                    accS[j][r] = accS[j][r] * p.scale + MK[(long long)row * lk + key];
+                    const int key = kb0 + 16 * j + 4 * g;      /* lk is a multiple of 4 here: all four or none */
+                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK + key) : z;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        accS[j][r] = fmaf(mk[r], LOG2E, accS[j][r] * scale2);
                 }
+            }
+            else {
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        int key = kb0 + 16 * j + 4 * g + r;
+                        key = key < lk ? key : lk - 1;
+                        accS[j][r] = fmaf(MK[key], LOG2E, accS[j][r] * scale2);
+                    }
             }
         }
         else {
 #pragma unroll
-            for (int r = 0; r < 16; r++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
-                    accS[j][r] *= p.scale;
+                for (int r = 0; r < 4; r++)
+                    accS[j][r] *= scale2;
+        }
+        if (kb0 + KB > lk) {                                   /* last, partial block: keys past the end count for nothing */
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (kb0 + 16 * j + 4 * g + r >= lk)
+                        accS[j][r] = -INFINITY;
         }
 
-        /* ---- running softmax ------------------------------------------------------------------- */
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float mx = -INFINITY;
-#pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                const int key = kb0 + j * 32 + l32;
-                const float s = key < lk ? accS[j][r] : -INFINITY;
-                accS[j][r] = s;
-                mx = fmaxf(mx, s);
-            }
-            mx = half_wave_max(mx);
-            const float newMax = fmaxf(rowMax[r], mx);
-            const float shift = newMax == -INFINITY ? 0.f : newMax;     /* a row with nothing to see yet */
-            const float corr = expf(rowMax[r] - shift);               /* exp(-inf) = 0 on the first block */
-            float sum = 0.f;
-#pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                const float e = expf(accS[j][r] - shift);
-                accS[j][r] = e;
-                sum += e;
-            }
-            sum = half_wave_sum(sum);
-            rowSum[r] = rowSum[r] * corr + sum;
-            rowMax[r] = newMax;
-#pragma unroll
-            for (int j = 0; j < NO; j++)
-                accO[j][r] *= corr;
-        }
-
-        /* ---- probabilities: accumulator layout -> operand layout through the wave's LDS ------ */
+        /* ---- running softmax of this lane's query row ------------------------------------------------ */
+        float mx = accS[0][0];
 #pragma unroll
         for (int j = 0; j < NJ; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-                myP[(8 * (r / 4) + 4 * lh + (r % 4)) * PP + j * 32 + l32] = accS[j][r];
-        /* the wave's own lanes exchange data: LDS runs one wave's instructions in order, the
-           fences keep the compiler from reordering */
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        /* ---- result += P times the value block ------------------------------------------------- */
+            for (int r = 0; r < 4; r++)
+                mx = fmaxf(mx, accS[j][r]);
+        mx = across_groups_max(mx);
+        const float newMax = fmaxf(rowMax, mx);
+        const float shift = newMax == -INFINITY ? 0.f : newMax;      /* a row with nothing to see yet */
+        const float corr = __builtin_amdgcn_exp2f(rowMax - shift);     /* 2^-inf = 0 on the first block */
+        float sum = 0.f;
 #pragma unroll
-        for (int g = 0; g < KB / 8; g++) {
-            const f32x4 pf = *reinterpret_cast<const f32x4 *>(&myP[l32 * PP + 8 * g + 4 * lh]);
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int kk = 8 * g + 4 * lh + e;
-#pragma unroll
-                for (int j = 0; j < NO; j++)
-                    if (j * 32 < dh)
-                        accO[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[e], Vs[kk * KP + j * 32 + l32], accO[j], 0, 0, 0);
+            for (int r = 0; r < 4; r++) {
+                const float e = __builtin_amdgcn_exp2f(accS[j][r] - shift);
+                accS[j][r] = e;
+                sum += e;
             }
+        sum = across_groups_sum(sum);
+        rowSum = rowSum * corr + sum;
+        rowMax = newMax;
+#pragma unroll
+        for (int d = 0; d < NT; d++)
+            accO[d] *= corr;
+
+        /* ---- values into LDS (every wave is past the first barrier: the previous block's Vs is done with) ---- */
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            *reinterpret_cast<f32x4 *>(&Vs[sLds + s * RSTEP * KP]) = vreg[s];
+        __syncthreads();                                 /* also: every wave has finished this block's Ks */
+        if (more)
+            load_v(kb0 + KB);
+
+        /* ---- O^T += V^T P^T: the probabilities are operands as they lie ---------------------------------- */
+        float vf[2][4][NT];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int d = 0; d < NT; d++)
+                vf[0][r][d] = Vs[(4 * g + r) * KP + m + 16 * d];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            if (j + 1 < NJ) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int d = 0; d < NT; d++)
+                        vf[(j + 1) & 1][r][d] = Vs[(16 * (j + 1) + 4 * g + r) * KP + m + 16 * d];
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int d = 0; d < NT; d++)
+                    accO[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j & 1][r][d], accS[j][r], accO[d], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     }
 
-    /* ---- out = result / row sum; a lane stores one column of 16 rows: 128 contiguous bytes per row ---- */
+    /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
+    if (row < lq) {
+        const float inv = rowSum > 0.f ? 1.f / rowSum : 0.f;
+        float * orow = O + (long long)row * p.oL;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int row = row0 + 8 * (r / 4) + 4 * lh + (r % 4);
-        if (row < lq) {
-            const float inv = rowSum[r] > 0.f ? 1.f / rowSum[r] : 0.f;
-            float * orow = O + (long long)row * p.oL;
-#pragma unroll
-            for (int j = 0; j < NO; j++) {
-                const int col = j * 32 + l32;
-                if (col < dh)
-                    orow[col] = accO[j][r] * inv;
-            }
+        for (int d = 0; d < NT; d++) {
+            const int c = 16 * d + 4 * g;
+            if (c < dh)
+                *reinterpret_cast<f32x4 *>(orow + c) = accO[d] * inv;
         }
     }
 }
@@ -262,9 +283,14 @@ attention_f32_kernel(const AttnParams p)
 int launch_attention_f32(const AttnParams & p0, hipStream_t stream)
 {
     AttnParams p = p0;
-    p.qTiles = (p.lq + 127) / 128;
+    p.qTiles = (p.lq + 63) / 64;
+    p.maskVec = (p.mask != nullptr && p.lk % 4 == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 15) == 0) ? 1 : 0;
     dim3 grid((unsigned)(p.heads * p.batch * p.qTiles));
-    if (p.dh <= 64)
+    if (p.dh <= 16)
+        hipLaunchKernelGGL((attention_f32_kernel<16, 128>), grid, dim3(256), 0, stream, p);
+    else if (p.dh <= 32)
+        hipLaunchKernelGGL((attention_f32_kernel<32, 128>), grid, dim3(256), 0, stream, p);
+    else if (p.dh <= 64)
         hipLaunchKernelGGL((attention_f32_kernel<64, 128>), grid, dim3(256), 0, stream, p);
     else
         hipLaunchKernelGGL((attention_f32_kernel<128, 64>), grid, dim3(256), 0, stream, p);

@@ -6,6 +6,7 @@
  */
 #include "../../include/ntsamd_gemm.h"
 #include "gemm_common.h"
+#include "attention.h"
 
 #include <atomic>
 #include <stdarg.h>
@@ -24,21 +25,6 @@ int launch_f16_tn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStre
 int launch_f16_tt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
 int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
-struct AttnParams {
-    const float * q;
-    const float * k;
-    const float * v;
-    const float * mask;
-    float * out;
-    int heads, batch, lq, lk, dh;
-    long long qH, qB, qL;
-    long long kH, kB, kL;
-    long long vH, vB, vL;
-    long long oH, oB, oL;
-    float scale;
-    int qTiles;
-};
-int launch_attention_f32(const AttnParams & p, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -486,8 +472,12 @@ int ntsamd_attention(int devID, void * stream,
     for (int t = 0; t < 4; t++)
         if (strides[3 * t + 2] < dh)
             return fail(NTSAMD_ERR_ARGUMENT, "row stride smaller than the head size");
-    if ((long long)heads * batch * ((lq + 127) / 128) > 0x7fffffffLL)
+    if ((long long)heads * batch * ((lq + 63) / 64) > 0x7fffffffLL)
         return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
+    /* the kernel addresses the rows of one head's k and v with 32-bit byte offsets, one block of keys ahead */
+    for (int t = 1; t <= 2; t++)
+        if (((long long)lk + 256) * strides[3 * t + 2] * 4 > 0x7fffffffLL)
+            return fail(NTSAMD_ERR_ARGUMENT, "tensor too large: the keys of one head span more than 2 GiB");
     int st = check_device(devID);
     if (st != NTSAMD_OK)
         return st;
