@@ -41,6 +41,7 @@ extern "C" {
 
 #define NTSAMD_X_TRANS 0
 #define NTSAMD_X_NOTRANS 1
+#define NTSAMD_X_INT 0
 #define NTSAMD_X_FLOAT 2
 #define NTSAMD_X_FLOAT16 3
 
@@ -189,6 +190,20 @@ int ntsamd_attention(int devID, void * stream,
                      const void * q, const void * k, const void * v, const void * mask, void * out, int dataType,
                      int heads, int batch, int lq, int lk, int dh,
                      const long long * strides, float scale);
+
+/*
+ * Element-wise data type conversion t[i] = (typeT) s[i], i < size.
+ * Replaces _CudaConvertDataType(devID, s, typeS, t, typeT, size) and the tensor form
+ * _CudaConvertDataType(input, output) (source/tensor/core/getandset/ConvertDataType.cu:78-99,
+ * :106-137) with their kernels (:31-66):
+ *   X_FLOAT -> X_FLOAT16  round to nearest even;  X_FLOAT16 -> X_FLOAT  exact;
+ *   X_FLOAT -> X_INT      toward zero, saturating, NaN -> 0;  X_INT -> X_FLOAT  round to nearest even.
+ * Equal types: nothing is done and nothing is copied, as in the reference (:81-82, :108-109).
+ * Every other pair: NTSAMD_ERR_DATATYPE, "Unsupported data types for conversion!".
+ * s and t must not overlap.
+ */
+int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS, void * t, int typeT,
+                             long long size);
 
 #ifdef __cplusplus
 }

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libntsamd.so")
 HOST_LIB_PATH = os.path.join(HERE, "lib", "libnts_amd.so")
 
 X_TRANS, X_NOTRANS = 0, 1           # MATRIX_TRANS_TYPE, source/tensor/XDataType.h:36
-X_FLOAT, X_FLOAT16 = 2, 3           # TENSOR_DATA_TYPE, source/tensor/XDataType.h:33
+X_INT, X_FLOAT, X_FLOAT16 = 0, 2, 3  # TENSOR_DATA_TYPE, source/tensor/XDataType.h:33
 BIAS_NONE, BIAS_COL, BIAS_ROW = 0, 1, 2
 
 EXPORTS = (
@@ -29,6 +29,7 @@ EXPORTS = (
     "ntsamd_matrix_mul_colsum",
     "ntsamd_reduce_sum_xz",
     "ntsamd_attention",
+    "ntsamd_convert_data_type",
 )
 
 
@@ -66,6 +67,7 @@ def load():
     L.ntsamd_matrix_mul_colsum.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, cf]
     L.ntsamd_reduce_sum_xz.argtypes = [ci, vp, vp, ci, ci, ci, ci, vp, cf]
     L.ntsamd_attention.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
+    L.ntsamd_convert_data_type.argtypes = [ci, vp, vp, ci, vp, ci, ll]
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
     _lib = L
@@ -83,6 +85,8 @@ def _dtype_code(t):
         return X_FLOAT
     if t.dtype == torch.float16:
         return X_FLOAT16
+    if t.dtype == torch.int32:
+        return X_INT
     raise NtsAmdError("Unsupported data type!")
 
 
@@ -194,3 +198,12 @@ def attention(q, k, v, out, heads, scale, mask=None, split=False):
                             heads, batch, lq, lk, dh, strides, scale)
     _check(rc)
     return out
+
+
+def convert_data_type(s, t):
+    """t[i] = (type of t) s[i] for dense device tensors of equal size (float32, float16, int32)."""
+    assert s.is_contiguous() and t.is_contiguous() and s.numel() == t.numel()
+    rc = load().ntsamd_convert_data_type(s.device.index, _stream_ptr(s), s.data_ptr(), _dtype_code(s),
+                                         t.data_ptr(), _dtype_code(t), s.numel())
+    _check(rc)
+    return t

@@ -25,6 +25,7 @@ int launch_f16_tn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStre
 int launch_f16_tt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
 int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
+int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -442,6 +443,43 @@ int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType
         return scope.status;
     int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,
                                   static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return NTSAMD_OK;
+}
+
+int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS, void * t, int typeT,
+                             long long size)
+{
+    if (typeS == typeT)
+        return NTSAMD_OK;
+    int kind = -1;
+    if (typeS == NTSAMD_X_FLOAT && typeT == NTSAMD_X_FLOAT16)
+        kind = 0;
+    else if (typeS == NTSAMD_X_FLOAT16 && typeT == NTSAMD_X_FLOAT)
+        kind = 1;
+    else if (typeS == NTSAMD_X_FLOAT && typeT == NTSAMD_X_INT)
+        kind = 2;
+    else if (typeS == NTSAMD_X_INT && typeT == NTSAMD_X_FLOAT)
+        kind = 3;
+    if (kind < 0)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data types for conversion!");
+    if (size < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
+    if (size == 0)
+        return NTSAMD_OK;
+    if (!s || !t)
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty input or output tensors!");
+    const size_t unitS = kind == 1 ? 2 : 4, unitT = kind == 0 ? 2 : 4;
+    if (reinterpret_cast<uintptr_t>(s) % unitS != 0 || reinterpret_cast<uintptr_t>(t) % unitT != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "misaligned tensor data");
+    int st = check_device(devID);
+    if (st != NTSAMD_OK)
+        return st;
+    DeviceScope scope(devID);
+    if (scope.status != NTSAMD_OK)
+        return scope.status;
+    int rc = launch_convert(kind, s, t, size, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

@@ -15,6 +15,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 X_TRANS, X_NOTRANS = 0, 1          # source/tensor/XDataType.h:36
 X_FLOAT, X_FLOAT16 = 2, 3          # source/tensor/XDataType.h:33
+X_INT = 0
+# numpy carriers of the three types: half travels as its bit pattern
+NP_TYPE_CODE = {np.float32: X_FLOAT, np.int32: X_INT, np.uint16: X_FLOAT16}
+TYPE_CODE_NP = {X_FLOAT: np.float32, X_INT: np.int32, X_FLOAT16: np.uint16}
 
 _fp = C.POINTER(C.c_float)
 _ip = C.POINTER(C.c_int)
@@ -84,6 +88,8 @@ class Oracle:
         L.oracle_softmax.restype = C.c_int
         L.oracle_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.oracle_attention.restype = C.c_int
+        L.oracle_convert_data_type.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_long]
+        L.oracle_convert_data_type.restype = C.c_int
         L.oracle_is_float_equal.argtypes = [C.c_float] * 4
         L.oracle_is_float_equal.restype = C.c_int
         L.oracle_check_data.argtypes = [_fp, _fp, C.c_int, C.c_float]
@@ -208,6 +214,19 @@ class Oracle:
             raise ValueError("Unmatched tensors in attention")
         return out
 
+    # -- data type conversion ------------------------------------------------
+    def convert(self, x, type_t):
+        """x: float32 (X_FLOAT), int32 (X_INT) or uint16 holding half bit patterns (X_FLOAT16);
+        returns the same for type_t."""
+        type_s = NP_TYPE_CODE[x.dtype.type]
+        x = np.ascontiguousarray(x)
+        out = np.empty(x.shape, TYPE_CODE_NP[type_t])
+        if type_s == type_t:
+            return x.copy()
+        if self.lib.oracle_convert_data_type(x.ctypes.data, type_s, out.ctypes.data, type_t, x.size) != 0:
+            raise ValueError("Unsupported data types for conversion!")
+        return out
+
     def is_float_equal(self, a, b, abs_err, rel_err=1e-4):
         return bool(self.lib.oracle_is_float_equal(a, b, abs_err, rel_err))
 
@@ -262,6 +281,7 @@ class Reference:
                                       _fp, _ip, C.c_int, _fp, _ip, C.c_float]
         L.ref_enum_values.argtypes = [_ip]
         L.ref_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.ref_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int]
         L.ref_softmax.argtypes = [_fp, _ip, C.c_int, _fp]
         L.ref_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.ref_grad.argtypes = [C.c_int, _fp, _ip, C.c_int, C.c_int, _fp, _ip, C.c_int, C.c_int,
@@ -341,6 +361,13 @@ class Reference:
         out = np.zeros_like(q)
         self.lib.ref_attention(_f(q), _f(k), _f(v), _f(mask) if mask is not None else None, _f(out),
                                batch, lq, k.shape[1], hidden, heads, scale)
+        return out
+
+    def convert(self, x, type_t):
+        type_s = NP_TYPE_CODE[x.dtype.type]
+        x = np.ascontiguousarray(x)
+        out = np.empty(x.shape, TYPE_CODE_NP[type_t])
+        self.lib.ref_convert(x.ctypes.data, type_s, out.ctypes.data, type_t, x.size)
         return out
 
     def run_matmul_tests(self):

@@ -685,6 +685,42 @@ int oracle_attention(const float *q, const float *k, const float *v, const float
     return r;
 }
 
+/* ---- data type conversion ------------------------------------------------- */
+
+int oracle_convert_data_type(const void *s, int typeS, void *t, int typeT, long n)
+{
+    if (typeS == typeT)
+        return 0;
+    if (typeS == 2 && typeT == 3)
+        oracle_f32_to_f16_array((const float *)s, (uint16_t *)t, n);
+    else if (typeS == 3 && typeT == 2)
+        oracle_f16_to_f32_array((const uint16_t *)s, (float *)t, n);
+    else if (typeS == 2 && typeT == 0) {
+        const float *in = (const float *)s;
+        int *out = (int *)t;
+        for (long i = 0; i < n; i++) {
+            float x = in[i];
+            if (x != x)
+                out[i] = 0;
+            else if (x >= 2147483648.0F)
+                out[i] = 0x7fffffff;
+            else if (x <= -2147483648.0F)
+                out[i] = (int)0x80000000;
+            else
+                out[i] = (int)x;
+        }
+    }
+    else if (typeS == 0 && typeT == 2) {
+        const int *in = (const int *)s;
+        float *out = (float *)t;
+        for (long i = 0; i < n; i++)
+            out[i] = (float)in[i];
+    }
+    else
+        return -1;
+    return 0;
+}
+
 /* ---- comparator ---------------------------------------------------------- */
 
 int oracle_is_float_equal(float a, float b, float absError, float relError)

@@ -103,6 +103,15 @@ int oracle_softmax(const float *x, long rows, int n, float *y);
 int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
                      int batch, int lq, int lk, int hidden, int heads, float scale);
 
+/* t[i] = (typeT) s[i] as the reference's GPU kernels convert (source/tensor/core/getandset/
+   ConvertDataType.cu:31-66): X_FLOAT -> X_FLOAT16 round to nearest even (__float2half), X_FLOAT16 -> X_FLOAT
+   exact, X_FLOAT -> X_INT toward zero (saturating, NaN -> 0: the GPU's cast), X_INT -> X_FLOAT round to
+   nearest even. float <-> int is also what the CPU branch computes for values inside the int range
+   (ConvertDataType.cpp:83-94); the CPU branch for half (:95-106) casts the VALUE to an integer and is not
+   followed. Types are the reference's TENSOR_DATA_TYPE values (X_INT 0, X_FLOAT 2, X_FLOAT16 3).
+   Returns 0, or -1 for a pair of types the reference refuses; equal types do nothing (:81-82). */
+int oracle_convert_data_type(const void *s, int typeS, void *t, int typeT, long n);
+
 /* comparator of the reference tests, CheckData.cpp:29-39 */
 int oracle_is_float_equal(float a, float b, float absError, float relError);
 /* CheckData.cpp:78-97 with its fixed relative bound 1e-4 */

@@ -243,6 +243,20 @@ int ref_attention(const float * q, const float * k, const float * v, const float
     return 0;
 }
 
+/* _ConvertDataType between X_FLOAT (2) and X_INT (0) on the host (ConvertDataType.cpp:83-94); the
+   half branches of the host code cast the value to an integer and are of no use as a reference */
+int ref_convert(const void * s, int typeS, void * t, int typeT, int n)
+{
+    int dims[1] = {n};
+    XTensor * ts = NewTensorV2(1, dims, (TENSOR_DATA_TYPE)typeS, 1.0F, -1);
+    XTensor * tt = NewTensorV2(1, dims, (TENSOR_DATA_TYPE)typeT, 1.0F, -1);
+    memcpy(ts->data, s, (size_t)n * ts->unitSize);
+    _ConvertDataType(ts, tt);
+    memcpy(t, tt->data, (size_t)n * tt->unitSize);
+    delete ts; delete tt;
+    return 0;
+}
+
 /* the reference's own known-answer tests for this path; bit i set = suite i passed */
 int ref_run_matmul_tests()
 {
