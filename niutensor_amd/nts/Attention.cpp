@@ -1,0 +1,63 @@
+/*
+ * Multi-head attention as one kernel launch.
+ * Shape rules follow the operators it stands for: Split(x, order - 1, nhead) turns (batch..., l, hidden)
+ * into (nhead, batch..., l, hidden / nhead) (source/tensor/core/shape/Split.cpp:39-124), the batched
+ * products pair equal leading dimensions (core/arithmetic/MatrixMulBatched.cpp:49-138), Softmax runs over
+ * the last dimension, Merge(x, order - 1) undoes the split (core/shape/Merge.cpp:41-150).
+ */
+#include "Attention.h"
+#include "../../include/ntsamd_gemm.h"
+
+namespace nts {
+
+void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, const XTensor * mask,
+                   XTensor * out, int nhead, DTYPE scale)
+{
+    CheckNTErrors((q && k && v && out), "Empty input tensors!");
+    CheckNTErrors((q->dataType == X_FLOAT && k->dataType == X_FLOAT && v->dataType == X_FLOAT && out->dataType == X_FLOAT),
+                  "TODO!");
+    CheckNTErrors((q->order >= 2 && q->order == k->order && q->order == v->order && q->order == out->order),
+                  "Input tensors must have the same order >= 2!");
+    CheckNTErrors((q->devID >= 0), "This code must be run on GPUs!");
+    CheckNTErrors((q->devID == k->devID && q->devID == v->devID && q->devID == out->devID),
+                  "The tensors must be on the same GPU!");
+    CheckNTErrors((_IsSameShaped(k, v) && _IsSameShaped(q, out)), "Unmatched tensors in attention!");
+
+    const int order = q->order;
+    const int hidden = q->dimSize[order - 1];
+    const int lq = q->dimSize[order - 2], lk = k->dimSize[order - 2];
+    CheckNTErrors((nhead > 0 && hidden % nhead == 0), "The hidden size must be a multiple of the number of heads!");
+    CheckNTErrors((k->dimSize[order - 1] == hidden), "Unmatched tensors in attention!");
+    int batch = 1;
+    for (int i = 0; i < order - 2; i++) {
+        CheckNTErrors((q->dimSize[i] == k->dimSize[i]), "Unmatched tensors in attention!");
+        batch *= q->dimSize[i];
+    }
+    if (mask != NULL) {
+        CheckNTErrors((mask->dataType == X_FLOAT && mask->devID == q->devID), "Unmatched tensors in attention!");
+        CheckNTErrors((mask->unitNum == nhead * batch * lq * lk), "Unmatched tensors in attention!");
+    }
+
+    const int dh = hidden / nhead;
+    /* head h of row r of batch item b starts at element b * rows * hidden + r * hidden + h * dh */
+    long long strides[12] = {dh, (long long)lq * hidden, hidden,
+                             dh, (long long)lk * hidden, hidden,
+                             dh, (long long)lk * hidden, hidden,
+                             dh, (long long)lq * hidden, hidden};
+    int rc = ntsamd_attention(q->devID, NULL, q->data, k->data, v->data, mask != NULL ? mask->data : NULL, out->data,
+                              X_FLOAT, nhead, batch, lq, lk, dh, strides, scale);
+    if (rc != NTSAMD_OK) {
+        ShowNTErrors(ntsamd_last_error());
+    }
+}
+
+XTensor AmdAttention(const XTensor & q, const XTensor & k, const XTensor & v, const XTensor * mask,
+                     int nhead, DTYPE scale)
+{
+    XTensor out(q.order, q.dimSize, q.dataType, 1.0F, q.devID, q.mem);
+    out.SetTMPFlag();
+    _AmdAttention(&q, &k, &v, mask, &out, nhead, scale);
+    return out;
+}
+
+}  // namespace nts

@@ -1,0 +1,24 @@
+/*
+ * Multi-head attention of the reference's transformer sample as one call on a gfx950 GPU:
+ * what Attention::MakeAttention (source/sample/transformer/submodel/Attention.cpp:186-239)
+ * computes between the input projections and the output projection when it is not training.
+ */
+#ifndef NTSAMD_ATTENTION_H
+#define NTSAMD_ATTENTION_H
+
+#include "XTensor.h"
+
+namespace nts {
+
+/* out = Merge(Softmax(Split(q) * scale x Split(k)^T + mask, -1) x Split(v))
+   q, out: (batch..., lq, hidden); k, v: (batch..., lk, hidden); nhead divides hidden;
+   mask: NULL or (nhead, batch..., lq, lk), added to the scaled scores. All X_FLOAT, one GPU. */
+void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, const XTensor * mask,
+                   XTensor * out, int nhead, DTYPE scale);
+
+/* the same into a new tensor shaped like q */
+XTensor AmdAttention(const XTensor & q, const XTensor & k, const XTensor & v, const XTensor * mask,
+                     int nhead, DTYPE scale);
+
+}  // namespace nts
+#endif

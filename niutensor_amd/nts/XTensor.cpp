@@ -8,12 +8,17 @@
 #include <hip/hip_runtime_api.h>
 
 #include <atomic>
+#include <mutex>
 #include <stdlib.h>
 #include <string.h>
+#include <unordered_map>
+#include <vector>
 
 namespace nts {
 
 static std::atomic<int> tensorIDGlobal(0);
+
+#define MAX_CACHED_DEVICES 16
 
 #define CheckHip(call, msg) \
 { \
@@ -47,6 +52,55 @@ struct DevScope {
     }
 };
 
+/* ---- device memory: blocks are kept and handed out again ----------------------
+   The reference takes the temporaries of a forward or backward step out of a memory pool
+   (XMem, source/tensor/XMem.h:150-420) when one is attached, and calls cudaMalloc / cudaFree
+   per tensor when none is (XUtility.cpp XMemAlloc / XMemFree). hipFree waits for the device
+   and hipMalloc costs tens of microseconds, more than an attention-sized product takes, so
+   here a freed block goes onto a per-device list of its size class and the next request of
+   that class takes it from there. That is safe because every kernel and copy of this layer
+   is issued to the NULL stream, as in the reference: whatever still reads or writes a block
+   when the host gives it up has been queued before anything that the block's next owner
+   queues. Size classes keep three leading bits (at most 12.5 % slack), 256 bytes at least.
+   NTSAMD_MEM_CACHE=0 switches the lists off; NTSAMD_MEM_CACHE_MB caps the bytes kept per
+   device (default 32768); XMemCacheRelease gives everything back. */
+
+struct MemCache {
+    std::mutex lock;
+    std::unordered_map<void *, size_t> live[MAX_CACHED_DEVICES];               /* block -> class size */
+    std::unordered_map<size_t, std::vector<void *> > spare[MAX_CACHED_DEVICES];  /* class size -> free blocks */
+    size_t spareBytes[MAX_CACHED_DEVICES];
+    long long hits, misses;
+    bool enabled;
+    size_t capBytes;
+    MemCache() : hits(0), misses(0)
+    {
+        for (int i = 0; i < MAX_CACHED_DEVICES; i++)
+            spareBytes[i] = 0;
+        const char * e = getenv("NTSAMD_MEM_CACHE");
+        enabled = !(e != NULL && e[0] == '0');
+        const char * c = getenv("NTSAMD_MEM_CACHE_MB");
+        capBytes = (size_t)(c != NULL ? atoll(c) : 32768) << 20;
+    }
+};
+
+static MemCache & Cache()
+{
+    static MemCache * c = new MemCache();      /* never destroyed: tensors with static lifetime may outlive it */
+    return *c;
+}
+
+static size_t SizeClass(size_t size)
+{
+    if (size <= 256)
+        return 256;
+    int top = 63 - __builtin_clzll((unsigned long long)(size - 1));      /* highest set bit of size - 1 */
+    size_t step = (size_t)1 << (top >= 3 ? top - 2 : 0);                  /* keep three leading bits */
+    if (step < 256)
+        step = 256;
+    return (size + step - 1) / step * step;
+}
+
 void * XMemAlloc(int devID, size_t size)
 {
     void * p = NULL;
@@ -55,11 +109,38 @@ void * XMemAlloc(int devID, size_t size)
     if (devID < 0) {
         p = malloc(size);
         CheckNTErrors(p != NULL, "Cannot allocate the memory.");
+        return p;
     }
-    else {
+    MemCache & mc = Cache();
+    if (!mc.enabled || devID >= MAX_CACHED_DEVICES) {
         DevScope scope(devID);
         CheckHip(hipMalloc(&p, size), "Cannot allocate the memory.");
+        return p;
     }
+    const size_t cls = SizeClass(size);
+    {
+        std::lock_guard<std::mutex> guard(mc.lock);
+        std::vector<void *> & list = mc.spare[devID][cls];
+        if (!list.empty()) {
+            p = list.back();
+            list.pop_back();
+            mc.spareBytes[devID] -= cls;
+            mc.live[devID][p] = cls;
+            mc.hits++;
+            return p;
+        }
+        mc.misses++;
+    }
+    DevScope scope(devID);
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+        /* out of memory with blocks lying idle: give them back and try once more */
+        (void)hipGetLastError();
+        XMemCacheRelease(devID);
+        CheckHip(hipMalloc(&p, cls), "Cannot allocate the memory.");
+    }
+    std::lock_guard<std::mutex> guard(mc.lock);
+    mc.live[devID][p] = cls;
     return p;
 }
 
@@ -67,12 +148,66 @@ void XMemFree(int devID, void * p)
 {
     if (p == NULL)
         return;
-    if (devID < 0)
+    if (devID < 0) {
         free(p);
-    else {
-        DevScope scope(devID);
-        CheckHip(hipFree(p), "Cannot free the memory.");
+        return;
     }
+    MemCache & mc = Cache();
+    if (devID < MAX_CACHED_DEVICES) {
+        std::lock_guard<std::mutex> guard(mc.lock);
+        std::unordered_map<void *, size_t>::iterator it = mc.live[devID].find(p);
+        if (it != mc.live[devID].end()) {
+            const size_t cls = it->second;
+            mc.live[devID].erase(it);
+            if (mc.enabled && mc.spareBytes[devID] + cls <= mc.capBytes) {
+                mc.spare[devID][cls].push_back(p);
+                mc.spareBytes[devID] += cls;
+                return;
+            }
+        }
+    }
+    DevScope scope(devID);
+    CheckHip(hipFree(p), "Cannot free the memory.");
+}
+
+void XMemCacheRelease(int devID)
+{
+    MemCache & mc = Cache();
+    if (devID < 0 || devID >= MAX_CACHED_DEVICES)
+        return;
+    std::vector<void *> blocks;
+    {
+        std::lock_guard<std::mutex> guard(mc.lock);
+        for (std::unordered_map<size_t, std::vector<void *> >::iterator it = mc.spare[devID].begin();
+             it != mc.spare[devID].end(); ++it)
+            blocks.insert(blocks.end(), it->second.begin(), it->second.end());
+        mc.spare[devID].clear();
+        mc.spareBytes[devID] = 0;
+    }
+    if (blocks.empty())
+        return;
+    DevScope scope(devID);
+    for (size_t i = 0; i < blocks.size(); i++)
+        CheckHip(hipFree(blocks[i]), "Cannot free the memory.");
+}
+
+void XMemCacheStats(int devID, size_t * spareBytes, long long * hits, long long * misses)
+{
+    MemCache & mc = Cache();
+    std::lock_guard<std::mutex> guard(mc.lock);
+    if (spareBytes != NULL)
+        *spareBytes = devID >= 0 && devID < MAX_CACHED_DEVICES ? mc.spareBytes[devID] : 0;
+    if (hits != NULL)
+        *hits = mc.hits;
+    if (misses != NULL)
+        *misses = mc.misses;
+}
+
+void XMemCacheEnable(bool on)
+{
+    MemCache & mc = Cache();
+    std::lock_guard<std::mutex> guard(mc.lock);
+    mc.enabled = on;
 }
 
 void XMemCopy(void * t, int devIDT, const void * s, int devIDS, size_t size)
@@ -114,7 +249,7 @@ void XLink::MakeLink(const XTensor * t1, const XTensor * t2, XTensor * h, int id
     h->income.typeID = id;
     h->income.tails[0] = t1;
     h->income.tails[1] = t2;
-    h->income.tailNum = 2;
+    h->income.tailNum = t2 != NULL ? 2 : 1;
 }
 
 void XLink::MakeLink(const XTensor * t1, const XTensor * t2, const XTensor * t3, XTensor * h, int id)

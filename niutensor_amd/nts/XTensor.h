@@ -19,6 +19,8 @@
 #include "XGlobal.h"
 #include "XDataType.h"
 
+#include <stddef.h>
+
 namespace nts {
 
 #define MAX_TENSOR_DIM_NUM 8
@@ -141,6 +143,14 @@ bool IsSameShaped(const XTensor & a, const XTensor & b);
 void * XMemAlloc(int devID, size_t size);
 void XMemFree(int devID, void * p);
 void XMemCopy(void * t, int devIDT, const void * s, int devIDS, size_t size);
+
+/* Freed device blocks are kept per device and size class and handed out again (see XTensor.cpp).
+   XMemCacheRelease returns every idle block of a device to the HIP runtime; XMemCacheStats reports the
+   idle bytes of a device and how many requests were (not) served from the lists; XMemCacheEnable(false)
+   makes every later request and release go straight to hipMalloc / hipFree. */
+void XMemCacheRelease(int devID);
+void XMemCacheStats(int devID, size_t * spareBytes, long long * hits, long long * misses);
+void XMemCacheEnable(bool on);
 
 }  // namespace nts
 #endif

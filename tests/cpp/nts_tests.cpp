@@ -8,6 +8,7 @@
  * MulAndShift, lists, the backward step) are checked against the CPU oracle on seeded inputs.
  *
  *   nts_tests                run everything on device 0, exit 0 if all passed
+ *   nts_tests --alloc-bench  time an allocating call with and without reuse of device blocks
  *   nts_tests --abort NAME   provoke one fatal error (no GPU needed): the process
  *                            must print the reference's message and abort
  */
@@ -17,8 +18,11 @@
 #include "../../niutensor_amd/nts/MatrixMulBatched.h"
 #include "../../niutensor_amd/nts/MulAndShift.h"
 #include "../../niutensor_amd/nts/XBackwardMath.h"
+#include "../../niutensor_amd/nts/ConvertDataType.h"
+#include "../../niutensor_amd/nts/Attention.h"
 #include "../../oracle/nts_oracle.h"
 
+#include <chrono>
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -608,6 +612,184 @@ static bool TestGradMulAndShift()
     return ok;
 }
 
+/* ---- data type conversion: the reference's TConvertDataType, GPU halves ------------------ */
+
+/* TConvertDataType.cpp case 1 (:36-90) float -> int and case 2 (:111-165) int -> float */
+static bool TestConvertDataType12()
+{
+    int dims[2] = {3, 2};
+    DTYPE aData[3][2] = {{1.0F, 2.0F}, {0.5F, 4.0F}, {5.0F, 6.0F}};
+    int answer[3][2] = {{1, 2}, {0, 4}, {5, 6}};
+    XTensor * a = NewTensorV2(2, dims, X_FLOAT, 1.0F, DEV);
+    XTensor * b = NewTensorV2(2, dims, X_INT, 1.0F, DEV);
+    a->SetData(aData, 6);
+    b->SetZeroAll();
+    _ConvertDataType(a, b);
+    int got[6];
+    b->GetData(got);
+    bool ok = memcmp(got, answer, sizeof(got)) == 0;
+
+    DTYPE answer2[3][2] = {{1.0F, 2.0F}, {0.0F, 4.0F}, {5.0F, 6.0F}};
+    XTensor * c = NewTensorV2(2, dims, X_FLOAT, 1.0F, DEV);
+    c->SetZeroAll();
+    _ConvertDataType(b, c);
+    ok = ok && CheckData(c, answer2, 6, 1e-4F);
+    delete a; delete b; delete c;
+    return ok;
+}
+
+/* TConvertDataType.cpp case 3 (:185-268): float -> half for both operands, the half product, half -> float;
+   the answer stands in the reference's test (:243-245) with its comparison commented out (:270) */
+static bool TestConvertDataType3()
+{
+    int d1[2] = {3, 2}, d2[2] = {2, 3}, d3[2] = {3, 3};
+    DTYPE data1[3][2] = {{1.0F, -2.0F}, {0.5F, -4.0F}, {0.0F, 6.0F}};
+    DTYPE data2[2][3] = {{1.0F, 2.0F, 3.0F}, {0.0F, 4.0F, 5.0F}};
+    DTYPE answer[3][3] = {{1.0F, -6.0F, -7.0F}, {0.5F, -15.0F, -18.5F}, {0.0F, 24.0F, 30.0F}};
+    XTensor * a = NewTensorV2(2, d1, X_FLOAT, 1.0F, DEV);
+    XTensor * b = NewTensorV2(2, d2, X_FLOAT, 1.0F, DEV);
+    XTensor * c = NewTensorV2(2, d1, X_FLOAT16, 1.0F, DEV);
+    XTensor * d = NewTensorV2(2, d2, X_FLOAT16, 1.0F, DEV);
+    XTensor * e = NewTensorV2(2, d3, X_FLOAT16, 1.0F, DEV);
+    XTensor * f = NewTensorV2(2, d3, X_FLOAT, 1.0F, DEV);
+    a->SetData(data1, 6);
+    b->SetData(data2, 6);
+    _ConvertDataType(a, c);
+    _ConvertDataType(b, d);
+    _MatrixMul(c, X_NOTRANS, d, X_NOTRANS, e);
+    _ConvertDataType(e, f);
+    bool ok = CheckData(f, answer, 9, 1e-4F);
+    /* the round trip of the test's CPU half (:229-235) */
+    XTensor back = ConvertDataType(ConvertDataType(*a, X_FLOAT16), X_FLOAT);
+    ok = ok && back.dataType == X_FLOAT && CheckData(&back, data1, 6, 1e-4F);
+    /* the allocating form records its edge only for a tensor that takes part in autograd */
+    a->enableGrad = true;
+    XTensor linked = ConvertDataType(*a, X_FLOAT16);
+    ok = ok && linked.income.typeID == GETANDSET_CONVERTDATATYPE && linked.income.tailNum == 1 && linked.income.tails[0] == a;
+    ok = ok && back.income.tailNum == 0;
+    delete a; delete b; delete c; delete d; delete e; delete f;
+    return ok;
+}
+
+/* ---- attention in one call against the oracle's restatement of the operator chain ------------- */
+
+static bool TestAttention()
+{
+    bool ok = true;
+    const int cases[3][5] = {{2, 37, 53, 64, 4}, {3, 128, 128, 96, 2}, {1, 70, 200, 128, 1}};   /* batch, lq, lk, hidden, heads */
+    for (int ci = 0; ci < 3; ci++)
+        for (int masked = 0; masked < 2; masked++) {
+            const int B = cases[ci][0], lq = cases[ci][1], lk = cases[ci][2], H = cases[ci][3], nh = cases[ci][4];
+            int dq[3] = {B, lq, H}, dk[3] = {B, lk, H}, dm[4] = {nh, B, lq, lk};
+            std::vector<float> q(B * lq * H), k(B * lk * H), v(B * lk * H), m(nh * B * lq * lk), ref(B * lq * H), got(B * lq * H);
+            oracle_fill_normal(q.data(), (long)q.size(), 71 + ci, 0, 1.0F);
+            oracle_fill_normal(k.data(), (long)k.size(), 72 + ci, 0, 1.0F);
+            oracle_fill_normal(v.data(), (long)v.size(), 73 + ci, 0, 1.0F);
+            oracle_fill_uniform(m.data(), (long)m.size(), 74 + ci, 0.0F, 1.0F);
+            for (size_t i = 0; i < m.size(); i++)
+                m[i] = (m[i] < 0.3F && i % lk != 0) ? -1e9F : 0.0F;
+            const float scale = 1.0F / sqrtf((float)(H / nh));
+            oracle_attention(q.data(), k.data(), v.data(), masked ? m.data() : NULL, ref.data(), B, lq, lk, H, nh, scale);
+            XTensor * gq = NewGPU(3, dq, q.data());
+            XTensor * gk = NewGPU(3, dk, k.data());
+            XTensor * gv = NewGPU(3, dk, v.data());
+            XTensor * gm = masked ? NewGPU(4, dm, m.data()) : NULL;
+            XTensor out = AmdAttention(*gq, *gk, *gv, gm, nh, scale);
+            out.GetData(got.data());
+            float e = MaxRelErr(got, ref);
+            if (!(e < 1e-5F * sqrtf((float)(H / nh + lk)))) {
+                fprintf(stderr, "attention case %d masked %d err=%g\n", ci, masked, e);
+                ok = false;
+            }
+            delete gq; delete gk; delete gv;
+            if (gm != NULL)
+                delete gm;
+        }
+    return ok;
+}
+
+/* ---- device blocks are handed out again: same results, no growth --------------------------------- */
+
+static bool TestMemoryReuse()
+{
+    bool ok = true;
+    int dq[3] = {16, 64, 32};
+    std::vector<float> q(16 * 64 * 32), k(16 * 64 * 32), first(16 * 64 * 64), again(16 * 64 * 64);
+    oracle_fill_normal(q.data(), (long)q.size(), 91, 0, 1.0F);
+    oracle_fill_normal(k.data(), (long)k.size(), 92, 0, 1.0F);
+    XTensor * gq = NewGPU(3, dq, q.data());
+    XTensor * gk = NewGPU(3, dq, k.data());
+    {
+        XTensor s = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        s.GetData(first.data());
+    }
+    long long h0, m0, h1, m1;
+    size_t spare0, spare1;
+    XMemCacheStats(DEV, &spare0, &h0, &m0);
+    void * seen = NULL;
+    for (int i = 0; i < 50; i++) {
+        XTensor s = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        if (i == 0)
+            seen = s.data;
+        ok = ok && s.data == seen;                     /* the block the previous result gave up */
+        if (i == 49)
+            s.GetData(again.data());
+    }
+    XMemCacheStats(DEV, &spare1, &h1, &m1);
+    ok = ok && h1 - h0 == 50 && m1 == m0 && spare1 == spare0;
+    ok = ok && memcmp(first.data(), again.data(), first.size() * sizeof(float)) == 0;
+    /* requests of another size class do not take that block; releasing empties the lists */
+    int dsmall[2] = {5, 7};
+    XTensor * t = NewTensorV2(2, dsmall, X_FLOAT, 1.0F, DEV);
+    ok = ok && t->data != seen;
+    delete t;
+    XMemCacheRelease(DEV);
+    XMemCacheStats(DEV, &spare1, NULL, NULL);
+    ok = ok && spare1 == 0;
+    /* switched off, a request goes to the runtime and a release goes back to it */
+    XMemCacheEnable(false);
+    {
+        XTensor s = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        s.GetData(again.data());
+        ok = ok && memcmp(first.data(), again.data(), first.size() * sizeof(float)) == 0;
+    }
+    XMemCacheStats(DEV, &spare1, NULL, NULL);
+    ok = ok && spare1 == 0;
+    XMemCacheEnable(true);
+    delete gq; delete gk;
+    return ok;
+}
+
+/* time per allocating call at the attention shape of the benchmark, with and without block reuse */
+static int AllocBench()
+{
+    int dq[3] = {256, 128, 64};
+    std::vector<float> q(256 * 128 * 64);
+    oracle_fill_normal(q.data(), (long)q.size(), 5, 0, 1.0F);
+    XTensor * gq = NewGPU(3, dq, q.data());
+    XTensor * gk = NewGPU(3, dq, q.data());
+    float sink;
+    for (int mode = 0; mode < 2; mode++) {
+        XMemCacheEnable(mode == 0);
+        for (int i = 0; i < 20; i++)
+            XTensor s = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        gq->GetData(q.data());                          /* a blocking copy: the queue is empty */
+        const int n = 500;
+        auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < n; i++)
+            XTensor s = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        XTensor last = MatrixMulBatched(*gq, X_NOTRANS, *gk, X_TRANS, 0.125F);
+        XMemCopy(&sink, -1, last.data, DEV, sizeof(float));
+        auto t1 = std::chrono::steady_clock::now();
+        printf("MatrixMulBatched [256x128x64] x [256x128x64]^T, new result tensor per call, blocks %s: %.1f us per call\n",
+               mode == 0 ? "handed out again" : "from hipMalloc / hipFree",
+               std::chrono::duration<double, std::micro>(t1 - t0).count() / (n + 1));
+    }
+    XMemCacheEnable(true);
+    delete gq; delete gk;
+    return 0;
+}
+
 /* ---- fatal errors: same message, same ending as the reference ---------------- */
 
 static int Provoke(const char * name)
@@ -661,6 +843,8 @@ int main(int argc, char ** argv)
 {
     if (argc == 3 && !strcmp(argv[1], "--abort"))
         return Provoke(argv[2]);
+    if (argc == 2 && !strcmp(argv[1], "--alloc-bench"))
+        return AllocBench();
 
     bool all = true;
     RUN(TestMatrixMul1);
@@ -679,6 +863,10 @@ int main(int argc, char ** argv)
     RUN(TestGradMatrixMulFlattenAndEfficient);
     RUN(TestGradMatrixMulBatched);
     RUN(TestGradMulAndShift);
+    RUN(TestConvertDataType12);
+    RUN(TestConvertDataType3);
+    RUN(TestAttention);
+    RUN(TestMemoryReuse);
     printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
     return all ? 0 : 1;
 }
