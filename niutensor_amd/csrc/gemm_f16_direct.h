@@ -76,10 +76,11 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
                  : "memory");
 }
 
-template <int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
+    static_assert(!CS || std::is_same<OutT, half_t>::value, "column sums have the type of b and of c");
     constexpr int BKT = 32, KS = 2, NSTAGE = 4;
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -105,7 +106,7 @@ gemm_f16_direct_kernel(const GemmParams p)
     const TileCoord tc = tile_of_workgroup(p);
     const half_t * __restrict__ A = static_cast<const half_t *>(p.a) + (long long)tc.batch * p.strideA;
     const half_t * __restrict__ B = static_cast<const half_t *>(p.b) + (long long)tc.batch * p.strideB;
-    half_t * __restrict__ C = static_cast<half_t *>(p.c) + (long long)tc.batch * p.strideC;
+    OutT * __restrict__ C = static_cast<OutT *>(p.c) + (long long)tc.batch * p.strideC;
 
     const int M = p.M, N = p.N, K = p.K;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
@@ -375,10 +376,10 @@ gemm_f16_direct_kernel(const GemmParams p)
     const int laneE = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     const int l32E = laneE & 31, lhE = laneE >> 5;
     const float alpha = p.alpha, beta = p.beta;
-    const half_t * __restrict__ bias = static_cast<const half_t *>(p.bias);
+    const OutT * __restrict__ bias = static_cast<const OutT *>(p.bias);     /* the bias has the type of c */
     const int biasMode = p.biasMode;
-    half_t * cw = C + (size_t)(m0 + wm0) * p.ldc;
-    const unsigned rowPitch = (unsigned)p.ldc * 2u;
+    OutT * cw = C + (size_t)(m0 + wm0) * p.ldc;
+    const unsigned rowPitch = (unsigned)p.ldc * (unsigned)sizeof(OutT);
 
     if constexpr (CS) {
         /* the first tile row's first wave row has seen every k of its columns */
@@ -402,8 +403,9 @@ gemm_f16_direct_kernel(const GemmParams p)
        lines, an eighth of the instructions. With beta == 0 the values cross LDS as halves;
        with beta != 0 they cross as fp32 and meet the old c (one 16-byte load per lane) on the
        far side, so the result is still rounded once. */
-    const bool wide = (p.ldc & 7) == 0 && (N & 7) == 0 && (reinterpret_cast<size_t>(C) & 15) == 0;
-    if (wide) {
+    const bool wide = std::is_same<OutT, half_t>::value &&
+                      (p.ldc & 7) == 0 && (N & 7) == 0 && (reinterpret_cast<size_t>(C) & 15) == 0;
+    if constexpr (std::is_same<OutT, half_t>::value) if (wide) {
         constexpr int LPR = TJ * 4;                  /* lanes that cover one row of the wave's tile */
         constexpr int RPI = 64 / LPR;                /* rows per 16-byte store instruction */
         __syncthreads();                             /* every wave has read its last fragments */
@@ -483,18 +485,20 @@ gemm_f16_direct_kernel(const GemmParams p)
         return;
     }
 
-    /* Narrow path: 2-byte stores straight from the accumulators, any alignment of c. beta is
-       tested outside the loops: inside them every load of c would sit in a block of its own,
-       one memory round trip after the other. */
+    /* Narrow path: element-wise stores straight from the accumulators, any alignment of c; also the
+       path of a float result (half products whose result feeds a softmax: no separate conversion pass),
+       where an instruction covers two rows of 128 contiguous bytes. beta is tested outside the loops:
+       inside them every load of c would sit in a block of its own, one memory round trip after the other. */
     if (m0 + wm0 >= M)
         return;
-    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * 2);
+    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * (long long)sizeof(OutT));
     auto narrow = [&](auto BETAC) {
         constexpr bool useOld = decltype(BETAC)::value != 0;
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = n0 + wn0 + j * 32 + l32E;
-            const unsigned cOff = col < N ? (unsigned)(4 * lhE * p.ldc + col) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+            const unsigned cOff = col < N ? (unsigned)(4 * lhE * p.ldc + col) * (unsigned)sizeof(OutT)
+                                          : (unsigned)NTSAMD_OOB_OFFSET;
             float bcol = 0.f;
             if (biasMode == BIAS_COL && col < N)
                 bcol = (float)bias[col];
@@ -504,7 +508,7 @@ gemm_f16_direct_kernel(const GemmParams p)
                 if constexpr (useOld) {
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        old[r] = buffer_load_out<half_t>(cr, (int)(cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch));
+                        old[r] = buffer_load_out<OutT>(cr, (int)(cOff + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch));
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
@@ -512,7 +516,7 @@ gemm_f16_direct_kernel(const GemmParams p)
                     float v = alpha * acc[i][j][r] + bcol;
                     if constexpr (useOld)
                         v += beta * old[r];
-                    buffer_store_out<half_t>((half_t)v, cr, (int)off);
+                    buffer_store_out<OutT>((OutT)v, cr, (int)off);
                 }
             }
         }
@@ -523,7 +527,7 @@ gemm_f16_direct_kernel(const GemmParams p)
         narrow(IntC<0>());
 }
 
-template <int CFG, bool AKC, bool BKC, bool CS>
+template <typename OutT, int CFG, bool AKC, bool BKC, bool CS>
 static int launch_f16_direct(const GemmParams & p0, hipStream_t stream)
 {
     typedef TileShape<CFG> S;
@@ -532,7 +536,7 @@ static int launch_f16_direct(const GemmParams & p0, hipStream_t stream)
     p.tilesN = (p.N + S::BN - 1) / S::BN;
     p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>),
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -547,23 +551,31 @@ static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
             return launch_f16_one<float, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
         return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
     }
-    /* half inputs with a float result are outside the main path: one generic instantiation */
-    if (outF32)
-        return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
-    if (!vec)
+    if (!vec) {
+        if (outF32)
+            return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
         return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
+    }
+    /* a float result: the same main loop, 4-byte stores from the accumulators */
+    if (outF32) {
+        if (cfg == CFG_256x256)
+            return launch_f16_direct<float, CFG_256x256, AKC, BKC, false>(p, stream);
+        if (cfg == CFG_128x128)
+            return launch_f16_direct<float, CFG_128x128, AKC, BKC, false>(p, stream);
+        return launch_f16_direct<float, CFG_64x64, AKC, BKC, false>(p, stream);
+    }
     /* column sums: the 256x256 tile has no registers to spare, and products that want column
        sums (weight gradients) are too small for it anyway */
     if (p.colSum != NULL) {
         if (cfg == CFG_64x64)
-            return launch_f16_direct<CFG_64x64, AKC, BKC, true>(p, stream);
-        return launch_f16_direct<CFG_128x128, AKC, BKC, true>(p, stream);
+            return launch_f16_direct<half_t, CFG_64x64, AKC, BKC, true>(p, stream);
+        return launch_f16_direct<half_t, CFG_128x128, AKC, BKC, true>(p, stream);
     }
     if (cfg == CFG_256x256)
-        return launch_f16_direct<CFG_256x256, AKC, BKC, false>(p, stream);
+        return launch_f16_direct<half_t, CFG_256x256, AKC, BKC, false>(p, stream);
     if (cfg == CFG_128x128)
-        return launch_f16_direct<CFG_128x128, AKC, BKC, false>(p, stream);
-    return launch_f16_direct<CFG_64x64, AKC, BKC, false>(p, stream);
+        return launch_f16_direct<half_t, CFG_128x128, AKC, BKC, false>(p, stream);
+    return launch_f16_direct<half_t, CFG_64x64, AKC, BKC, false>(p, stream);
 }
 
 }  // namespace ntsamd

@@ -252,7 +252,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column
        only. It keeps a tile's byte offsets in 31 bits, so rows longer than 2M elements
        go through the generic path, like everything unaligned and row-indexed bias */
-    bool vec = !ptrs && kind != KIND_F16_F32OUT &&
+    bool vec = !ptrs &&
                lda % vecElems == 0 && ldb % vecElems == 0 && aligned16(a) && aligned16(b) &&
                strideA % vecElems == 0 && strideB % vecElems == 0 &&
                lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) &&

@@ -218,6 +218,30 @@ def test_half_in_float_out(gpu, oracle):
     assert_fp32(c.cpu().numpy(), ref, 77)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_in_float_out_on_the_main_path(gpu, oracle, ta, tb):
+    """16-byte aligned half operands with a float result (a half product that feeds a softmax, as
+    the reference converts the scores and the output layer's logits to float): every tile shape,
+    ragged edges, beta, and a float bias by column. The products of halves are exact in fp32, so
+    the fp32 limit applies."""
+    torch = torch_()
+    for cfg in ("0", "1", "2"):
+        os.environ["NTSAMD_TILE_CFG"] = cfg
+        for i, (M, N, K) in enumerate([(8, 8, 8), (64, 72, 40), (136, 264, 96), (257, 120, 64), (300, 520, 128)]):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 7000 + i, 0, 0.5)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 7100 + i, 0, 0.5)))
+            c0 = oracle.uniform((M, N), 7200 + i)
+            bias = oracle.normal((N,), 7300 + i)
+            for alpha, beta, with_bias in ((1.0, 0.0, False), (0.5, 1.0, False), (1.0, 0.0, True)):
+                ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                if with_bias:
+                    ref = ref + bias[None, :]
+                c = dev_tensor(c0, gpu) if beta != 0 else torch.full((M, N), float("nan"), device=gpu)
+                nt.matrix_mul(dev_tensor(a, gpu, True), ta, dev_tensor(b, gpu, True), tb, c, alpha, beta,
+                              bias=dev_tensor(bias, gpu) if with_bias else None)
+                assert_fp32(c.cpu().numpy(), ref, K, what="cfg%s %dx%dx%d alpha=%g beta=%g bias=%s" % (cfg, M, N, K, alpha, beta, with_bias))
+
+
 def test_unaligned_operands_take_the_generic_path(gpu, oracle):
     """Base pointers and leading dimensions that rule out 16-byte loads."""
     torch = torch_()
