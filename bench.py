@@ -48,6 +48,9 @@ def configs():
         8: dict(name="cfg8 fp32 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v [32x128x512], 8 heads (cfg3 with the "
                      "softmax between its products and the head split/merge folded in)",
                 dtype="f32", M=128, N=128, K=64, batch=256),
+        9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
+                     "fp32 accumulation and softmax",
+                dtype="f16", M=128, N=128, K=64, batch=256),
     }
 
 
@@ -135,15 +138,16 @@ class Workload:
             self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
             self.bytes = 2 * 4.0 * 256 * (128 * 128 + 128 * 64 + 2 * 128 * 64)
             self.launches = 2
-        elif idx == 8:
-            self.q = g(oracle.normal((32, 128, 512), 1))
-            self.k = g(oracle.normal((32, 128, 512), 2))
-            self.v = g(oracle.normal((32, 128, 512), 3))
-            self.o = torch.empty((32, 128, 512), device=dev)
+        elif idx in (8, 9):
+            cast = (lambda t: t.half()) if idx == 9 else (lambda t: t)
+            self.q = cast(g(oracle.normal((32, 128, 512), 1)))
+            self.k = cast(g(oracle.normal((32, 128, 512), 2)))
+            self.v = cast(g(oracle.normal((32, 128, 512), 3)))
+            self.o = torch.empty((32, 128, 512), device=dev, dtype=self.q.dtype)
             self.run = lambda: nt.attention(self.q, self.k, self.v, self.o, 8, 0.125)
             self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
             # q, k, v read once, the result written once; the scores never reach memory
-            self.bytes = 4 * 4.0 * 32 * 128 * 512
+            self.bytes = 4 * (4.0 if idx == 8 else 2.0) * 32 * 128 * 512
             self.launches = 1
         else:
             raise SystemExit("no such configuration: %d" % idx)
@@ -183,7 +187,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -193,9 +197,12 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 4.0 * 128 * 128 * 64
         sample = "%d of 256 batch items, both products" % nb
-    elif idx == 8:
+    elif idx in (8, 9):
         nb = max(1, min(32, int(budget_s * rate / (8 * 4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 512), 1), o.normal((nb, 128, 512), 2), o.normal((nb, 128, 512), 3)
+        if idx == 9:
+            # fp32 arithmetic on the half-rounded values: the reference has no CPU half path
+            q, k, v = (o.from_f16_bits(o.to_f16_bits(t)) for t in (q, k, v))
         t0 = time.perf_counter()
         o.attention(q, k, v, 8, 0.125)
         dt = time.perf_counter() - t0
@@ -284,7 +291,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
     # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
-    if idx in (3, 7):
+    if idx in (3, 7, 9):
         roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
                 "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
     else:
@@ -323,7 +330,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-8 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 the one-kernel attention)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-9 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -351,7 +358,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

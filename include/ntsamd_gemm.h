@@ -175,14 +175,19 @@ int ntsamd_matrix_mul_batched(int devID, void * stream,
  * BMMul(att, v) (:232-235) and Merge of the heads (:239, core/shape/Merge.cpp). The scores
  * are never written to memory, and the head split and merge are addressing:
  *   element (h, b, row, col) of q is q[h * strides[0] + b * strides[1] + row * strides[2] + col],
- *   likewise strides[3..5] for k, [6..8] for v, [9..11] for out (in elements, multiples of 4).
+ *   likewise strides[3..5] for k, [6..8] for v, [9..11] for out (in elements).
  * For tensors stored [batch][rows][heads * dh], as before Split and after Merge, the strides
  * are (dh, rows * heads * dh, heads * dh); for tensors stored [heads][batch][rows][dh], as
  * after Split, they are (batch * rows * dh, rows * dh, dh).
- * q and out have lq rows, k and v have lk rows, every row has dh columns (dh a multiple of 4,
- * at most 128). mask is NULL or a dense X_FLOAT tensor [heads][batch][lq][lk] added to the
- * scaled scores (the reference's masks hold 0 and -1e9). dataType is X_FLOAT for q, k, v and
- * out. The training path of the reference applies dropout between the softmax and the second
+ * q and out have lq rows, k and v have lk rows, every row has dh columns (at most 128).
+ * mask is NULL or a dense X_FLOAT tensor [heads][batch][lq][lk] added to the scaled scores
+ * (the reference's masks hold 0 and -1e9). dataType is the type of q, k, v and out:
+ *   X_FLOAT    fp32 throughout; dh and the strides are multiples of 4.
+ *   X_FLOAT16  half products with fp32 accumulation, the softmax in fp32 on the unrounded scores,
+ *              probabilities and result rounded to half once each: the reference's half path
+ *              (:216-218 scores converted to float for the mask and the softmax, :229-230 back to
+ *              half) without its two conversion passes; dh and the strides are multiples of 8.
+ * The training path of the reference applies dropout between the softmax and the second
  * product (:226-227) and keeps the probabilities for the backward step: it stays on the
  * batched-product entry points above.
  */

@@ -8,11 +8,11 @@
 namespace ntsamd {
 
 struct AttnParams {
-    const float * q;
-    const float * k;
-    const float * v;
-    const float * mask;                 /* NULL, or dense [heads][batch][lq][lk] added to the scaled scores */
-    float * out;
+    const void * q;                     /* q, k, v, out: float or half, one type for all four */
+    const void * k;
+    const void * v;
+    const float * mask;                 /* NULL, or dense float [heads][batch][lq][lk] added to the scaled scores */
+    void * out;
     int heads, batch, lq, lk, dh;
     long long qH, qB, qL;               /* element strides: head, batch item, row (columns are contiguous) */
     long long kH, kB, kL;
@@ -24,5 +24,6 @@ struct AttnParams {
 };
 
 int launch_attention_f32(const AttnParams & p, hipStream_t stream);
+int launch_attention_f16(const AttnParams & p, hipStream_t stream);
 
 }  // namespace ntsamd

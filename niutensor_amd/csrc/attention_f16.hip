@@ -1,0 +1,266 @@
+/*
+ * out = softmax(scale * Q K^T + mask) V per head for half tensors, in one kernel for gfx950:
+ * half products with fp32 accumulation, the softmax in fp32, one rounding of the
+ * probabilities to half before the second product and one of the result.
+ *
+ * Stands where the reference's attention, run with half tensors, issues
+ * (source/sample/transformer/submodel/Attention.cpp:186-237) Split, ScaleMe,
+ * BMMul(q, k^T) in half, ConvertDataType to float (:216-218), the mask add and the Softmax
+ * in float, ConvertDataType back to half (:229-230), BMMul with v in half, Merge. The scores
+ * stay in fp32 registers from the first product to the softmax (the reference rounds them to
+ * half in between), so the two conversion passes and their tensors disappear.
+ *
+ * Same plan as the fp32 kernel (attention_f32.hip): 64 query rows of one (head, batch item)
+ * per workgroup, 16 per wave; keys and values stream through LDS in blocks of 128; both
+ * products are computed transposed so that the probabilities pass from accumulator to
+ * operand inside a lane:
+ *   S^T = K Q^T   v_mfma_f32_16x16x32_f16: lane (m, g) = (l%16, l/16) feeds key m / query m with the
+ *                 eight columns 32 t + 8 g .. + 7 (one 16-byte read) and receives the scores of query m
+ *                 against keys 16 j + 4 g + r, r = 0..3.
+ *   O^T = V^T P^T v_mfma_f32_16x16x16_f16: B wants four consecutive k per lane, k = 4 g + r: the four
+ *                 scores above, rounded to half. A wants V[key 16 j + 4 g + r][column m], four values
+ *                 one LDS row apart: a transposing read (ds_read_b64_tr_b16) of the 4 x 16 block whose
+ *                 rows the lane groups 0-3, 4-7, 8-11, 12-15 of every 16 lanes point at.
+ */
+#include "gemm_common.h"
+#include "gemm_f16.h"       /* half_t, make_rsrc, buffer_load_f16x8, lds_read_tr16 */
+#include "attention.h"
+
+namespace ntsamd {
+
+__device__ __forceinline__ float groups_max(float x)
+{
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
+}
+
+__device__ __forceinline__ float groups_sum(float x)
+{
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
+/* DHM: head size the kernel is built for (dh <= DHM, a multiple of 8; columns past dh are zero) */
+template <int DHM>
+__global__ void __launch_bounds__(256, 2)
+attention_f16_kernel(const AttnParams p)
+{
+    constexpr int KB = 128;                  /* keys per block */
+    constexpr int PITCH = DHM * 2 + 16;      /* bytes per LDS row: 16 mod 128, so 16-byte reads of consecutive rows
+                                                walk through the banks */
+    constexpr int NT = DHM / 32;             /* k steps of the first product */
+    constexpr int ND = DHM / 16;             /* 16-column blocks of the result */
+    constexpr int NJ = KB / 16;              /* 16-key blocks */
+    constexpr int TPR = DHM / 8;             /* threads per row when staging (16 bytes each) */
+    constexpr int RSTEP = 256 / TPR;
+    constexpr int LOADS = KB / RSTEP;
+    constexpr float LOG2E = 1.4426950408889634f;
+
+    __shared__ __attribute__((aligned(16))) char Ks[KB * PITCH];
+    __shared__ __attribute__((aligned(16))) char Vs[KB * PITCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 15, g = lane >> 4;
+
+    const int id = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
+    const int qt = id % p.qTiles;
+    const int pair = id / p.qTiles;
+    const int h = pair / p.batch, b = pair - h * p.batch;
+    const int lq = p.lq, lk = p.lk, dh = p.dh;
+
+    const half_t * Q = static_cast<const half_t *>(p.q) + h * p.qH + b * p.qB;
+    const half_t * K = static_cast<const half_t *>(p.k) + h * p.kH + b * p.kB;
+    const half_t * V = static_cast<const half_t *>(p.v) + h * p.vH + b * p.vB;
+    half_t * O = static_cast<half_t *>(p.out) + h * p.oH + b * p.oB;
+
+    const int row = qt * 64 + wave * 16 + m;
+    const int rowc = row < lq ? row : lq - 1;
+    const float * MK = p.mask ? p.mask + ((long long)pair * lq + rowc) * lk : nullptr;
+
+    /* ---- staging of keys and values, as in the fp32 kernel ---- */
+    const int sr0 = tid / TPR, sc = (tid % TPR) * 8;
+    const int sLds = sr0 * PITCH + sc * 2;
+    const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K, ((long long)(lk - 1) * p.kL + dh) * 2);
+    const __amdgpu_buffer_rsrc_t vRsrc = make_rsrc(V, ((long long)(lk - 1) * p.vL + dh) * 2);
+    const int kL2 = (int)p.kL * 2, vL2 = (int)p.vL * 2;
+    const int kOff0 = sr0 * kL2 + sc * 2, vOff0 = sr0 * vL2 + sc * 2;
+    f16x8 kreg[LOADS], vreg[LOADS];
+    auto load_k = [&](int kb0) {
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            kreg[s] = buffer_load_f16x8(kRsrc, sc < dh ? kOff0 + (kb0 + s * RSTEP) * kL2 : NTSAMD_OOB_OFFSET);
+    };
+    auto load_v = [&](int kb0) {
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            vreg[s] = buffer_load_f16x8(vRsrc, sc < dh ? vOff0 + (kb0 + s * RSTEP) * vL2 : NTSAMD_OOB_OFFSET);
+    };
+    load_k(0);
+
+    /* ---- Q fragments ---- */
+    f16x8 qf[NT];
+    {
+        const half_t * qr = Q + (long long)rowc * p.qL;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int c = 32 * t + 8 * g;
+            f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            qf[t] = c < dh ? *reinterpret_cast<const f16x8 *>(qr + c) : z;
+        }
+    }
+    load_v(0);
+
+    f32x4 accO[ND];
+#pragma unroll
+    for (int d = 0; d < ND; d++)
+        accO[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float rowMax = -INFINITY, rowSum = 0.f;
+    const float scale2 = p.scale * LOG2E;
+
+    /* where this lane points for the transposing reads: row 4 g + (m / 4) of a 16-key block, columns 4 (m % 4) .. + 3 */
+    const int trOff = (4 * g + (m >> 2)) * PITCH + (m & 3) * 8;
+
+    for (int kb0 = 0; kb0 < lk; kb0 += KB) {
+        const bool more = kb0 + KB < lk;
+
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            *reinterpret_cast<f16x8 *>(&Ks[sLds + s * RSTEP * PITCH]) = kreg[s];
+        __syncthreads();
+        if (more)
+            load_k(kb0 + KB);
+
+        /* ---- S^T = K Q^T ---- */
+        f32x4 accS[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+            accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const f16x8 kf = *reinterpret_cast<const f16x8 *>(&Ks[(16 * j + m) * PITCH + 64 * t + 16 * g]);
+                accS[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t], accS[j], 0, 0, 0);
+            }
+        }
+
+        /* ---- scale and mask ---- */
+        if (MK != nullptr) {
+            if (p.maskVec) {
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    const int key = kb0 + 16 * j + 4 * g;
+                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK + key) : z;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        accS[j][r] = fmaf(mk[r], LOG2E, accS[j][r] * scale2);
+                }
+            }
+            else {
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        int key = kb0 + 16 * j + 4 * g + r;
+                        key = key < lk ? key : lk - 1;
+                        accS[j][r] = fmaf(MK[key], LOG2E, accS[j][r] * scale2);
+                    }
+            }
+        }
+        else {
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    accS[j][r] *= scale2;
+        }
+        if (kb0 + KB > lk) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (kb0 + 16 * j + 4 * g + r >= lk)
+                        accS[j][r] = -INFINITY;
+        }
+
+        /* ---- running softmax of this lane's query row, in fp32 ---- */
+        float mx = accS[0][0];
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                mx = fmaxf(mx, accS[j][r]);
+        mx = groups_max(mx);
+        const float newMax = fmaxf(rowMax, mx);
+        const float shift = newMax == -INFINITY ? 0.f : newMax;
+        const float corr = __builtin_amdgcn_exp2f(rowMax - shift);
+        float sum = 0.f;
+        f16x4 pf[NJ];                                    /* the probabilities as the second product's operand */
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float e = __builtin_amdgcn_exp2f(accS[j][r] - shift);
+                sum += e;
+                pf[j][r] = (half_t)e;
+            }
+        sum = groups_sum(sum);
+        rowSum = rowSum * corr + sum;
+        rowMax = newMax;
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+            accO[d] *= corr;
+
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            *reinterpret_cast<f16x8 *>(&Vs[sLds + s * RSTEP * PITCH]) = vreg[s];
+        __syncthreads();
+        if (more)
+            load_v(kb0 + KB);
+
+        /* ---- O^T += V^T P^T ---- */
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int d = 0; d < ND; d++) {
+                const f16x4 vf = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * j * PITCH + trOff + 32 * d]));
+                accO[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf[j], accO[d], 0, 0, 0);
+            }
+    }
+
+    /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
+    if (row < lq) {
+        const float inv = rowSum > 0.f ? 1.f / rowSum : 0.f;
+        half_t * orow = O + (long long)row * p.oL;
+#pragma unroll
+        for (int d = 0; d < ND; d++) {
+            const int c = 16 * d + 4 * g;
+            if (c < dh) {
+                f16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    o[r] = (half_t)(accO[d][r] * inv);
+                *reinterpret_cast<f16x4 *>(orow + c) = o;
+            }
+        }
+    }
+}
+
+int launch_attention_f16(const AttnParams & p0, hipStream_t stream)
+{
+    AttnParams p = p0;
+    p.qTiles = (p.lq + 63) / 64;
+    p.maskVec = (p.mask != nullptr && p.lk % 4 == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 15) == 0) ? 1 : 0;
+    dim3 grid((unsigned)(p.heads * p.batch * p.qTiles));
+    if (p.dh <= 32)
+        hipLaunchKernelGGL((attention_f16_kernel<32>), grid, dim3(256), 0, stream, p);
+    else if (p.dh <= 64)
+        hipLaunchKernelGGL((attention_f16_kernel<64>), grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((attention_f16_kernel<128>), grid, dim3(256), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+}  // namespace ntsamd

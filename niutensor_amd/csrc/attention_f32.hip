@@ -76,10 +76,10 @@ attention_f32_kernel(const AttnParams p)
     const int h = pair / p.batch, b = pair - h * p.batch;
     const int lq = p.lq, lk = p.lk, dh = p.dh;
 
-    const float * Q = p.q + h * p.qH + b * p.qB;
-    const float * K = p.k + h * p.kH + b * p.kB;
-    const float * V = p.v + h * p.vH + b * p.vB;
-    float * O = p.out + h * p.oH + b * p.oB;
+    const float * Q = static_cast<const float *>(p.q) + h * p.qH + b * p.qB;
+    const float * K = static_cast<const float *>(p.k) + h * p.kH + b * p.kB;
+    const float * V = static_cast<const float *>(p.v) + h * p.vH + b * p.vB;
+    float * O = static_cast<float *>(p.out) + h * p.oH + b * p.oB;
 
     const int row = qt * 64 + wave * 16 + m;              /* this lane's query row */
     const int rowc = row < lq ? row : lq - 1;             /* rows past the end repeat the last one; never stored */

@@ -490,7 +490,7 @@ int ntsamd_attention(int devID, void * stream,
                      int heads, int batch, int lq, int lk, int dh,
                      const long long * strides, float scale)
 {
-    if (dataType != NTSAMD_X_FLOAT)
+    if (dataType != NTSAMD_X_FLOAT && dataType != NTSAMD_X_FLOAT16)
         return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
     if (heads < 0 || batch < 0 || lq < 0 || lk < 0 || dh < 0)
         return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
@@ -500,13 +500,18 @@ int ntsamd_attention(int devID, void * stream,
         return fail(NTSAMD_ERR_ARGUMENT, "attention over no keys");
     if (!q || !k || !v || !out || !strides)
         return fail(NTSAMD_ERR_ARGUMENT, "Empty input tensors!");
-    if (dh > 128 || dh % 4 != 0)
-        return fail(NTSAMD_ERR_ARGUMENT, "head size %d is not served by the fused kernel (a multiple of 4 up to 128 is)", dh);
+    /* rows are moved 16 bytes at a time: 4 floats or 8 halves */
+    const int vecElems = dataType == NTSAMD_X_FLOAT ? 4 : 8;
+    if (dh > 128 || dh % vecElems != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "head size %d is not served by the fused kernel (a multiple of %d up to 128 is)",
+                    dh, vecElems);
     for (int i = 0; i < 12; i++)
-        if (strides[i] < 0 || strides[i] % 4 != 0)
-            return fail(NTSAMD_ERR_ARGUMENT, "strides must be non-negative multiples of 4 elements");
+        if (strides[i] < 0 || strides[i] % vecElems != 0)
+            return fail(NTSAMD_ERR_ARGUMENT, "strides must be non-negative multiples of %d elements", vecElems);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
         return fail(NTSAMD_ERR_ARGUMENT, "q, k, v and out must be 16-byte aligned");
+    if (mask && (reinterpret_cast<uintptr_t>(mask) & 3) != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "misaligned mask");
     for (int t = 0; t < 4; t++)
         if (strides[3 * t + 2] < dh)
             return fail(NTSAMD_ERR_ARGUMENT, "row stride smaller than the head size");
@@ -524,11 +529,11 @@ int ntsamd_attention(int devID, void * stream,
         return scope.status;
     AttnParams p;
     memset(&p, 0, sizeof(p));
-    p.q = static_cast<const float *>(q);
-    p.k = static_cast<const float *>(k);
-    p.v = static_cast<const float *>(v);
+    p.q = q;
+    p.k = k;
+    p.v = v;
     p.mask = static_cast<const float *>(mask);
-    p.out = static_cast<float *>(out);
+    p.out = out;
     p.heads = heads;
     p.batch = batch;
     p.lq = lq;
@@ -539,7 +544,8 @@ int ntsamd_attention(int devID, void * stream,
     p.vH = strides[6]; p.vB = strides[7]; p.vL = strides[8];
     p.oH = strides[9]; p.oB = strides[10]; p.oL = strides[11];
     p.scale = scale;
-    int rc = launch_attention_f32(p, static_cast<hipStream_t>(stream));
+    int rc = dataType == NTSAMD_X_FLOAT ? launch_attention_f32(p, static_cast<hipStream_t>(stream))
+                                        : launch_attention_f16(p, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

@@ -14,8 +14,9 @@ void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, cons
                    XTensor * out, int nhead, DTYPE scale)
 {
     CheckNTErrors((q && k && v && out), "Empty input tensors!");
-    CheckNTErrors((q->dataType == X_FLOAT && k->dataType == X_FLOAT && v->dataType == X_FLOAT && out->dataType == X_FLOAT),
-                  "TODO!");
+    CheckNTErrors((q->dataType == X_FLOAT || q->dataType == X_FLOAT16), "TODO!");
+    CheckNTErrors((k->dataType == q->dataType && v->dataType == q->dataType && out->dataType == q->dataType),
+                  "Input tensors should have the same data type!");
     CheckNTErrors((q->order >= 2 && q->order == k->order && q->order == v->order && q->order == out->order),
                   "Input tensors must have the same order >= 2!");
     CheckNTErrors((q->devID >= 0), "This code must be run on GPUs!");
@@ -45,7 +46,7 @@ void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, cons
                              dh, (long long)lk * hidden, hidden,
                              dh, (long long)lq * hidden, hidden};
     int rc = ntsamd_attention(q->devID, NULL, q->data, k->data, v->data, mask != NULL ? mask->data : NULL, out->data,
-                              X_FLOAT, nhead, batch, lq, lk, dh, strides, scale);
+                              q->dataType, nhead, batch, lq, lk, dh, strides, scale);
     if (rc != NTSAMD_OK) {
         ShowNTErrors(ntsamd_last_error());
     }

@@ -12,7 +12,8 @@ namespace nts {
 
 /* out = Merge(Softmax(Split(q) * scale x Split(k)^T + mask, -1) x Split(v))
    q, out: (batch..., lq, hidden); k, v: (batch..., lk, hidden); nhead divides hidden;
-   mask: NULL or (nhead, batch..., lq, lk), added to the scaled scores. All X_FLOAT, one GPU. */
+   mask: NULL or an X_FLOAT tensor (nhead, batch..., lq, lk), added to the scaled scores.
+   q, k, v, out: all X_FLOAT or all X_FLOAT16 (half products, fp32 softmax); one GPU. */
 void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, const XTensor * mask,
                    XTensor * out, int nhead, DTYPE scale);
 

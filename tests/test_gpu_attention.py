@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import niutensor_amd as nt
-from tolerance import assert_fp32
+from tolerance import FP16_LIMIT, assert_fp32, normwise, scaled
 
 pytestmark = pytest.mark.gpu
 
@@ -124,6 +124,80 @@ def test_attention_shape_of_the_benchmark(gpu, oracle):
     assert np.abs(got - vc).max() <= 1e-5 * np.abs(vc).max() * 4
 
 
+def halfed(oracle, x):
+    return oracle.from_f16_bits(oracle.to_f16_bits(x))
+
+
+def assert_half(got, ref, mag, what):
+    """Limit 1e-2 (half against the fp32 reference), measured norm-wise and component-wise against
+    mag = sum_k p_k |v_k|: a result element is a sum of probabilities times values, each probability
+    enters the second product rounded to half (as in the reference's half path), so its error is a
+    multiple of 2^-11 mag however much of the sum cancels."""
+    assert np.isfinite(got).all(), what
+    e = normwise(got, ref)
+    assert e <= FP16_LIMIT, "%s: normwise error %.3g > %.3g" % (what, e, FP16_LIMIT)
+    e = scaled(got, ref, mag)
+    assert e <= FP16_LIMIT, "%s: component-wise error %.3g > %.3g" % (what, e, FP16_LIMIT)
+
+
+def run_half(gpu, q, k, v, heads, scale, mask=None):
+    torch = torch_()
+    out = torch.full(q.shape, float("nan"), device=gpu, dtype=torch.float16)
+    nt.attention(dev(q, gpu).half(), dev(k, gpu).half(), dev(v, gpu).half(), out, heads, scale,
+                 mask=dev(mask, gpu) if mask is not None else None)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
+    (2, 128, 128, 128, 2, False),      # head size 64, one key block
+    (3, 100, 77, 96, 3, True),         # head size 32, ragged rows and keys
+    (1, 300, 513, 64, 1, True),        # several query tiles and key blocks
+    (2, 40, 260, 256, 2, False),       # head size 128
+    (2, 33, 65, 80, 2, True),          # head size 40 inside the 64 kernel
+    (4, 9, 5, 16, 2, False),           # head size 8
+    (1, 1, 1, 8, 1, False),            # a single score
+])
+def test_half_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
+    """Half tensors: the fp32 oracle on the half-rounded inputs, result within 1e-2 (the limit the
+    task statement sets for half against the fp32 reference)."""
+    q, k, v = (halfed(oracle, oracle.normal(s, seed)) for s, seed in (((B, lq, H), 51), ((B, lk, H), 52), ((B, lk, H), 53)))
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 54, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., lk // 2] = 0.0
+    scale = float(np.float32(1.0 / np.sqrt(H // nh)))
+    ref = oracle.attention(q, k, v, nh, scale, mask)
+    mag = oracle.attention(q, k, np.abs(v), nh, scale, mask)
+    got = run_half(gpu, q, k, v, nh, scale, mask)
+    assert_half(got, ref, mag, str((B, lq, lk, H, nh, masked)))
+
+
+def test_half_exact_cases_and_benchmark_shape(gpu, oracle):
+    torch = torch_()
+    # one key: probabilities exactly 1, the result is v's row, bit for bit
+    B, lq, H, nh = 2, 70, 64, 2
+    q, k1, v1 = halfed(oracle, oracle.normal((B, lq, H), 61)), halfed(oracle, oracle.normal((B, 1, H), 62)), halfed(oracle, oracle.normal((B, 1, H), 63))
+    got = run_half(gpu, q, k1, v1, nh, 0.3)
+    assert np.array_equal(got, np.broadcast_to(v1, (B, lq, H)))
+    # scale 0: uniform probabilities (1/64 is exact in half), the result is the mean of v's rows
+    k, v = halfed(oracle, oracle.normal((B, 64, H), 64)), halfed(oracle, oracle.normal((B, 64, H), 65))
+    got = run_half(gpu, q, k, v, nh, 0.0)
+    mean = v.astype(np.float64).mean(1, keepdims=True)
+    assert np.abs(got - mean).max() <= 2e-3 * np.abs(mean).max() + 1e-3
+    # 32 sentences x 8 heads x 128 positions, head size 64; and the split layout gives the same bits
+    B, L, H, nh = 32, 128, 512, 8
+    q, k, v = (halfed(oracle, oracle.normal((B, L, H), s)) for s in (66, 67, 68))
+    ref = oracle.attention(q, k, v, nh, 0.125)
+    got = run_half(gpu, q, k, v, nh, 0.125)
+    assert_half(got, ref, oracle.attention(q, k, np.abs(v), nh, 0.125), "benchmark shape, half")
+    sp = lambda x: np.ascontiguousarray(x.reshape(B, L, nh, 64).transpose(2, 0, 1, 3))
+    out = torch.full((nh, B, L, 64), float("nan"), device=gpu, dtype=torch.float16)
+    nt.attention(dev(sp(q), gpu).half(), dev(sp(k), gpu).half(), dev(sp(v), gpu).half(), out, nh, 0.125, split=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy().transpose(1, 2, 0, 3).reshape(B, L, H), got)
+
+
 def test_bad_arguments_are_refused(gpu):
     torch = torch_()
     L = nt.load()
@@ -131,7 +205,9 @@ def test_bad_arguments_are_refused(gpu):
     t = torch.zeros(4096, device=gpu)
     st = (C.c_longlong * 12)(*([8, 64, 8] * 4))
     p = t.data_ptr()
-    assert L.ntsamd_attention(0, None, p, p, p, None, p, 3, 1, 1, 8, 8, 8, st, 1.0) == 2           # fp16: not served
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 4, 1, 1, 8, 8, 8, st, 1.0) == 2           # double: not served
+    st4 = (C.c_longlong * 12)(*([4, 64, 4] * 4))
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 3, 1, 1, 8, 8, 4, st4, 1.0) != 0          # half: head size 4
     assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 6, st, 1.0) != 0           # head size 6
     assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 132, st, 1.0) != 0         # head size 132
     assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 0, 8, st, 1.0) != 0           # no keys
