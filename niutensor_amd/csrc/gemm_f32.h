@@ -121,8 +121,10 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             aK[s] = g / (BM / 4);
             aMN[s] = (g % (BM / 4)) * 4;
             aLds[s] = aK[s] * BM + aMN[s];
-            int c = m0 + aMN[s] < M - 4 ? aMN[s] : M - 4 - m0;  /* 16-byte path: M % 4 == 0 */
-            aOff[s] = (aK[s] * p.lda + c) * 4;
+            /* four columns from aMN[s] on. A run that starts inside the row may end in the next one (rows
+               need not be multiples of four long): what it brings from there lands in columns past M,
+               whose results are never stored. A run that starts past the row reads as zero. */
+            aOff[s] = m0 + aMN[s] < M ? (aK[s] * p.lda + aMN[s]) * 4 : NTSAMD_OOB_OFFSET;
         }
     }
 #pragma unroll
@@ -140,8 +142,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             bK[s] = g / (BN / 4);
             bMN[s] = (g % (BN / 4)) * 4;
             bLds[s] = bK[s] * BN + bMN[s];
-            int c = n0 + bMN[s] < N - 4 ? bMN[s] : N - 4 - n0;
-            bOff[s] = (bK[s] * p.ldb + c) * 4;
+            bOff[s] = n0 + bMN[s] < N ? (bK[s] * p.ldb + bMN[s]) * 4 : NTSAMD_OOB_OFFSET;
         }
     }
 
@@ -178,6 +179,27 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                 if (BKC && tail && k0 + bK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
                 rb[s] = buffer_load_f32x4(br, off);
+            }
+            /* K need not be a multiple of four: the run that straddles it keeps its k < K only */
+            if constexpr (mayHangOver && AKC) {
+                if (tail) {
+#pragma unroll
+                    for (int s = 0; s < NA; s++)
+#pragma unroll
+                        for (int e = 1; e < 4; e++)
+                            if (k0 + aK[s] + e >= K)
+                                ra[s][e] = 0.f;
+                }
+            }
+            if constexpr (mayHangOver && BKC) {
+                if (tail) {
+#pragma unroll
+                    for (int s = 0; s < NB; s++)
+#pragma unroll
+                        for (int e = 1; e < 4; e++)
+                            if (k0 + bK[s] + e >= K)
+                                rb[s][e] = 0.f;
+                }
             }
         }
         else {

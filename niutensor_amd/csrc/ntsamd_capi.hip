@@ -248,15 +248,15 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.batch = count;
     p.groupM = 8;
 
-    const int vecElems = kind == KIND_F32 ? 4 : 8;
-    /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column
-       only. It keeps a tile's byte offsets in 31 bits, so rows longer than 2M elements
-       go through the generic path, like everything unaligned and row-indexed bias */
-    bool vec = !ptrs &&
-               lda % vecElems == 0 && ldb % vecElems == 0 && aligned16(a) && aligned16(b) &&
-               strideA % vecElems == 0 && strideB % vecElems == 0 &&
-               lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) &&
-               biasMode != NTSAMD_BIAS_ROW;
+    /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. It keeps a
+       tile's byte offsets in 31 bits, so rows longer than 2M elements go through the generic path, like
+       pointer lists and row-indexed bias. Float operands need no alignment beyond their own 4 bytes (a
+       16-byte buffer load may start on any dword, and is range-checked dword by dword); half operands
+       travel to LDS 16 bytes at a time and must have 16-byte aligned rows. */
+    bool vec = !ptrs && lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
+    if (kind != KIND_F32)
+        vec = vec && lda % 8 == 0 && ldb % 8 == 0 && aligned16(a) && aligned16(b) &&
+              strideA % 8 == 0 && strideB % 8 == 0;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight

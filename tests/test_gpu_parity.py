@@ -242,8 +242,67 @@ def test_half_in_float_out_on_the_main_path(gpu, oracle, ta, tb):
                 assert_fp32(c.cpu().numpy(), ref, K, what="cfg%s %dx%dx%d alpha=%g beta=%g bias=%s" % (cfg, M, N, K, alpha, beta, with_bias))
 
 
-def test_unaligned_operands_take_the_generic_path(gpu, oracle):
-    """Base pointers and leading dimensions that rule out 16-byte loads."""
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_fp32_rows_of_any_length_and_alignment(gpu, oracle, ta, tb):
+    """Float operands whose rows are not multiples of four long and whose first element sits on any
+    dword: k tails of 1, 2 and 3, ragged m and n, batches whose items start on odd elements. Both
+    operands lie inside larger buffers filled with NaN, so a read past either end of a matrix, or a
+    k >= K that is not discarded, would poison the result."""
+    torch = torch_()
+    for cfg in ("0", "1"):
+        os.environ["NTSAMD_TILE_CFG"] = cfg
+        for i, (M, N, K, shift) in enumerate([(129, 67, 33, 1), (70, 131, 130, 3), (255, 257, 63, 2), (3, 2, 1, 1), (64, 64, 515, 5)]):
+            a = oracle.uniform(stored((M, K), ta), 8100 + i)
+            b = oracle.uniform(stored((K, N), tb), 8200 + i)
+            c0 = oracle.uniform((M, N), 8300 + i)
+            abuf = torch.full((a.size + shift + 7,), float("nan"), device=gpu)
+            bbuf = torch.full((b.size + shift + 7,), float("nan"), device=gpu)
+            abuf[shift:shift + a.size] = dev_tensor(a.ravel(), gpu)
+            bbuf[shift:shift + b.size] = dev_tensor(b.ravel(), gpu)
+            av, bv = abuf[shift:shift + a.size].view(a.shape), bbuf[shift:shift + b.size].view(b.shape)
+            for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+                ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                c = dev_tensor(c0, gpu) if beta != 0 else torch.full((M, N), float("nan"), device=gpu)
+                nt.matrix_mul(av, ta, bv, tb, c, alpha, beta)
+                assert_fp32(c.cpu().numpy(), ref, K, magnitude(oracle, a, ta, b, tb, alpha, beta, c0),
+                            what="cfg%s %dx%dx%d shift %d alpha=%g beta=%g" % (cfg, M, N, K, shift, alpha, beta))
+    os.environ.pop("NTSAMD_TILE_CFG", None)
+    # a batch of products whose items are an odd number of elements apart
+    count, M, N, K = 5, 45, 51, 37
+    a = oracle.uniform((count,) + stored((M, K), ta), 8400)
+    b = oracle.uniform((count,) + stored((K, N), tb), 8401)
+    ref = oracle.matmul_batched(a, ta, b, tb, None, 0.75)
+    c = torch.full((count, M, N), float("nan"), device=gpu)
+    sa, sb = stored((M, K), ta), stored((K, N), tb)
+    nt.matrix_mul_batched_strided(dev_tensor(a, gpu), ta, dev_tensor(b, gpu), tb, c, count, M * K, K * N, M * N,
+                                  sa[0], sa[1], sb[0], sb[1], M, N, 0.75, 0.0)
+    assert_fp32(c.cpu().numpy(), ref, K, what="odd strides")
+
+
+def test_backward_of_the_ragged_vocabulary_projection(gpu, oracle):
+    """The two gradient products of configuration 5's layer: dE/dh = dE/dc w (k = 30011, rows of dE/dc
+    30011 long) and dE/dw = dE/dc^T h (m = 30011), beta = 1, checked on sampled rows in double precision."""
+    torch = torch_()
+    V = 30011
+    dy = oracle.normal((4096, V), 8500, 0, 0.1)
+    w = oracle.normal((V, 512), 8501, 0, 0.02)
+    h = oracle.uniform((4096, 512), 8502)
+    dh0, dw0 = oracle.uniform((4096, 512), 8503), oracle.uniform((V, 512), 8504)
+    dh, dw = dev_tensor(dh0, gpu), dev_tensor(dw0, gpu)
+    dyd = dev_tensor(dy, gpu)
+    nt.matrix_mul(dyd, X_NOTRANS, dev_tensor(w, gpu), X_NOTRANS, dh, 1.0, 1.0)
+    nt.matrix_mul(dyd, X_TRANS, dev_tensor(h, gpu), X_NOTRANS, dw, 1.0, 1.0)
+    rows = np.array([0, 1, 127, 128, 2047, 4095])
+    ref = dy[rows].astype(np.float64) @ w.astype(np.float64) + dh0[rows]
+    assert_fp32(dh.cpu().numpy()[rows], ref, V, what="dE/dh")
+    vr = np.array([0, 3, 127, 128, 30000, 30008, 30009, 30010])
+    ref = dy[:, vr].astype(np.float64).T @ h.astype(np.float64) + dw0[vr]
+    assert_fp32(dw.cpu().numpy()[vr], ref, 4096, what="dE/dw")
+
+
+def test_unaligned_operands(gpu, oracle):
+    """Base pointers and leading dimensions that are not multiples of 16 bytes (float: still the main
+    path; half: the generic path)."""
     torch = torch_()
     M, N, K = 70, 52, 36
     for ta, tb in TRANS:
