@@ -561,8 +561,12 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
 {
     NoPtrs none = {0};
     if (ptrs) {
-        /* pointer lists are the rare path: one instantiation, element-wise loads */
-        return launch_f32_one<CFG_64x64, AKC, BKC, false, false, PtrBatch>(p, *ptrs, stream);
+        /* a list of matrices: the same kernels, each workgroup looks its matrices up in the argument block */
+        if (!vec)
+            return launch_f32_one<CFG_64x64, AKC, BKC, false, false, PtrBatch>(p, *ptrs, stream);
+        if (cfg == CFG_128x128)
+            return launch_f32_one<CFG_128x128, AKC, BKC, true, false, PtrBatch>(p, *ptrs, stream);
+        return launch_f32_one<CFG_64x64, AKC, BKC, true, false, PtrBatch>(p, *ptrs, stream);
     }
     if (!vec)
         return launch_f32_one<CFG_64x64, AKC, BKC, false, false, NoPtrs>(p, none, stream);

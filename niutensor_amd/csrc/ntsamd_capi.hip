@@ -250,18 +250,18 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
 
     /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. It keeps a
        tile's byte offsets in 31 bits, so rows longer than 2M elements go through the generic path, like
-       pointer lists and row-indexed bias. Float operands need no alignment beyond their own 4 bytes (a
+       row-indexed bias and lists of half matrices. Float operands need no alignment beyond their own 4 bytes (a
        16-byte buffer load may start on any dword, and is range-checked dword by dword); half operands
        travel to LDS 16 bytes at a time and must have 16-byte aligned rows. */
-    bool vec = !ptrs && lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
+    bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
     if (kind != KIND_F32)
-        vec = vec && lda % 8 == 0 && ldb % 8 == 0 && aligned16(a) && aligned16(b) &&
+        vec = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && aligned16(a) && aligned16(b) &&
               strideA % 8 == 0 && strideB % 8 == 0;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
-    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec);
+    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec && !ptrs);
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;
