@@ -109,7 +109,6 @@ attention_f16_kernel(const AttnParams p)
             qf[t] = c < dh ? *reinterpret_cast<const f16x8 *>(qr + c) : z;
         }
     }
-    load_v(0);
 
     f32x4 accO[ND];
 #pragma unroll
@@ -128,6 +127,10 @@ attention_f16_kernel(const AttnParams p)
         for (int s = 0; s < LOADS; s++)
             *reinterpret_cast<f16x8 *>(&Ks[sLds + s * RSTEP * PITCH]) = kreg[s];
         __syncthreads();
+        /* the first values are asked for only now: at the start every workgroup of the grid wants its keys and
+           queries at once, and values queued among them would hold back the keys of the workgroups that start later */
+        if (kb0 == 0)
+            load_v(0);
         if (more)
             load_k(kb0 + KB);
 

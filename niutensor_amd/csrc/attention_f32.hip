@@ -121,7 +121,6 @@ attention_f32_kernel(const AttnParams p)
             qf[t] = c < dh ? *reinterpret_cast<const f32x4 *>(qr + c) : z;
         }
     }
-    load_v(0);
 
     f32x4 accO[NT];
 #pragma unroll
@@ -138,6 +137,10 @@ attention_f32_kernel(const AttnParams p)
         for (int s = 0; s < LOADS; s++)
             *reinterpret_cast<f32x4 *>(&Ks[sLds + s * RSTEP * KP]) = kreg[s];
         __syncthreads();                                 /* also: every wave has finished the previous block's Vs */
+        /* the first values are asked for only now: at the start every workgroup of the grid wants its keys and
+           queries at once, and values queued among them would hold back the keys of the workgroups that start later */
+        if (kb0 == 0)
+            load_v(0);
         if (more)
             load_k(kb0 + KB);
 
