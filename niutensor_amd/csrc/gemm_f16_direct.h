@@ -19,14 +19,14 @@
  *       consecutive k rows of one transposing read sit in four different chunks,
  *       32 bytes apart modulo 128.
  *
- * Pipeline: loads for slab t+3 are issued while slab t is multiplied (about 2.5
- * slabs = 2500 cycles of cover for the global latency). A slab is two MFMA k
- * steps; its fragments are double-buffered per k step. The one barrier of a slab
- * sits between the two steps: by then the wave has waited for its own loads of
- * slab t+1 (vmcnt) and for its own last reads of slab t (lgkmcnt), so after the
- * barrier every wave may read slab t+1 and, one step later, overwrite the stage
- * of slab t-1... and the MFMAs of the second step are ready to issue the moment
- * the barrier opens, because their fragments were read before it.
+ * Pipeline: loads for slab t+4 are issued during the second k step of slab t, the
+ * moment the stage of slab t is free (about 3 slabs = 3000 cycles of cover for the
+ * global latency). A slab is two MFMA k steps; its fragments are double-buffered
+ * per k step. The one barrier of a slab sits between the two steps: by then the
+ * wave has waited for its own loads of slab t+1 (vmcnt) and for its own last reads
+ * of slab t (lgkmcnt), so after the barrier every wave may read slab t+1 and
+ * overwrite the stage of slab t, and the MFMAs of the second step are ready to
+ * issue the moment the barrier opens, because their fragments were read before it.
  */
 #pragma once
 #include "gemm_common.h"
@@ -305,15 +305,15 @@ gemm_f16_direct_kernel(const GemmParams p)
         }
     };
 
-    /* One slab. AHEAD = how many later slabs exist (capped at 3): decides which loads are
+    /* One slab. AHEAD = how many later slabs exist (capped at 4): decides which loads are
        issued and how many may still be in flight at the barrier. */
     auto slab = [&](auto AHEADC, auto TAILC, int kt) {
         constexpr int ahead = decltype(AHEADC)::value;
         const char * stage = lds + (kt % NSTAGE) * STAGE;
         const char * next = lds + ((kt + 1) % NSTAGE) * STAGE;
 
-        /* k step 0: multiply it, fetch step 1 of this slab, start the loads of slab kt+3 */
-        k_step(IntC<0>(), IntC<1>(), IntC<(ahead >= 3)>(), TAILC, stage, kt + 3);
+        /* k step 0: multiply it, fetch step 1 of this slab */
+        k_step(IntC<0>(), IntC<1>(), IntC<0>(), TAILC, stage, 0);
         __builtin_amdgcn_sched_barrier(0);
 
         /* slab kt+1 must have landed: at most the loads of slabs kt+2 and kt+3 stay in flight */
@@ -327,19 +327,26 @@ gemm_f16_direct_kernel(const GemmParams p)
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
 
-        /* k step 1: multiply it, fetch step 0 of the next slab */
-        k_step(IntC<1>(), IntC<(ahead >= 1)>(), IntC<0>(), TAILC, next, 0);
+        /* k step 1: multiply it, fetch step 0 of the next slab. Every wave has read the last fragment of
+           this slab's stage before the barrier (its second step's fragments were fetched during the first),
+           so the stage is free from here on: the loads of slab kt+4 go into it now, half a slab earlier
+           than if they waited for the next slab to begin */
+        k_step(IntC<1>(), IntC<(ahead >= 1)>(), IntC<(ahead >= 4)>(), TAILC, next, kt + 4);
         __builtin_amdgcn_sched_barrier(0);
     };
 
     if (nk > 0) {
-        /* prologue: three slabs in flight, then wait for the first */
+        /* prologue: all four stages in flight, then wait for the first */
         issue_loads(IntC<1>(), 0);
         if (nk > 1)
             issue_loads(IntC<1>(), 1);
         if (nk > 2)
             issue_loads(IntC<1>(), 2);
-        if (nk > 2)
+        if (nk > 3)
+            issue_loads(IntC<1>(), 3);
+        if (nk > 3)
+            wait_vmcnt<3 * NL>();
+        else if (nk > 2)
             wait_vmcnt<2 * NL>();
         else if (nk > 1)
             wait_vmcnt<NL>();
@@ -351,10 +358,14 @@ gemm_f16_direct_kernel(const GemmParams p)
 
         const int nkFull = K / BKT;              /* slabs entirely inside K */
         int kt = 0;
-        for (; kt + 3 < nkFull; kt++)
-            slab(IntC<3>(), IntC<0>(), kt);      /* slab kt+3 is complete: no tail handling */
-        for (; kt + 3 < nk; kt++)
-            slab(IntC<3>(), IntC<1>(), kt);
+        for (; kt + 4 < nkFull; kt++)
+            slab(IntC<4>(), IntC<0>(), kt);      /* slab kt+4 is complete: no tail handling */
+        for (; kt + 4 < nk; kt++)
+            slab(IntC<4>(), IntC<1>(), kt);
+        if (kt + 3 < nk) {
+            slab(IntC<3>(), IntC<0>(), kt);
+            kt++;
+        }
         if (kt + 2 < nk) {
             slab(IntC<2>(), IntC<0>(), kt);
             kt++;
