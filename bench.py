@@ -48,6 +48,8 @@ def configs():
         8: dict(name="cfg8 fp32 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v [32x128x512], 8 heads (cfg3 with the "
                      "softmax between its products and the head split/merge folded in)",
                 dtype="f32", M=128, N=128, K=64, batch=256),
+        10: dict(name="cfg10 fp32 Rectify(MulAndShift(X[32x128x512], W[512x2048], b[2048])) in one kernel (first step of the feed-forward block)",
+                 dtype="f32", M=4096, N=2048, K=512, batch=1),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -64,15 +66,16 @@ class Workload:
         self.cfg = configs()[idx]
         T, NT = nt.X_TRANS, nt.X_NOTRANS
         g = lambda x: torch.from_numpy(x).to(dev)
-        if idx in (1, 2):
+        if idx in (1, 2, 10):
             self.x = g(oracle.uniform((4096, 512), 1))
             self.w = g(oracle.uniform((512, 2048), 2) if idx == 1 else oracle.normal((512, 2048), 2, 0, 0.02))
             self.b = g(oracle.normal((2048,), 3, 0, 0.02))
             self.c = torch.full((4096, 2048), float("nan"), device=dev)
-            bias = self.b if idx == 2 else None
-            self.run = lambda: nt.matrix_mul(self.x, NT, self.w, NT, self.c, 1.0, 0.0, bias=bias)
+            bias = self.b if idx != 1 else None
+            act = nt.ACT_RECTIFY if idx == 10 else nt.ACT_NONE
+            self.run = lambda: nt.matrix_mul(self.x, NT, self.w, NT, self.c, 1.0, 0.0, bias=bias, act=act)
             self.flops = 2.0 * 4096 * 2048 * 512
-            self.bytes = 4.0 * (4096 * 512 + 512 * 2048 + 4096 * 2048) + (8192 if idx == 2 else 0)
+            self.bytes = 4.0 * (4096 * 512 + 512 * 2048 + 4096 * 2048) + (8192 if idx != 1 else 0)
             self.launches = 1
         elif idx == 3:
             self.q = g(oracle.normal((256, 128, 64), 1))
@@ -186,7 +189,7 @@ def cpu_baseline(idx, budget_s=12.0):
     # the forward configurations in float run the REAL reference (its CPU sources compiled by oracle/Makefile into
     # oracle/_ref, which travels with the tree) when that library is there; the others (half: the reference has no
     # CPU half arithmetic; the gradient steps) and a tree without it run the restatement
-    use_ref = idx in (1, 2, 3, 5, 8) and Reference.available()
+    use_ref = idx in (1, 2, 3, 5, 8, 10) and Reference.available()
     o = Reference() if use_ref else gen
     if use_ref:
         o.uniform, o.normal = gen.uniform, gen.normal
@@ -196,7 +199,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -237,14 +240,16 @@ def cpu_baseline(idx, budget_s=12.0):
         sample = "%d of %d rows of x and dE/dc, all of w: both gradient products and the bias sums" % (rows, M)
     else:
         rows = max(8, min(M, int(budget_s * rate / (2.0 * N * K))))
-        if idx in (1, 2):
+        if idx in (1, 2, 10):
             a, b = o.uniform((rows, K), 1), o.uniform((K, N), 2)
             bias = o.normal((N,), 3, 0, 0.02)
             t0 = time.perf_counter()
             if idx == 1:
                 o.matmul2d(a, X_NOTRANS, b, X_NOTRANS)
-            else:
+            elif idx == 2:
                 o.mulandshift(a.reshape(1, rows, K), b, bias)
+            else:
+                o.rectify(o.mulandshift(a.reshape(1, rows, K), b, bias)[0])
             dt = time.perf_counter() - t0
         elif idx == 4:
             # fp32 arithmetic on the half-rounded values: the reference has no CPU half product
@@ -339,7 +344,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-9 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-10 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -367,7 +372,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

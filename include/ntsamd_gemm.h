@@ -57,6 +57,10 @@ extern "C" {
 #define NTSAMD_BIAS_COL 1         /* c[i][j] += bias[j]                      */
 #define NTSAMD_BIAS_ROW 2         /* c[i][j] += bias[(i / rowDiv) % biasLen] */
 
+/* function applied to every result element of ntsamd_matrix_mul_bias_act */
+#define NTSAMD_ACT_NONE 0
+#define NTSAMD_ACT_RECTIFY 1      /* y = x < 0 ? 0 : x */
+
 /* Message of the last failure on this thread ("" if none). */
 const char * ntsamd_last_error(void);
 
@@ -100,6 +104,24 @@ int ntsamd_matrix_mul_bias(int devID, void * stream,
                            int na, int ma, int nb, int mb, int nc, int mc,
                            float alpha, float beta,
                            const void * bias, int biasMode, int biasLen, int biasRowDiv);
+
+/*
+ * The same with a function applied to the result on its way out:
+ *   c = f(alpha * op(a) * op(b) + beta * c + broadcast(bias)).
+ * NTSAMD_ACT_RECTIFY is the reference's Rectify (source/tensor/function/Rectify.cpp:34-56,
+ * _CudaRectify Rectify.cu:39-83): the feed-forward block computes
+ * Rectify(MulAndShift(input, w1, b1)) (source/sample/transformer/submodel/FFN.cpp:94), which
+ * in the reference is the product, the broadcast add and then a third pass that reads and
+ * writes the whole hidden activation once more. A negative zero and a NaN pass unchanged, as
+ * in the reference's kernel (x < 0 is false for both).
+ */
+int ntsamd_matrix_mul_bias_act(int devID, void * stream,
+                               const void * a, int transposedA, int dataTypeA,
+                               const void * b, int transposedB, int dataTypeB,
+                               void * c, int dataTypeC,
+                               int na, int ma, int nb, int mb, int nc, int mc,
+                               float alpha, float beta,
+                               const void * bias, int biasMode, int biasLen, int biasRowDiv, int activation);
 
 /*
  * One product that also returns the column sums of op(b), gathered from the

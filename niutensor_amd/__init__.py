@@ -17,6 +17,7 @@ HOST_LIB_PATH = os.path.join(HERE, "lib", "libnts_amd.so")
 X_TRANS, X_NOTRANS = 0, 1           # MATRIX_TRANS_TYPE, source/tensor/XDataType.h:36
 X_INT, X_FLOAT, X_FLOAT16 = 0, 2, 3  # TENSOR_DATA_TYPE, source/tensor/XDataType.h:33
 BIAS_NONE, BIAS_COL, BIAS_ROW = 0, 1, 2
+ACT_NONE, ACT_RECTIFY = 0, 1
 
 EXPORTS = (
     "ntsamd_last_error",
@@ -24,6 +25,7 @@ EXPORTS = (
     "ntsamd_init",
     "ntsamd_matrix_mul",
     "ntsamd_matrix_mul_bias",
+    "ntsamd_matrix_mul_bias_act",
     "ntsamd_matrix_mul_batched_strided",
     "ntsamd_matrix_mul_batched",
     "ntsamd_matrix_mul_colsum",
@@ -60,6 +62,7 @@ def load():
     L.ntsamd_init.argtypes = [ci]
     L.ntsamd_matrix_mul.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_bias.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, ci, ci, ci]
+    L.ntsamd_matrix_mul_bias_act.argtypes = L.ntsamd_matrix_mul_bias.argtypes + [ci]
     L.ntsamd_matrix_mul_batched_strided.argtypes = [ci, vp, vp, ci, ci, ll, vp, ci, ci, ll, vp, ci, ll,
                                                     ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_batched.argtypes = [ci, vp, C.POINTER(vp), ci, ci, C.POINTER(vp), ci, ci, C.POINTER(vp), ci,
@@ -101,8 +104,9 @@ def _mat(t):
     return int(t.shape[-2]), int(t.shape[-1])
 
 
-def matrix_mul(a, transA, b, transB, c, alpha=1.0, beta=0.0, bias=None, bias_mode=BIAS_COL, bias_row_div=1):
-    """c = alpha * op(a) op(b) + beta * c (+ bias) on 2-D device tensors, through the C ABI."""
+def matrix_mul(a, transA, b, transB, c, alpha=1.0, beta=0.0, bias=None, bias_mode=BIAS_COL, bias_row_div=1, act=ACT_NONE):
+    """c = f(alpha * op(a) op(b) + beta * c (+ bias)) on 2-D device tensors, through the C ABI;
+    f is the identity or, with act=ACT_RECTIFY (needs a bias), max(0, .)."""
     L = load()
     na, ma = _mat(a)
     nb, mb = _mat(b)
@@ -113,10 +117,10 @@ def matrix_mul(a, transA, b, transB, c, alpha=1.0, beta=0.0, bias=None, bias_mod
                                  b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
                                  na, ma, nb, mb, nc, mc, alpha, beta)
     else:
-        rc = L.ntsamd_matrix_mul_bias(dev, _stream_ptr(a), a.data_ptr(), transA, _dtype_code(a),
-                                      b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
-                                      na, ma, nb, mb, nc, mc, alpha, beta,
-                                      bias.data_ptr(), bias_mode, bias.numel(), bias_row_div)
+        rc = L.ntsamd_matrix_mul_bias_act(dev, _stream_ptr(a), a.data_ptr(), transA, _dtype_code(a),
+                                          b.data_ptr(), transB, _dtype_code(b), c.data_ptr(), _dtype_code(c),
+                                          na, ma, nb, mb, nc, mc, alpha, beta,
+                                          bias.data_ptr(), bias_mode, bias.numel(), bias_row_div, act)
     _check(rc)
     return c
 

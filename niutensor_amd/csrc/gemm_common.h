@@ -22,6 +22,14 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 enum BiasMode { BIAS_NONE = 0, BIAS_COL = 1, BIAS_ROW = 2 };
 
+/* applied to a result element on its way out: y = x < 0 ? 0 : x is the reference's Rectify
+   (source/tensor/function/Rectify.cpp:47-55, Rectify.cu:39-49; a NaN stays a NaN) */
+enum Activation { ACT_NONE = 0, ACT_RECTIFY = 1 };
+__device__ __forceinline__ float activate(float v, int act)
+{
+    return (act == ACT_RECTIFY && v < 0.f) ? 0.f : v;
+}
+
 /* pointer-array batches travel in the kernel argument block: no device
    allocation, no host-to-device copy. One launch covers PTR_BATCH_MAX items. */
 #define NTSAMD_PTR_BATCH_MAX 128
@@ -56,6 +64,7 @@ struct GemmParams {
        depth), one workgroup each, which ADD alpha * (their partial product) to c with atomics;
        the caller has already applied beta to c. 1 = one workgroup per tile, plain stores. */
     int splits, kPerSplit;
+    int act;                               /* Activation of the epilogue */
 };
 
 /* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and

@@ -414,7 +414,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                     float v = alpha * acc[i][j][r] + bcol;
                     if (beta != 0.f)
                         v += beta * buffer_load_out<OutT>(cr, (int)off);
-                    buffer_store_out<OutT>((OutT)v, cr, (int)off);
+                    buffer_store_out<OutT>((OutT)activate(v, p.act), cr, (int)off);
                 }
             }
         }
@@ -443,7 +443,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                             v += (float)bias[(row / p.biasRowDiv) % p.biasLen];
                         else
                             v += bcol;
-                        *cp = (OutT)v;
+                        *cp = (OutT)activate(v, p.act);
                     }
                 }
             }

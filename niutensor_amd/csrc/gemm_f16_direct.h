@@ -389,6 +389,7 @@ gemm_f16_direct_kernel(const GemmParams p)
     const float alpha = p.alpha, beta = p.beta;
     const OutT * __restrict__ bias = static_cast<const OutT *>(p.bias);     /* the bias has the type of c */
     const int biasMode = p.biasMode;
+    const int act = p.act;
     OutT * cw = C + (size_t)(m0 + wm0) * p.ldc;
     const unsigned rowPitch = (unsigned)p.ldc * (unsigned)sizeof(OutT);
 
@@ -457,7 +458,7 @@ gemm_f16_direct_kernel(const GemmParams p)
                     for (int r = 0; r < 16; r++) {
                         const int row = 8 * (r / 4) + 4 * lhE + (r % 4);
                         *reinterpret_cast<StageT *>(buf + row * PITCH + (j * 32 + l32E) * (int)sizeof(StageT)) =
-                            (StageT)(alpha * acc[i][j][r] + bcol[j]);
+                            (StageT)(useOld ? alpha * acc[i][j][r] + bcol[j] : activate(alpha * acc[i][j][r] + bcol[j], act));
                     }
                 /* the wave's own lanes exchange data through LDS: LDS executes one wave's
                    instructions in order, the fences only keep the compiler from reordering */
@@ -475,8 +476,8 @@ gemm_f16_direct_kernel(const GemmParams p)
                         f16x8 v;
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            v[e] = (half_t)(lo[e] + beta * (float)o[e]);
-                            v[4 + e] = (half_t)(hi[e] + beta * (float)o[4 + e]);
+                            v[e] = (half_t)activate(lo[e] + beta * (float)o[e], act);
+                            v[4 + e] = (half_t)activate(hi[e] + beta * (float)o[4 + e], act);
                         }
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(f32x4, v), cr, (int)off, 0, 0);
                     }
@@ -527,7 +528,7 @@ gemm_f16_direct_kernel(const GemmParams p)
                     float v = alpha * acc[i][j][r] + bcol;
                     if constexpr (useOld)
                         v += beta * old[r];
-                    buffer_store_out<OutT>((OutT)v, cr, (int)off);
+                    buffer_store_out<OutT>((OutT)activate(v, act), cr, (int)off);
                 }
             }
         }

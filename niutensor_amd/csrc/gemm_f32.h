@@ -412,6 +412,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     const float alpha = p.alpha, beta = p.beta;
     const float * __restrict__ bias = static_cast<const float *>(p.bias);
     const int biasMode = p.biasMode;
+    const int act = p.act;
 
     if constexpr (VEC) {
         /* The wave's rows of c as one buffer that ends where c ends: rows past M drop
@@ -490,7 +491,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
-                        const float v = alpha * acc[i][j][r] + bcol[j] + beta * old[i][j][r];
+                        const float v = activate(alpha * acc[i][j][r] + bcol[j] + beta * old[i][j][r], act);
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
                     }
         }
@@ -502,7 +503,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
-                        const float v = alpha * acc[i][j][r] + bcol[j];
+                        const float v = activate(alpha * acc[i][j][r] + bcol[j], act);
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
                     }
         }
@@ -533,7 +534,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                             v += bias[((rowBase + dr) / p.biasRowDiv) % p.biasLen];
                         else
                             v += bcol;
-                        *cp = v;
+                        *cp = activate(v, act);
                     }
                 }
             }

@@ -213,7 +213,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         const PtrBatch * ptrs,
         float alpha, float beta,
         const void * bias, int biasMode, int biasLen, int biasRowDiv,
-        void * colSum = NULL, float colSumBeta = 0.f)
+        void * colSum = NULL, float colSumBeta = 0.f, int act = ACT_NONE)
 {
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
@@ -247,6 +247,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.biasLen = biasLen > 0 ? biasLen : 1;
     p.batch = count;
     p.groupM = 8;
+    p.act = act;
 
     /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. It keeps a
        tile's byte offsets in 31 bits, so rows longer than 2M elements go through the generic path, like
@@ -261,7 +262,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
-    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec && !ptrs);
+    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec && !ptrs && act == ACT_NONE);
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;
@@ -354,6 +355,21 @@ int ntsamd_matrix_mul_bias(int devID, void * stream,
                            float alpha, float beta,
                            const void * bias, int biasMode, int biasLen, int biasRowDiv)
 {
+    return ntsamd_matrix_mul_bias_act(devID, stream, a, transposedA, dataTypeA, b, transposedB, dataTypeB,
+                                      c, dataTypeC, na, ma, nb, mb, nc, mc, alpha, beta,
+                                      bias, biasMode, biasLen, biasRowDiv, NTSAMD_ACT_NONE);
+}
+
+int ntsamd_matrix_mul_bias_act(int devID, void * stream,
+                               const void * a, int transposedA, int dataTypeA,
+                               const void * b, int transposedB, int dataTypeB,
+                               void * c, int dataTypeC,
+                               int na, int ma, int nb, int mb, int nc, int mc,
+                               float alpha, float beta,
+                               const void * bias, int biasMode, int biasLen, int biasRowDiv, int activation)
+{
+    if (activation != NTSAMD_ACT_NONE && activation != NTSAMD_ACT_RECTIFY)
+        return fail(NTSAMD_ERR_ARGUMENT, "unknown activation %d", activation);
     Kind kind;
     Shape s;
     int st = check_types(dataTypeA, dataTypeB, dataTypeC, kind);
@@ -377,7 +393,7 @@ int ntsamd_matrix_mul_bias(int devID, void * stream,
             return fail(NTSAMD_ERR_ARGUMENT, "bias row divisor must be positive");
     }
     return run(devID, stream, kind, s, a, b, c, ma, mb, mc, 0, 0, 0, 1, NULL, alpha, beta,
-               biasMode == NTSAMD_BIAS_NONE ? NULL : bias, biasMode, biasLen, biasRowDiv);
+               biasMode == NTSAMD_BIAS_NONE ? NULL : bias, biasMode, biasLen, biasRowDiv, NULL, 0.f, activation);
 }
 
 int ntsamd_matrix_mul_colsum(int devID, void * stream,

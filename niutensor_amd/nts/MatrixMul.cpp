@@ -54,6 +54,7 @@ static BiasSpec RowOrColumnBias(const XTensor * c, const XTensor * bias, int n, 
        (row / product of the dimensions between n and the last) mod dimSize[n] */
     BiasSpec s;
     s.data = bias->data;
+    s.act = 0;
     if (n == SCALAR_BIAS) {
         s.mode = 2;
         s.len = 1;
@@ -75,7 +76,7 @@ static BiasSpec RowOrColumnBias(const XTensor * c, const XTensor * bias, int n, 
 }
 
 void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
-                    XTensor * c, DTYPE alpha, DTYPE beta, const XTensor * bias, int n)
+                    XTensor * c, DTYPE alpha, DTYPE beta, const XTensor * bias, int n, int act)
 {
     CheckNTErrors(a && b && c, "Empty input tensors!");
     CheckNTErrors(a->dataType == b->dataType && a->dataType == c->dataType,
@@ -101,6 +102,7 @@ void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
             _MatrixMul2D(a2, transposedA, b, transposedB, c2, alpha, beta);
         else {
             BiasSpec spec = RowOrColumnBias(c, bias, n, c->order - 2);
+            spec.act = act;
             CheckNTErrors(a2->devID >= 0, "Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
             _AmdMatrixMul2DBias(a2, transposedA, b, transposedB, c2, alpha, beta, &spec);
         }
@@ -168,6 +170,7 @@ void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
                     spec.len = 1;
                     spec.rowDiv = 1;
                 }
+                spec.act = act;
                 _AmdMatrixMul2DBias(ai, transposedA, bi, transposedB, ci, alpha, beta, &spec);
             }
         }

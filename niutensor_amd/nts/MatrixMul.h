@@ -35,10 +35,11 @@ bool CheckMMulShape(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
 
 /* _MatrixMul with the broadcast add of `bias` along dimension n of c fused into
    the product (bias == NULL: plain _MatrixMul; n == SCALAR_BIAS: a one-element
-   bias added to every element). Used by MulAndShift. */
+   bias added to every element). act == 1 applies Rectify to the result on its way out (needs a
+   bias: the epilogue is the fused one). Used by MulAndShift and MulAndShiftRectify. */
 #define SCALAR_BIAS (-2)
 void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
-                    XTensor * c, DTYPE alpha, DTYPE beta, const XTensor * bias, int n);
+                    XTensor * c, DTYPE alpha, DTYPE beta, const XTensor * bias, int n, int act = 0);
 
 }  // namespace nts
 #endif

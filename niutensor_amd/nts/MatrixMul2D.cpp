@@ -64,7 +64,7 @@ void _AmdMatrixMul2DBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const
             _AmdMatrixMULBias(a->devID, a->data, transposedA, a->dataType, b->data, transposedB, a->dataType,
                               c->data, c->dataType,
                               a->dimSize[0], a->dimSize[1], b->dimSize[0], b->dimSize[1], c->dimSize[0], c->dimSize[1],
-                              alpha, beta, bias->data, bias->mode, bias->len, bias->rowDiv);
+                              alpha, beta, bias->data, bias->mode, bias->len, bias->rowDiv, bias->act);
     }
     else {
         ShowNTErrors("TODO!");

@@ -20,6 +20,7 @@ struct BiasSpec {
     int mode;      /* 1: bias[column]; 2: bias[(row / rowDiv) % len] */
     int len;
     int rowDiv;
+    int act;       /* 0: nothing; 1: Rectify applied to the result (NTSAMD_ACT_RECTIFY) */
 };
 
 void _AmdMatrixMul2DBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,

@@ -43,7 +43,7 @@ int GetBroadcastDimIndex(const XTensor & a, const XTensor & b)
 
 static XTensor MulAndShiftCore(const XTensor & x, MATRIX_TRANS_TYPE transposedX,
                                const XTensor & w, MATRIX_TRANS_TYPE transposedW,
-                               const XTensor & b, DTYPE alpha, bool firstOverload)
+                               const XTensor & b, DTYPE alpha, bool firstOverload, int act = 0)
 {
     CheckNTErrors(x.dataType == w.dataType, "Input tensors should have the same data type!");
     CheckNTErrors(x.order >= 2 && w.order >= 2, "Input tensors must have a order >= 2!");
@@ -95,9 +95,9 @@ static XTensor MulAndShiftCore(const XTensor & x, MATRIX_TRANS_TYPE transposedX,
     XTensor c(order, dimSize, x.dataType, 1.0F, x.devID, x.mem);
     c.SetTMPFlag();
 
-    _MatrixMulBias(&x, transposedX, &w, transposedW, &c, alpha, 0, &b, n);
+    _MatrixMulBias(&x, transposedX, &w, transposedW, &c, alpha, 0, &b, n, act);
 
-    if (n == SCALAR_BIAS)
+    if (n == SCALAR_BIAS || act != 0)
         return c;
 
     /* autograd edge: tails x, w, b, then n, transposedX, transposedW and, in the
@@ -118,6 +118,11 @@ XTensor MulAndShift(const XTensor & x, const XTensor & w, const XTensor & b, DTY
 {
     (void)parallelRunner;
     return MulAndShiftCore(x, X_NOTRANS, w, X_NOTRANS, b, alpha, true);
+}
+
+XTensor MulAndShiftRectify(const XTensor & x, const XTensor & w, const XTensor & b, DTYPE alpha)
+{
+    return MulAndShiftCore(x, X_NOTRANS, w, X_NOTRANS, b, alpha, true, 1);
 }
 
 XTensor MulAndShift(const XTensor & x, MATRIX_TRANS_TYPE transposedX, const XTensor & w, MATRIX_TRANS_TYPE transposedW,

@@ -17,6 +17,12 @@ XTensor MulAndShift(const XTensor & x, MATRIX_TRANS_TYPE transposedX,
                     const XTensor & w, MATRIX_TRANS_TYPE transposedW,
                     const XTensor & b, DTYPE alpha = (DTYPE)1.0, XPRunner * parallelRunner = NULL);
 
+/* Rectify(MulAndShift(x, w, b, alpha)) as ONE kernel: what the feed-forward block of the transformer sample
+   computes first (source/sample/transformer/submodel/FFN.cpp:94, Rectify: source/tensor/function/Rectify.cpp:34-56).
+   For inference: no autograd edge is recorded (the reference links Rectify to the product's output, which does
+   not exist here). */
+XTensor MulAndShiftRectify(const XTensor & x, const XTensor & w, const XTensor & b, DTYPE alpha = (DTYPE)1.0);
+
 /* the dimension of a that b is broadcast along, or -1 */
 int GetBroadcastDimIndex(const XTensor & a, const XTensor & b);
 

@@ -62,10 +62,10 @@ void _AmdMatrixMULBias(int devID,
                        const void * b, MATRIX_TRANS_TYPE transposedB, TENSOR_DATA_TYPE dataTypeB,
                        void * c, TENSOR_DATA_TYPE dataTypeC,
                        int na, int ma, int nb, int mb, int nc, int mc, DTYPE alpha, DTYPE beta,
-                       const void * bias, int biasMode, int biasLen, int biasRowDiv)
+                       const void * bias, int biasMode, int biasLen, int biasRowDiv, int activation)
 {
-    Check(ntsamd_matrix_mul_bias(devID, NULL, a, transposedA, dataTypeA, b, transposedB, dataTypeB, c, dataTypeC,
-                                 na, ma, nb, mb, nc, mc, alpha, beta, bias, biasMode, biasLen, biasRowDiv));
+    Check(ntsamd_matrix_mul_bias_act(devID, NULL, a, transposedA, dataTypeA, b, transposedB, dataTypeB, c, dataTypeC,
+                                     na, ma, nb, mb, nc, mc, alpha, beta, bias, biasMode, biasLen, biasRowDiv, activation));
 }
 
 void _AmdMatrixMULColSum(int devID,

@@ -49,13 +49,14 @@ void _AmdMatrixMULList(int devID, const TensorList * a, MATRIX_TRANS_TYPE transp
                        int count, DTYPE alpha = (DTYPE)1.0, DTYPE beta = 1.0);
 
 /* one product with the broadcast add of MulAndShift fused into its epilogue:
-   biasMode 1 adds bias[column], biasMode 2 adds bias[(row / biasRowDiv) % biasLen] */
+   biasMode 1 adds bias[column], biasMode 2 adds bias[(row / biasRowDiv) % biasLen];
+   activation 1 applies Rectify to the result as well */
 void _AmdMatrixMULBias(int devID,
                        const void * a, MATRIX_TRANS_TYPE transposedA, TENSOR_DATA_TYPE dataTypeA,
                        const void * b, MATRIX_TRANS_TYPE transposedB, TENSOR_DATA_TYPE dataTypeB,
                        void * c, TENSOR_DATA_TYPE dataTypeC,
                        int na, int ma, int nb, int mb, int nc, int mc, DTYPE alpha, DTYPE beta,
-                       const void * bias, int biasMode, int biasLen, int biasRowDiv);
+                       const void * bias, int biasMode, int biasLen, int biasRowDiv, int activation = 0);
 
 /* one product that also returns the column sums of op(b):
    colSum[j] = colSumBeta * colSum[j] + sum_k op(b)[k][j]; for the backward step of MulAndShift,

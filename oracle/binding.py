@@ -88,6 +88,7 @@ class Oracle:
         L.oracle_softmax.restype = C.c_int
         L.oracle_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.oracle_attention.restype = C.c_int
+        L.oracle_rectify.argtypes = [_fp, C.c_long, _fp]
         L.oracle_convert_data_type.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_long]
         L.oracle_convert_data_type.restype = C.c_int
         L.oracle_is_float_equal.argtypes = [C.c_float] * 4
@@ -214,6 +215,11 @@ class Oracle:
             raise ValueError("Unmatched tensors in attention")
         return out
 
+    def rectify(self, x):
+        y = np.empty_like(x)
+        self.lib.oracle_rectify(_f(x), x.size, _f(y))
+        return y
+
     # -- data type conversion ------------------------------------------------
     def convert(self, x, type_t):
         """x: float32 (X_FLOAT), int32 (X_INT) or uint16 holding half bit patterns (X_FLOAT16);
@@ -281,6 +287,7 @@ class Reference:
                                       _fp, _ip, C.c_int, _fp, _ip, C.c_float]
         L.ref_enum_values.argtypes = [_ip]
         L.ref_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.ref_rectify.argtypes = [_fp, C.c_int, _fp]
         L.ref_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int]
         L.ref_softmax.argtypes = [_fp, _ip, C.c_int, _fp]
         L.ref_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
@@ -362,6 +369,11 @@ class Reference:
         self.lib.ref_attention(_f(q), _f(k), _f(v), _f(mask) if mask is not None else None, _f(out),
                                batch, lq, k.shape[1], hidden, heads, scale)
         return out
+
+    def rectify(self, x):
+        y = np.empty_like(x)
+        self.lib.ref_rectify(_f(x), x.size, _f(y))
+        return y
 
     def convert(self, x, type_t):
         type_s = NP_TYPE_CODE[x.dtype.type]

@@ -685,6 +685,18 @@ int oracle_attention(const float *q, const float *k, const float *v, const float
     return r;
 }
 
+/* ---- rectify ------------------------------------------------------------------ */
+
+void oracle_rectify(const float *x, long n, float *y)
+{
+    for (long i = 0; i < n; i++) {
+        float p = x[i];
+        if (p < 0)
+            p = 0;
+        y[i] = p;
+    }
+}
+
 /* ---- data type conversion ------------------------------------------------- */
 
 int oracle_convert_data_type(const void *s, int typeS, void *t, int typeT, long n)

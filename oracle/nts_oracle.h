@@ -103,6 +103,10 @@ int oracle_softmax(const float *x, long rows, int n, float *y);
 int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
                      int batch, int lq, int lk, int hidden, int heads, float scale);
 
+/* y = max(0, x) as _Rectify computes it (source/tensor/function/Rectify.cpp:47-55): a value below zero
+   becomes 0, everything else (negative zero and NaN included) passes */
+void oracle_rectify(const float *x, long n, float *y);
+
 /* t[i] = (typeT) s[i] as the reference's GPU kernels convert (source/tensor/core/getandset/
    ConvertDataType.cu:31-66): X_FLOAT -> X_FLOAT16 round to nearest even (__float2half), X_FLOAT16 -> X_FLOAT
    exact, X_FLOAT -> X_INT toward zero (saturating, NaN -> 0: the GPU's cast), X_INT -> X_FLOAT round to

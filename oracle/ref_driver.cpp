@@ -243,6 +243,17 @@ int ref_attention(const float * q, const float * k, const float * v, const float
     return 0;
 }
 
+int ref_rectify(const float * x, int n, float * y)
+{
+    int dims[1] = {n};
+    XTensor * tx = Make(dims, 1, x);
+    XTensor * ty = Make(dims, 1, NULL);
+    _Rectify(tx, ty);
+    memcpy(y, ty->data, sizeof(float) * (size_t)n);
+    delete tx; delete ty;
+    return 0;
+}
+
 /* _ConvertDataType between X_FLOAT (2) and X_INT (0) on the host (ConvertDataType.cpp:83-94); the
    half branches of the host code cast the value to an integer and are of no use as a reference */
 int ref_convert(const void * s, int typeS, void * t, int typeT, int n)

@@ -708,6 +708,49 @@ static bool TestAttention()
     return ok;
 }
 
+/* ---- Rectify(MulAndShift(x, w, b)) in one kernel: the reference's TRectify values through a unit product, and a
+   seeded feed-forward layer against the oracle ------------------------------------------------------------ */
+
+static bool TestMulAndShiftRectify()
+{
+    bool ok = true;
+    {
+        /* TRectify.cpp:43-46: x times the identity plus a zero bias, rectified */
+        int dx[2] = {2, 3}, dw[2] = {3, 3}, db[1] = {3};
+        DTYPE xData[2][3] = {{0.0F, -1.0F, 2.0F}, {3.0F, -4.0F, -5.0F}};
+        DTYPE eye[3][3] = {{1, 0, 0}, {0, 1, 0}, {0, 0, 1}};
+        DTYPE zero[3] = {0, 0, 0};
+        DTYPE answer[2][3] = {{0.0F, 0.0F, 2.0F}, {3.0F, 0.0F, 0.0F}};
+        XTensor * x = NewGPU(2, dx, &xData[0][0]);
+        XTensor * w = NewGPU(2, dw, &eye[0][0]);
+        XTensor * b = NewGPU(1, db, zero);
+        XTensor y = MulAndShiftRectify(*x, *w, *b);
+        ok = ok && CheckData(&y, answer, 6, 1e-4F);
+        delete x; delete w; delete b;
+    }
+    int dx[3] = {4, 33, 96}, dw[2] = {96, 200}, db[1] = {200};
+    std::vector<float> x(4 * 33 * 96), w(96 * 200), b(200), pre(4 * 33 * 200), ref(4 * 33 * 200), got(4 * 33 * 200);
+    oracle_fill_uniform(x.data(), (long)x.size(), 501, -1.0F, 1.0F);
+    oracle_fill_normal(w.data(), (long)w.size(), 502, 0, 0.1F);
+    oracle_fill_normal(b.data(), (long)b.size(), 503, 0, 0.1F);
+    int dc[8], cOrder = 0;
+    oracle_mulandshift(x.data(), X_NOTRANS, dx, 3, w.data(), X_NOTRANS, dw, 2, b.data(), db, 1, pre.data(), dc, &cOrder, 1.0F);
+    oracle_rectify(pre.data(), (long)pre.size(), ref.data());
+    XTensor * gx = NewGPU(3, dx, x.data());
+    XTensor * gw = NewGPU(2, dw, w.data());
+    XTensor * gb = NewGPU(1, db, b.data());
+    XTensor y = MulAndShiftRectify(*gx, *gw, *gb);
+    y.GetData(got.data());
+    ok = ok && y.order == 3 && y.dimSize[0] == 4 && y.dimSize[1] == 33 && y.dimSize[2] == 200 && y.income.tailNum == 0;
+    float e = MaxRelErr(got, ref);
+    if (!(e < 1e-5F * sqrtf(96.0F))) {
+        fprintf(stderr, "mulandshift+rectify err=%g\n", e);
+        ok = false;
+    }
+    delete gx; delete gw; delete gb;
+    return ok;
+}
+
 /* ---- device blocks are handed out again: same results, no growth --------------------------------- */
 
 static bool TestMemoryReuse()
@@ -866,6 +909,7 @@ int main(int argc, char ** argv)
     RUN(TestConvertDataType12);
     RUN(TestConvertDataType3);
     RUN(TestAttention);
+    RUN(TestMulAndShiftRectify);
     RUN(TestMemoryReuse);
     printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
     return all ? 0 : 1;

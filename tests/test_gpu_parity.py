@@ -447,6 +447,58 @@ def test_fused_bias(gpu, oracle, half):
             assert_fp32(got, ref, 48, mag, what=str(bshape))
 
 
+@pytest.mark.parametrize("half", (False, True))
+def test_fused_bias_and_rectify(gpu, oracle, half):
+    """Rectify(MulAndShift(x, w, b)) in the epilogue (the first step of the reference's feed-forward block):
+    against the oracle's product + broadcast add + rectify, on the main path and on the generic one
+    (row-indexed bias), with beta, and with a NaN and a negative zero forced into the result."""
+    torch = torch_()
+    for cfg in ("0", "1", "2") if half else ("0", "1"):
+        os.environ["NTSAMD_TILE_CFG"] = cfg
+        for i, (M, N, K) in enumerate([(64, 64, 32), (136, 264, 96), (257, 120, 64), (33, 35, 37) if not half else (40, 48, 56)]):
+            x = oracle.normal((M, K), 9000 + i)
+            w = oracle.normal((K, N), 9100 + i, 0, 0.3)
+            b = oracle.normal((N,), 9200 + i)
+            c0 = oracle.uniform((M, N), 9300 + i)
+            if half:
+                x, w, b, c0 = (oracle.from_f16_bits(oracle.to_f16_bits(t)) for t in (x, w, b, c0))
+            for beta in (0.0, 0.5):
+                pre = oracle.matmul2d(x, X_NOTRANS, w, X_NOTRANS, c0.copy(), 1.0, beta) + b[None, :]
+                ref = oracle.rectify(np.ascontiguousarray(pre, np.float32))
+                c = dev_tensor(c0, gpu, half) if beta != 0 else torch.full((M, N), float("nan"), device=gpu, dtype=torch.float16 if half else torch.float32)
+                nt.matrix_mul(dev_tensor(x, gpu, half), X_NOTRANS, dev_tensor(w, gpu, half), X_NOTRANS, c, 1.0, beta,
+                              bias=dev_tensor(b, gpu, half), act=nt.ACT_RECTIFY)
+                got = c.float().cpu().numpy()
+                assert (got >= 0).all() and (got[ref == 0] <= 1e-3).all()
+                # elements whose pre-activation is within rounding of zero may fall on either side
+                if half:
+                    assert_fp16(got, ref, what="cfg%s %dx%dx%d beta=%g" % (cfg, M, N, K, beta))
+                else:
+                    assert_fp32(got, ref, K, what="cfg%s %dx%dx%d beta=%g" % (cfg, M, N, K, beta))
+    os.environ.pop("NTSAMD_TILE_CFG", None)
+    if not half:
+        # bias by row group (generic path) with the activation
+        x, w, b = oracle.normal((60, 20), 9400), oracle.normal((20, 30), 9401), oracle.normal((6,), 9402)
+        pre = oracle.matmul2d(x, X_NOTRANS, w, X_NOTRANS) + np.repeat(b, 10)[:, None]
+        c = torch.full((60, 30), float("nan"), device=gpu)
+        nt.matrix_mul(dev_tensor(x, gpu), X_NOTRANS, dev_tensor(w, gpu), X_NOTRANS, c, 1.0, 0.0,
+                      bias=dev_tensor(b, gpu), bias_mode=nt.BIAS_ROW, bias_row_div=10, act=nt.ACT_RECTIFY)
+        assert_fp32(c.cpu().numpy(), oracle.rectify(np.ascontiguousarray(pre, np.float32)), 20, what="row bias")
+        # special values: NaN in, NaN out; an exact negative zero stays a negative zero
+        x = np.zeros((8, 8), np.float32)
+        x[0, 0] = np.nan
+        w = np.eye(8, dtype=np.float32)
+        b = np.full((8,), -0.0, np.float32)
+        c = torch.full((8, 8), 7.0, device=gpu)
+        nt.matrix_mul(dev_tensor(x, gpu), X_NOTRANS, dev_tensor(w, gpu), X_NOTRANS, c, 1.0, 0.0, bias=dev_tensor(b, gpu), act=nt.ACT_RECTIFY)
+        got = c.cpu().numpy()
+        assert np.isnan(got[0]).all() and not np.isnan(got[1:]).any() and (got[1:] == 0).all()
+    L = nt.load()
+    t = torch.zeros(64, device=gpu)
+    p = t.data_ptr()
+    assert L.ntsamd_matrix_mul_bias_act(0, None, p, 1, 2, p, 1, 2, p, 2, 8, 8, 8, 8, 8, 8, 1.0, 0.0, p, 1, 8, 1, 5) == 1
+
+
 def test_runs_on_the_callers_stream(gpu, oracle):
     torch = torch_()
     a = dev_tensor(oracle.uniform((256, 128), 1), gpu)
