@@ -22,10 +22,15 @@
 #include "../../niutensor_amd/nts/Attention.h"
 #include "../../oracle/nts_oracle.h"
 
+#include "../../include/ntsamd_gemm.h"
+#include <hip/hip_runtime_api.h>
+
 #include <chrono>
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
+#include <string.h>
+#include <thread>
 #include <vector>
 
 using namespace nts;
@@ -751,6 +756,72 @@ static bool TestMulAndShiftRectify()
     return ok;
 }
 
+/* ---- the C ABI from several host threads at once, each on a stream of its own (the reference runs one worker
+   thread per device and more than one model replica per process): same bits as a single-threaded run --------- */
+
+static void ThreadBody(int id, const float * a, const float * b, const float * bias, float * out, int * status)
+{
+    const int M = 200, N = 136, K = 96;
+    hipStream_t stream;
+    *status = 1;
+    if (hipSetDevice(DEV) != hipSuccess || hipStreamCreate(&stream) != hipSuccess)
+        return;
+    float *da, *db, *dbias, *dc;
+    if (hipMalloc((void **)&da, M * K * 4) != hipSuccess || hipMalloc((void **)&db, K * N * 4) != hipSuccess ||
+        hipMalloc((void **)&dbias, N * 4) != hipSuccess || hipMalloc((void **)&dc, M * N * 4) != hipSuccess)
+        return;
+    hipMemcpy(da, a, M * K * 4, hipMemcpyHostToDevice);
+    hipMemcpy(db, b, K * N * 4, hipMemcpyHostToDevice);
+    hipMemcpy(dbias, bias, N * 4, hipMemcpyHostToDevice);
+    int rc = 0;
+    for (int it = 0; it < 40 && rc == 0; it++) {
+        /* every thread asks for something else in between, so that the calls really interleave */
+        if ((it + id) % 3 == 0)
+            rc = ntsamd_matrix_mul(DEV, stream, da, X_NOTRANS, X_FLOAT, db, X_NOTRANS, X_FLOAT, dc, X_FLOAT, M, K, K, N, M, N, 0.5F, 0.0F);
+        rc = rc != 0 ? rc : ntsamd_matrix_mul_bias_act(DEV, stream, da, X_NOTRANS, X_FLOAT, db, X_NOTRANS, X_FLOAT, dc, X_FLOAT,
+                                                       M, K, K, N, M, N, 1.0F + id, 0.0F, dbias, NTSAMD_BIAS_COL, N, 1, NTSAMD_ACT_RECTIFY);
+        /* a call that must fail leaves its message with THIS thread only */
+        int bad = ntsamd_matrix_mul(DEV, stream, da, X_NOTRANS, 4, db, X_NOTRANS, 4, dc, 4, M, K, K, N, M, N, 1.0F, 0.0F);
+        if (bad != NTSAMD_ERR_DATATYPE || strcmp(ntsamd_last_error(), "Unsupported data type!") != 0)
+            rc = -1;
+    }
+    hipStreamSynchronize(stream);
+    hipMemcpy(out, dc, M * N * 4, hipMemcpyDeviceToHost);
+    hipFree(da); hipFree(db); hipFree(dbias); hipFree(dc);
+    hipStreamDestroy(stream);
+    *status = rc;
+}
+
+static bool TestThreads()
+{
+    const int M = 200, N = 136, K = 96, T = 4;
+    std::vector<float> a(M * K), b(K * N), bias(N), pre(M * N), ref(M * N);
+    oracle_fill_uniform(a.data(), M * K, 601, -1.0F, 1.0F);
+    oracle_fill_uniform(b.data(), K * N, 602, -1.0F, 1.0F);
+    oracle_fill_normal(bias.data(), N, 603, 0, 1.0F);
+    std::vector<std::vector<float> > out(T, std::vector<float>(M * N));
+    int status[T];
+    std::vector<std::thread> threads;
+    for (int t = 0; t < T; t++)
+        threads.push_back(std::thread(ThreadBody, t, a.data(), b.data(), bias.data(), out[t].data(), &status[t]));
+    for (int t = 0; t < T; t++)
+        threads[t].join();
+    bool ok = true;
+    for (int t = 0; t < T; t++) {
+        ok = ok && status[t] == 0;
+        oracle_matmul2d(a.data(), X_NOTRANS, b.data(), X_NOTRANS, pre.data(), M, K, K, N, M, N, 1.0F + t, 0.0F);
+        for (int i = 0; i < M * N; i++)
+            pre[i] += bias[i % N];
+        oracle_rectify(pre.data(), M * N, ref.data());
+        float e = MaxRelErr(out[t], ref);
+        if (!(e < 1e-5F * sqrtf((float)K))) {
+            fprintf(stderr, "thread %d err=%g\n", t, e);
+            ok = false;
+        }
+    }
+    return ok;
+}
+
 /* ---- device blocks are handed out again: same results, no growth --------------------------------- */
 
 static bool TestMemoryReuse()
@@ -910,6 +981,7 @@ int main(int argc, char ** argv)
     RUN(TestConvertDataType3);
     RUN(TestAttention);
     RUN(TestMulAndShiftRectify);
+    RUN(TestThreads);
     RUN(TestMemoryReuse);
     printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
     return all ? 0 : 1;

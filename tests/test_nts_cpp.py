@@ -19,4 +19,4 @@ def test_nts_host_layer_on_gpu():
     print(p.stderr)
     assert p.returncode == 0, p.stdout + p.stderr
     assert "OK! Everything is good!" in p.stdout
-    assert p.stdout.count("passed") == 21 and "FAILED" not in p.stdout
+    assert p.stdout.count("passed") == 22 and "FAILED" not in p.stdout
