@@ -942,6 +942,23 @@ static int Provoke(const char * name)
         cc.grad = new XTensor(3, d223, X_FLOAT, 1.0F, 0, NULL);
         XMathGrad::MakeGrad(&cc, true);
     }
+    else if (!strcmp(name, "converthost")) {
+        XTensor hostHalf(2, d22, X_FLOAT16, 1.0F, -1, NULL);
+        _ConvertDataType(&host, &hostHalf);              /* host tensors: the reference's CPU path, not this library */
+    }
+    else if (!strcmp(name, "convertsize")) {
+        XTensor big(3, d223, X_FLOAT16, 1.0F, 0, NULL);
+        _ConvertDataType(&a, &big);                      /* 6 elements into 12 */
+    }
+    else if (!strcmp(name, "attentionheads")) {
+        /* a hidden size of 3 does not split into 2 heads */
+        XTensor o3(3, d223, X_FLOAT, 1.0F, 0, NULL);
+        _AmdAttention(&t3, &t3, &t3, NULL, &o3, 2, 1.0F);
+    }
+    else if (!strcmp(name, "attentiontype")) {
+        XTensor o3(3, d223, X_FLOAT16, 1.0F, 0, NULL);
+        _AmdAttention(&t3, &t3, &t3, NULL, &o3, 1, 1.0F);
+    }
     else if (!strcmp(name, "biasshape")) {
         XTensor bias(2, d22, X_FLOAT, 1.0F, 0, NULL);
         MulAndShift(a, b, bias);

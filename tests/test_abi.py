@@ -116,6 +116,33 @@ def test_empty_products_succeed_without_a_device():
     assert rc == 0
 
 
+def test_convert_and_attention_argument_errors_need_no_device():
+    L = nt.load()
+    p = 0x1000
+    assert L.ntsamd_convert_data_type(0, None, p, 2, p, 4, 8) == 2
+    assert L.ntsamd_last_error().decode() == "Unsupported data types for conversion!"
+    assert L.ntsamd_convert_data_type(0, None, p, 3, p, 0, 8) == 2                # half -> int: refused like the reference
+    assert L.ntsamd_convert_data_type(0, None, p, 2, p, 2, 8) == 0                # equal types: nothing to do
+    assert L.ntsamd_convert_data_type(0, None, p, 2, p, 3, -5) == 1
+    assert L.ntsamd_convert_data_type(0, None, None, 2, p, 3, 5) == 1
+    assert L.ntsamd_convert_data_type(0, None, p + 2, 2, p, 3, 5) == 1            # a float array on an odd half
+    st = (C.c_longlong * 12)(*([8, 64, 8] * 4))
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 4, 1, 1, 8, 8, 8, st, 1.0) == 2
+    assert L.ntsamd_last_error().decode() == "Unsupported data type!"
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 132, st, 1.0) == 1
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 0, 8, st, 1.0) == 1
+    assert "no keys" in L.ntsamd_last_error().decode()
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, -1, 1, 8, 8, 8, st, 1.0) == 1
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 0, 1, 8, 8, 8, st, 1.0) == 0            # no heads: nothing to do
+    assert L.ntsamd_attention(0, None, p + 4, p, p, None, p, 2, 1, 1, 8, 8, 8, st, 1.0) == 1        # q not 16-byte aligned
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 8, None, 1.0) == 1
+    big = (C.c_longlong * 12)(*([8, 64, 8, 8, 64, 1 << 24, 8, 64, 8, 8, 64, 8]))
+    assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 1000, 8, big, 1.0) == 1
+    assert "2 GiB" in L.ntsamd_last_error().decode()
+    # an unknown activation
+    assert L.ntsamd_matrix_mul_bias_act(0, None, p, 1, 2, p, 1, 2, p, 2, 8, 8, 8, 8, 8, 8, 1.0, 0.0, p, 1, 8, 1, 7) == 1
+
+
 def test_invalid_device_is_an_error():
     L = nt.load()
     rc = L.ntsamd_init(12345)
@@ -134,6 +161,10 @@ def test_invalid_device_is_an_error():
     ("biasshape", "TODO!"),
     ("nograd", "No gradient found!"),
     ("gradtodo", "TODO!"),
+    ("converthost", "does not replace"),
+    ("convertsize", "Unmatched tensors!"),
+    ("attentionheads", "The hidden size must be a multiple of the number of heads!"),
+    ("attentiontype", "Input tensors should have the same data type!"),
 ])
 def test_nts_layer_fatal_errors(case, message):
     """CheckNTErrors / ShowNTErrors of the reference: '[ERROR] ...' on stderr, then std::terminate."""
