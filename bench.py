@@ -50,6 +50,9 @@ def configs():
                 dtype="f32", M=128, N=128, K=64, batch=256),
         10: dict(name="cfg10 fp32 Rectify(MulAndShift(X[32x128x512], W[512x2048], b[2048])) in one kernel (first step of the feed-forward block)",
                  dtype="f32", M=4096, N=2048, K=512, batch=1),
+        11: dict(name="cfg11 fp32 attention probabilities in one kernel: softmax(Q.K^T/8) per head as [8x32x128x128] from q,k [32x128x512] "
+                      "(cfg3's first product with the scale, the softmax and the head split folded in)",
+                 dtype="f32", M=128, N=128, K=64, batch=256),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -152,6 +155,14 @@ class Workload:
             # q, k, v read once, the result written once; the scores never reach memory
             self.bytes = 4 * (4.0 if idx == 8 else 2.0) * 32 * 128 * 512
             self.launches = 1
+        elif idx == 11:
+            self.q = g(oracle.normal((32, 128, 512), 1))
+            self.k = g(oracle.normal((32, 128, 512), 2))
+            self.p = torch.empty((8, 32, 128, 128), device=dev)
+            self.run = lambda: nt.attention_probs(self.q, self.k, self.p, 8, 0.125)
+            self.flops = 2.0 * 256 * 128 * 128 * 64
+            self.bytes = 4.0 * (2 * 32 * 128 * 512 + 256 * 128 * 128)
+            self.launches = 1
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
@@ -189,7 +200,7 @@ def cpu_baseline(idx, budget_s=12.0):
     # the forward configurations in float run the REAL reference (its CPU sources compiled by oracle/Makefile into
     # oracle/_ref, which travels with the tree) when that library is there; the others (half: the reference has no
     # CPU half arithmetic; the gradient steps) and a tree without it run the restatement
-    use_ref = idx in (1, 2, 3, 5, 8, 10) and Reference.available()
+    use_ref = idx in (1, 2, 3, 5, 8, 10, 11) and Reference.available()
     o = Reference() if use_ref else gen
     if use_ref:
         o.uniform, o.normal = gen.uniform, gen.normal
@@ -199,7 +210,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -220,6 +231,14 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 8 * 4.0 * 128 * 128 * 64
         sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax, product, merge" % nb
+    elif idx == 11:
+        nb = max(1, min(32, int(budget_s * rate / (8 * 2.0 * 128 * 128 * 64))))
+        q, k = o.normal((nb, 128, 512), 1), o.normal((nb, 128, 512), 2)
+        t0 = time.perf_counter()
+        o.attention_probs(q, k, 8, 0.125)
+        dt = time.perf_counter() - t0
+        fl = nb * 8 * 2.0 * 128 * 128 * 64
+        sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax" % nb
     elif idx == 7:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, ds = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 128), 3)
@@ -305,7 +324,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
     # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
-    if idx in (3, 7, 9):
+    if idx in (3, 7, 9, 11):
         roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
                 "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
     else:
@@ -344,7 +363,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-10 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-11 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -372,7 +391,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

@@ -219,6 +219,20 @@ int ntsamd_attention(int devID, void * stream,
                      const long long * strides, float scale);
 
 /*
+ * The first half of the attention, for callers that need the probabilities themselves:
+ *   probs[h][b] = softmax(scale * q[h][b] * k[h][b]^T + mask[h][b])   (dense [heads][batch][lq][lk], X_FLOAT).
+ * Replaces Split of q and k, ScaleMe, BMMul(q, X_NOTRANS, k, X_TRANS), SumMe with the mask and Softmax(att, -1)
+ * (source/sample/transformer/submodel/Attention.cpp:194-224) with one launch; the training path of the
+ * reference goes on from here with Dropout and BMMul(att, v) (:226-235), and its backward step reads the
+ * probabilities. strides[0..2] address q and strides[3..5] address k as in ntsamd_attention; dataType is
+ * X_FLOAT; dh is a multiple of 4, at most 128.
+ */
+int ntsamd_attention_probs(int devID, void * stream,
+                           const void * q, const void * k, const void * mask, void * probs, int dataType,
+                           int heads, int batch, int lq, int lk, int dh,
+                           const long long * strides, float scale);
+
+/*
  * Element-wise data type conversion t[i] = (typeT) s[i], i < size.
  * Replaces _CudaConvertDataType(devID, s, typeS, t, typeT, size) and the tensor form
  * _CudaConvertDataType(input, output) (source/tensor/core/getandset/ConvertDataType.cu:78-99,

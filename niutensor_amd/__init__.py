@@ -31,6 +31,7 @@ EXPORTS = (
     "ntsamd_matrix_mul_colsum",
     "ntsamd_reduce_sum_xz",
     "ntsamd_attention",
+    "ntsamd_attention_probs",
     "ntsamd_convert_data_type",
 )
 
@@ -70,6 +71,7 @@ def load():
     L.ntsamd_matrix_mul_colsum.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, cf]
     L.ntsamd_reduce_sum_xz.argtypes = [ci, vp, vp, ci, ci, ci, ci, vp, cf]
     L.ntsamd_attention.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
+    L.ntsamd_attention_probs.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     L.ntsamd_convert_data_type.argtypes = [ci, vp, vp, ci, vp, ci, ll]
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
@@ -202,6 +204,22 @@ def attention(q, k, v, out, heads, scale, mask=None, split=False):
                             heads, batch, lq, lk, dh, strides, scale)
     _check(rc)
     return out
+
+
+def attention_probs(q, k, probs, heads, scale, mask=None):
+    """probs[h][b] = softmax(scale q_h k_h^T + mask[h][b]); q [batch][lq][heads*dh], k [batch][lk][heads*dh],
+    probs and mask dense float [heads][batch][lq][lk]."""
+    batch, lq, hd = (int(x) for x in q.shape)
+    lk = int(k.shape[1])
+    dh = hd // heads
+    for t in (q, k, probs):
+        assert t.is_contiguous()
+    strides = (C.c_longlong * 6)(dh, lq * hd, hd, dh, lk * hd, hd)
+    rc = load().ntsamd_attention_probs(q.device.index, _stream_ptr(q), q.data_ptr(), k.data_ptr(),
+                                       mask.data_ptr() if mask is not None else None, probs.data_ptr(), _dtype_code(q),
+                                       heads, batch, lq, lk, dh, strides, scale)
+    _check(rc)
+    return probs
 
 
 def convert_data_type(s, t):

@@ -21,9 +21,12 @@ struct AttnParams {
     float scale;
     int qTiles;                         /* filled in by the launcher */
     int maskVec;                        /* filled in by the launcher: 16-byte mask loads are possible */
+    int probsVec;                       /* filled in by the launcher (attention_probs): 16-byte stores are possible */
 };
 
 int launch_attention_f32(const AttnParams & p, hipStream_t stream);
 int launch_attention_f16(const AttnParams & p, hipStream_t stream);
+/* probabilities only: out is the dense [heads][batch][lq][lk] tensor, v is not used */
+int launch_attention_probs_f32(const AttnParams & p, hipStream_t stream);
 
 }  // namespace ntsamd

@@ -567,6 +567,60 @@ int ntsamd_attention(int devID, void * stream,
     return NTSAMD_OK;
 }
 
+int ntsamd_attention_probs(int devID, void * stream,
+                           const void * q, const void * k, const void * mask, void * probs, int dataType,
+                           int heads, int batch, int lq, int lk, int dh,
+                           const long long * strides, float scale)
+{
+    if (dataType != NTSAMD_X_FLOAT)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
+    if (heads < 0 || batch < 0 || lq < 0 || lk < 0 || dh < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
+    if (heads == 0 || batch == 0 || lq == 0 || lk == 0)
+        return NTSAMD_OK;
+    if (!q || !k || !probs || !strides)
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty input tensors!");
+    if (dh == 0 || dh > 128 || dh % 4 != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "head size %d is not served by the fused kernel (a multiple of 4 up to 128 is)", dh);
+    for (int i = 0; i < 6; i++)
+        if (strides[i] < 0 || strides[i] % 4 != 0)
+            return fail(NTSAMD_ERR_ARGUMENT, "strides must be non-negative multiples of 4 elements");
+    if (!aligned16(q) || !aligned16(k))
+        return fail(NTSAMD_ERR_ARGUMENT, "q and k must be 16-byte aligned");
+    if ((mask && (reinterpret_cast<uintptr_t>(mask) & 3) != 0) || (reinterpret_cast<uintptr_t>(probs) & 3) != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "misaligned mask or result");
+    if (strides[2] < dh || strides[5] < dh)
+        return fail(NTSAMD_ERR_ARGUMENT, "row stride smaller than the head size");
+    if ((long long)heads * batch * ((lq + 63) / 64) > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
+    if (((long long)lk + 256) * strides[5] * 4 > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "tensor too large: the keys of one head span more than 2 GiB");
+    int st = check_device(devID);
+    if (st != NTSAMD_OK)
+        return st;
+    DeviceScope scope(devID);
+    if (scope.status != NTSAMD_OK)
+        return scope.status;
+    AttnParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = q;
+    p.k = k;
+    p.mask = static_cast<const float *>(mask);
+    p.out = probs;
+    p.heads = heads;
+    p.batch = batch;
+    p.lq = lq;
+    p.lk = lk;
+    p.dh = dh;
+    p.qH = strides[0]; p.qB = strides[1]; p.qL = strides[2];
+    p.kH = strides[3]; p.kB = strides[4]; p.kL = strides[5];
+    p.scale = scale;
+    int rc = launch_attention_probs_f32(p, static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return NTSAMD_OK;
+}
+
 int ntsamd_matrix_mul(int devID, void * stream,
                       const void * a, int transposedA, int dataTypeA,
                       const void * b, int transposedB, int dataTypeB,

@@ -61,4 +61,52 @@ XTensor AmdAttention(const XTensor & q, const XTensor & k, const XTensor & v, co
     return out;
 }
 
+void _AmdAttentionProbs(const XTensor * q, const XTensor * k, const XTensor * mask, XTensor * probs, int nhead, DTYPE scale)
+{
+    CheckNTErrors((q && k && probs), "Empty input tensors!");
+    CheckNTErrors((q->dataType == X_FLOAT && k->dataType == X_FLOAT && probs->dataType == X_FLOAT), "TODO!");
+    CheckNTErrors((q->order >= 2 && q->order == k->order && probs->order == q->order + 1),
+                  "Input tensors must have the same order >= 2!");
+    CheckNTErrors((q->devID >= 0), "This code must be run on GPUs!");
+    CheckNTErrors((q->devID == k->devID && q->devID == probs->devID), "The tensors must be on the same GPU!");
+
+    const int order = q->order;
+    const int hidden = q->dimSize[order - 1];
+    const int lq = q->dimSize[order - 2], lk = k->dimSize[order - 2];
+    CheckNTErrors((nhead > 0 && hidden % nhead == 0), "The hidden size must be a multiple of the number of heads!");
+    CheckNTErrors((k->dimSize[order - 1] == hidden), "Unmatched tensors in attention!");
+    int batch = 1;
+    for (int i = 0; i < order - 2; i++) {
+        CheckNTErrors((q->dimSize[i] == k->dimSize[i]), "Unmatched tensors in attention!");
+        batch *= q->dimSize[i];
+    }
+    CheckNTErrors((probs->unitNum == nhead * batch * lq * lk), "Unmatched tensors in attention!");
+    if (mask != NULL) {
+        CheckNTErrors((mask->dataType == X_FLOAT && mask->devID == q->devID), "Unmatched tensors in attention!");
+        CheckNTErrors((mask->unitNum == probs->unitNum), "Unmatched tensors in attention!");
+    }
+    const int dh = hidden / nhead;
+    long long strides[6] = {dh, (long long)lq * hidden, hidden, dh, (long long)lk * hidden, hidden};
+    int rc = ntsamd_attention_probs(q->devID, NULL, q->data, k->data, mask != NULL ? mask->data : NULL, probs->data,
+                                    X_FLOAT, nhead, batch, lq, lk, dh, strides, scale);
+    if (rc != NTSAMD_OK) {
+        ShowNTErrors(ntsamd_last_error());
+    }
+}
+
+XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * mask, int nhead, DTYPE scale)
+{
+    CheckNTErrors((q.order >= 2 && q.order + 1 <= MAX_TENSOR_DIM_NUM), "Input tensors must have the same order >= 2!");
+    /* (nhead, batch..., lq, lk): the shape BMMul(Split(q), Split(k)^T) has in the reference */
+    int dims[MAX_TENSOR_DIM_NUM];
+    dims[0] = nhead;
+    for (int i = 0; i < q.order - 1; i++)
+        dims[i + 1] = q.dimSize[i];
+    dims[q.order] = k.dimSize[k.order - 2];
+    XTensor probs(q.order + 1, dims, q.dataType, 1.0F, q.devID, q.mem);
+    probs.SetTMPFlag();
+    _AmdAttentionProbs(&q, &k, mask, &probs, nhead, scale);
+    return probs;
+}
+
 }  // namespace nts

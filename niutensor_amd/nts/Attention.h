@@ -21,5 +21,11 @@ void _AmdAttention(const XTensor * q, const XTensor * k, const XTensor * v, cons
 XTensor AmdAttention(const XTensor & q, const XTensor & k, const XTensor & v, const XTensor * mask,
                      int nhead, DTYPE scale);
 
+/* probs = Softmax(Split(q) * scale x Split(k)^T + mask, -1) as a (nhead, batch..., lq, lk) tensor: the part of
+   MakeAttention that training shares with inference (:194-224); Dropout and BMMul(probs, Split(v)) follow in the
+   caller, and the backward step reads probs. X_FLOAT. */
+void _AmdAttentionProbs(const XTensor * q, const XTensor * k, const XTensor * mask, XTensor * probs, int nhead, DTYPE scale);
+XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * mask, int nhead, DTYPE scale);
+
 }  // namespace nts
 #endif

@@ -88,6 +88,8 @@ class Oracle:
         L.oracle_softmax.restype = C.c_int
         L.oracle_attention.argtypes = [_fp, _fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.oracle_attention.restype = C.c_int
+        L.oracle_attention_probs.argtypes = [_fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
+        L.oracle_attention_probs.restype = C.c_int
         L.oracle_rectify.argtypes = [_fp, C.c_long, _fp]
         L.oracle_convert_data_type.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_long]
         L.oracle_convert_data_type.restype = C.c_int
@@ -233,6 +235,16 @@ class Oracle:
             raise ValueError("Unsupported data types for conversion!")
         return out
 
+    def attention_probs(self, q, k, heads, scale, mask=None):
+        """Softmax(scale q_h k_h^T + mask) as [heads][batch][lq][lk]; q [batch][lq][hidden], k [batch][lk][hidden]."""
+        batch, lq, hidden = q.shape
+        probs = np.zeros((heads, batch, lq, k.shape[1]), np.float32)
+        r = self.lib.oracle_attention_probs(_f(q), _f(k), _f(mask) if mask is not None else None, _f(probs),
+                                            batch, lq, k.shape[1], hidden, heads, scale)
+        if r != 0:
+            raise ValueError("Unmatched tensors in attention")
+        return probs
+
     def is_float_equal(self, a, b, abs_err, rel_err=1e-4):
         return bool(self.lib.oracle_is_float_equal(a, b, abs_err, rel_err))
 
@@ -287,6 +299,7 @@ class Reference:
                                       _fp, _ip, C.c_int, _fp, _ip, C.c_float]
         L.ref_enum_values.argtypes = [_ip]
         L.ref_reduce_sum.argtypes = [_fp, _ip, C.c_int, C.c_int, _fp]
+        L.ref_attention_probs.argtypes = [_fp, _fp, _fp, _fp] + [C.c_int] * 5 + [C.c_float]
         L.ref_rectify.argtypes = [_fp, C.c_int, _fp]
         L.ref_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int]
         L.ref_softmax.argtypes = [_fp, _ip, C.c_int, _fp]
@@ -369,6 +382,13 @@ class Reference:
         self.lib.ref_attention(_f(q), _f(k), _f(v), _f(mask) if mask is not None else None, _f(out),
                                batch, lq, k.shape[1], hidden, heads, scale)
         return out
+
+    def attention_probs(self, q, k, heads, scale, mask=None):
+        batch, lq, hidden = q.shape
+        probs = np.zeros((heads, batch, lq, k.shape[1]), np.float32)
+        self.lib.ref_attention_probs(_f(q), _f(k), _f(mask) if mask is not None else None, _f(probs),
+                                     batch, lq, k.shape[1], hidden, heads, scale)
+        return probs
 
     def rectify(self, x):
         y = np.empty_like(x)

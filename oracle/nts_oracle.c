@@ -630,8 +630,9 @@ int oracle_softmax(const float *x, long rows, int n, float *y)
     return 0;
 }
 
-int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
-                     int batch, int lq, int lk, int hidden, int heads, float scale)
+/* shared by the two entry points below: probs (may be NULL) receives Softmax(...), out (may be NULL, then v may be) the result */
+static int attention_chain(const float *q, const float *k, const float *v, const float *mask, float *probs, float *out,
+                           int batch, int lq, int lk, int hidden, int heads, float scale)
 {
     if (heads <= 0 || hidden % heads != 0)
         return -1;
@@ -657,7 +658,8 @@ int oracle_attention(const float *q, const float *k, const float *v, const float
                 for (int l = 0; l < lk; l++)
                     for (int j = 0; j < dh; j++) {
                         kh[(((long)h * batch + b) * lk + l) * dh + j] = k[((long)b * lk + l) * hidden + h * dh + j];
-                        vh[(((long)h * batch + b) * lk + l) * dh + j] = v[((long)b * lk + l) * hidden + h * dh + j];
+                        if (v)
+                            vh[(((long)h * batch + b) * lk + l) * dh + j] = v[((long)b * lk + l) * hidden + h * dh + j];
                     }
             }
         int dq[4] = {heads, batch, lq, dh}, dk[4] = {heads, batch, lk, dh}, da[4] = {heads, batch, lq, lk};
@@ -670,11 +672,13 @@ int oracle_attention(const float *q, const float *k, const float *v, const float
         /* :224 Softmax(att, -1) */
         if (r == 0)
             r = oracle_softmax(att, (long)heads * batch * lq, lk, prob);
+        if (r == 0 && probs)
+            memcpy(probs, prob, sizeof(float) * (size_t)na);
         /* :232-235 BMMul(att, vheads) */
-        if (r == 0)
+        if (r == 0 && out)
             r = oracle_matmul_batched(prob, ORACLE_X_NOTRANS, da, vh, ORACLE_X_NOTRANS, dk, oh, dq, 4, 1.0F, 0.0F);
         /* :239 Merge(att, order - 1): block h goes back to columns h*dh .. (Merge.cpp) */
-        if (r == 0)
+        if (r == 0 && out)
             for (int h = 0; h < heads; h++)
                 for (int b = 0; b < batch; b++)
                     for (int l = 0; l < lq; l++)
@@ -683,6 +687,18 @@ int oracle_attention(const float *q, const float *k, const float *v, const float
     }
     free(qh); free(kh); free(vh); free(att); free(prob); free(oh);
     return r;
+}
+
+int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
+                     int batch, int lq, int lk, int hidden, int heads, float scale)
+{
+    return attention_chain(q, k, v, mask, NULL, out, batch, lq, lk, hidden, heads, scale);
+}
+
+int oracle_attention_probs(const float *q, const float *k, const float *mask, float *probs,
+                           int batch, int lq, int lk, int hidden, int heads, float scale)
+{
+    return attention_chain(q, k, NULL, mask, probs, NULL, batch, lq, lk, hidden, heads, scale);
 }
 
 /* ---- rectify ------------------------------------------------------------------ */

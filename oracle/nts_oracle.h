@@ -103,6 +103,12 @@ int oracle_softmax(const float *x, long rows, int n, float *y);
 int oracle_attention(const float *q, const float *k, const float *v, const float *mask, float *out,
                      int batch, int lq, int lk, int hidden, int heads, float scale);
 
+/* The first half of the same chain, as far as the training path shares it with inference (:194-224): Split, scale of
+   q, BMMul(q, k^T), the mask, Softmax. probs is [heads][batch][lq][lk]: what the reference then passes through Dropout
+   and multiplies with v, and what its backward step needs. */
+int oracle_attention_probs(const float *q, const float *k, const float *mask, float *probs,
+                           int batch, int lq, int lk, int hidden, int heads, float scale);
+
 /* y = max(0, x) as _Rectify computes it (source/tensor/function/Rectify.cpp:47-55): a value below zero
    becomes 0, everything else (negative zero and NaN included) passes */
 void oracle_rectify(const float *x, long n, float *y);

@@ -243,6 +243,33 @@ int ref_attention(const float * q, const float * k, const float * v, const float
     return 0;
 }
 
+/* the same chain up to the Softmax: probs [heads][batch][lq][lk] */
+int ref_attention_probs(const float * q, const float * k, const float * mask, float * probs,
+                        int batch, int lq, int lk, int hidden, int heads, float scale)
+{
+    int dq[3] = {batch, lq, hidden}, dk[3] = {batch, lk, hidden}, dm[4] = {heads, batch, lq, lk};
+    XTensor * tq = Make(dq, 3, q);
+    XTensor * tk = Make(dk, 3, k);
+    XTensor * tm = mask != NULL ? Make(dm, 4, mask) : NULL;
+    bool backup = X_ENABLE_GRAD;
+    X_ENABLE_GRAD = false;
+    {
+        XTensor qh = Split(*tq, 2, heads);
+        XTensor kh = Split(*tk, 2, heads);
+        ScaleAndShiftMe(qh, scale, 0.0F);
+        XTensor att = BMMul(qh, X_NOTRANS, kh, X_TRANS);
+        if (tm != NULL)
+            SumMe(att, *tm);
+        att = Softmax(att, -1);
+        memcpy(probs, att.data, sizeof(float) * (size_t)att.unitNum);
+    }
+    delete tq; delete tk;
+    if (tm != NULL)
+        delete tm;
+    X_ENABLE_GRAD = backup;
+    return 0;
+}
+
 int ref_rectify(const float * x, int n, float * y)
 {
     int dims[1] = {n};

@@ -701,6 +701,21 @@ static bool TestAttention()
             XTensor * gm = masked ? NewGPU(4, dm, m.data()) : NULL;
             XTensor out = AmdAttention(*gq, *gk, *gv, gm, nh, scale);
             out.GetData(got.data());
+            /* the probabilities on their own, as the training path keeps them */
+            {
+                std::vector<float> pref(nh * B * lq * lk), pgot(nh * B * lq * lk);
+                oracle_attention_probs(q.data(), k.data(), masked ? m.data() : NULL, pref.data(), B, lq, lk, H, nh, scale);
+                XTensor probs = AmdAttentionProbs(*gq, *gk, gm, nh, scale);
+                probs.GetData(pgot.data());
+                ok = ok && probs.order == 4 && probs.dimSize[0] == nh && probs.dimSize[1] == B && probs.dimSize[2] == lq && probs.dimSize[3] == lk;
+                float pe = 0;
+                for (size_t i = 0; i < pgot.size(); i++)
+                    pe = fmaxf(pe, fabsf(pgot[i] - pref[i]));
+                if (!(pe < 1e-5F * sqrtf((float)(H / nh)))) {
+                    fprintf(stderr, "attention probabilities case %d masked %d err=%g\n", ci, masked, pe);
+                    ok = false;
+                }
+            }
             float e = MaxRelErr(got, ref);
             if (!(e < 1e-5F * sqrtf((float)(H / nh + lk)))) {
                 fprintf(stderr, "attention case %d masked %d err=%g\n", ci, masked, e);

@@ -124,6 +124,43 @@ def test_attention_shape_of_the_benchmark(gpu, oracle):
     assert np.abs(got - vc).max() <= 1e-5 * np.abs(vc).max() * 4
 
 
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
+    (2, 128, 128, 128, 2, False),      # one key block: one pass
+    (3, 100, 77, 96, 3, True),         # ragged rows and keys: scalar stores
+    (1, 300, 516, 64, 1, True),        # several key blocks: two passes, 16-byte stores
+    (2, 40, 261, 256, 2, False),       # head size 128, ragged
+    (4, 9, 5, 8, 2, False),            # head size 4
+    (1, 1, 1, 12, 1, False),
+])
+def test_probabilities_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
+    """The first half on its own (what the training path keeps): softmax(scale q k^T + mask) as a
+    [heads][batch][lq][lk] tensor, against the oracle's Split, Scale, BMMul, Sum, Softmax."""
+    torch = torch_()
+    q, k = oracle.normal((B, lq, H), 71), oracle.normal((B, lk, H), 72)
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 73, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., lk // 2] = 0.0
+    scale = float(np.float32(1.0 / np.sqrt(H // nh)))
+    ref = oracle.attention_probs(q, k, nh, scale, mask)
+    probs = torch.full((nh, B, lq, lk), float("nan"), device=gpu)
+    nt.attention_probs(dev(q, gpu), dev(k, gpu), probs, nh, scale, mask=dev(mask, gpu) if masked else None)
+    torch.cuda.synchronize()
+    got = probs.cpu().numpy()
+    # probabilities: absolute error against a largest value of at most 1, and rows that sum to 1
+    assert np.isfinite(got).all()
+    assert np.abs(got - ref).max() <= 1e-5 * np.sqrt(H // nh)
+    assert np.abs(got.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+    if masked:
+        assert (got[mask < 0] == 0).all()
+    # followed by the second product it gives the attention of the one-kernel path
+    v = oracle.normal((B, lk, H), 74)
+    whole = run(gpu, q, k, v, nh, scale, mask)
+    vh = v.reshape(B, lk, nh, H // nh).transpose(2, 0, 1, 3).astype(np.float64)
+    two_step = (got.astype(np.float64) @ vh).transpose(1, 2, 0, 3).reshape(B, lq, H)
+    assert np.abs(whole - two_step).max() <= 1e-5 * np.sqrt(H // nh + lk) * np.abs(two_step).max()
+
+
 def halfed(oracle, x):
     return oracle.from_f16_bits(oracle.to_f16_bits(x))
 

@@ -132,3 +132,27 @@ def test_attention_special_cases(oracle):
     # hidden size not divisible by the heads is refused
     with pytest.raises(ValueError):
         oracle.attention(q, k, v, 5, 0.2)
+
+
+def test_attention_probs_against_compiled_reference_and_closed_form(oracle, reference):
+    """The first half of the chain on its own: bit for bit against the reference's operators, rows sum to 1,
+    the closed form in double precision, and consistency with the whole chain."""
+    for i, (B, lq, lk, H, nh, masked) in enumerate([(2, 6, 10, 16, 2, False), (1, 35, 33, 48, 3, True), (2, 17, 96, 64, 4, True)]):
+        q, k, v = oracle.normal((B, lq, H), 170 + i), oracle.normal((B, lk, H), 180 + i), oracle.normal((B, lk, H), 190 + i)
+        mask = None
+        if masked:
+            mask = np.where(oracle.uniform((nh, B, lq, lk), 200 + i, 0.0, 1.0) < 0.4, -1e9, 0.0).astype(np.float32)
+            mask[..., -1] = 0.0
+        scale = float(np.float32(1.0 / np.sqrt(H / nh)))
+        p = oracle.attention_probs(q, k, nh, scale, mask)
+        assert np.array_equal(p, reference.attention_probs(q, k, nh, scale, mask)), i
+        assert np.abs(p.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+        dh = H // nh
+        qh = q.astype(np.float64).reshape(B, lq, nh, dh).transpose(2, 0, 1, 3)
+        kh = k.astype(np.float64).reshape(B, lk, nh, dh).transpose(2, 0, 1, 3)
+        s = scale * (qh @ kh.transpose(0, 1, 3, 2)) + (mask if mask is not None else 0.0)
+        assert np.abs(p - softmax64(s)).max() <= 2e-6
+        # the whole chain is these probabilities times v, merged (in the oracle's own arithmetic: bit for bit)
+        vh = np.ascontiguousarray(v.reshape(B, lk, nh, dh).transpose(2, 0, 1, 3))
+        o = oracle.matmul_batched(p, 1, vh, 1)
+        assert np.array_equal(o.transpose(1, 2, 0, 3).reshape(B, lq, H), oracle.attention(q, k, v, nh, scale, mask))
