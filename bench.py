@@ -53,6 +53,9 @@ def configs():
         11: dict(name="cfg11 fp32 attention probabilities in one kernel: softmax(Q.K^T/8) per head as [8x32x128x128] from q,k [32x128x512] "
                       "(cfg3's first product with the scale, the softmax and the head split folded in)",
                  dtype="f32", M=128, N=128, K=64, batch=256),
+        12: dict(name="cfg12 fp32 attention context on merged tensors: Merge(BMMul(att[8x32x128x128], Split(v[32x128x512]))) as one "
+                      "batched product that reads the heads of v and writes the merged result where they stand",
+                 dtype="f32", M=128, N=64, K=128, batch=256),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -163,6 +166,15 @@ class Workload:
             self.flops = 2.0 * 256 * 128 * 128 * 64
             self.bytes = 4.0 * (2 * 32 * 128 * 512 + 256 * 128 * 128)
             self.launches = 1
+        elif idx == 12:
+            self.p = torch.softmax(g(oracle.normal((8, 32, 128, 128), 1)), -1)
+            self.v = g(oracle.normal((32, 128, 512), 3))
+            self.o = torch.empty((32, 128, 512), device=dev)
+            self.run = lambda: nt.matrix_mul_batched_grid(self.p, NT, 128, (16384, 32 * 16384), self.v, NT, 512, (65536, 64),
+                                                          self.o, 512, (65536, 64), 32, 8, 128, 128, 128, 64, 128, 64)
+            self.flops = 2.0 * 256 * 128 * 128 * 64
+            self.bytes = 4.0 * (256 * 128 * 128 + 2 * 32 * 128 * 512)
+            self.launches = 1
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
@@ -200,7 +212,7 @@ def cpu_baseline(idx, budget_s=12.0):
     # the forward configurations in float run the REAL reference (its CPU sources compiled by oracle/Makefile into
     # oracle/_ref, which travels with the tree) when that library is there; the others (half: the reference has no
     # CPU half arithmetic; the gradient steps) and a tree without it run the restatement
-    use_ref = idx in (1, 2, 3, 5, 8, 10, 11) and Reference.available()
+    use_ref = idx in (1, 2, 3, 5, 8, 10, 11, 12) and Reference.available()
     o = Reference() if use_ref else gen
     if use_ref:
         o.uniform, o.normal = gen.uniform, gen.normal
@@ -210,7 +222,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -239,6 +251,17 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 8 * 2.0 * 128 * 128 * 64
         sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax" % nb
+    elif idx == 12:
+        nb = max(1, min(32, int(budget_s * rate / (8 * 2.0 * 128 * 128 * 64))))
+        p, v = o.uniform((8, nb, 128, 128), 1, 0.0, 1.0), o.normal((nb, 128, 512), 3)
+        t0 = time.perf_counter()
+        # Split and Merge as numpy copies (the reference's are copies too), the product through the library
+        vs = np.ascontiguousarray(v.reshape(nb, 128, 8, 64).transpose(2, 0, 1, 3))
+        c = o.matmul_batched(p, X_NOTRANS, vs, X_NOTRANS)
+        np.ascontiguousarray(c.transpose(1, 2, 0, 3)).reshape(nb, 128, 512)
+        dt = time.perf_counter() - t0
+        fl = nb * 8 * 2.0 * 128 * 128 * 64
+        sample = "%d of 32 sentences, 8 heads each: split of v, batched product, merge" % nb
     elif idx == 7:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, ds = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 128), 3)
@@ -324,7 +347,7 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
     # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
-    if idx in (3, 7, 9, 11):
+    if idx in (3, 7, 9, 11, 12):
         roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
                 "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
     else:
@@ -363,7 +386,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-11 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-12 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -391,7 +414,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

@@ -171,6 +171,30 @@ int ntsamd_matrix_mul_batched_strided(int devID, void * stream,
                                       float alpha, float beta);
 
 /*
+ * count0 x count1 products whose matrices stand inside larger tensors: item
+ * (i0, i1), i0 < count0, i1 < count1, is the na x ma matrix whose rows are
+ * lda >= ma elements apart and whose first element is a + i0 * strideA0 +
+ * i1 * strideA1 (likewise b and c; strides in ELEMENTS, 0 shares an operand).
+ * This is how the heads of a merged [batch, length, heads * width] tensor are
+ * multiplied where they stand, and how the result is written in merged form:
+ * it replaces _CudaBLASMatrixMULBatchedStrided (source/tensor/core/arithmetic/
+ * XTensorBLAS.cu:181-247, where cuBLAS's lda/ldb/ldc are fixed to ma/mb/mc)
+ * TOGETHER WITH the Split before it and the Merge after it, which copy
+ * every tensor once (source/tensor/core/shape/Split.cpp:42-150, Merge.cpp:47-165;
+ * used so in source/sample/transformer/submodel/Attention.cpp:197-201 and :241-242).
+ * The result matrices may interleave but must not overlap.
+ */
+int ntsamd_matrix_mul_batched_grid(int devID, void * stream,
+                                   const void * a, int transposedA, int dataTypeA, int lda,
+                                   long long strideA0, long long strideA1,
+                                   const void * b, int transposedB, int dataTypeB, int ldb,
+                                   long long strideB0, long long strideB1,
+                                   void * c, int dataTypeC, int ldc,
+                                   long long strideC0, long long strideC1,
+                                   int count0, int count1, int na, int ma, int nb, int mb, int nc, int mc,
+                                   float alpha, float beta);
+
+/*
  * `count` products over arbitrary same-shaped matrices. a, b and c are HOST
  * arrays of `count` DEVICE pointers. Replaces
  *   _CudaBLASMatrixMULBatched(handle, a, ..., count, na, ma, nb, mb, nc, mc, alpha, beta)

@@ -28,6 +28,7 @@ EXPORTS = (
     "ntsamd_matrix_mul_bias_act",
     "ntsamd_matrix_mul_batched_strided",
     "ntsamd_matrix_mul_batched",
+    "ntsamd_matrix_mul_batched_grid",
     "ntsamd_matrix_mul_colsum",
     "ntsamd_reduce_sum_xz",
     "ntsamd_attention",
@@ -66,6 +67,8 @@ def load():
     L.ntsamd_matrix_mul_bias_act.argtypes = L.ntsamd_matrix_mul_bias.argtypes + [ci]
     L.ntsamd_matrix_mul_batched_strided.argtypes = [ci, vp, vp, ci, ci, ll, vp, ci, ci, ll, vp, ci, ll,
                                                     ci] + [ci] * 6 + [cf, cf]
+    L.ntsamd_matrix_mul_batched_grid.argtypes = [ci, vp, vp, ci, ci, ci, ll, ll, vp, ci, ci, ci, ll, ll,
+                                                 vp, ci, ci, ll, ll, ci, ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_batched.argtypes = [ci, vp, C.POINTER(vp), ci, ci, C.POINTER(vp), ci, ci, C.POINTER(vp), ci,
                                             ci] + [ci] * 6 + [cf, cf]
     L.ntsamd_matrix_mul_colsum.argtypes = [ci, vp, vp, ci, ci, vp, ci, ci, vp, ci] + [ci] * 6 + [cf, cf, vp, cf]
@@ -135,6 +138,20 @@ def matrix_mul_batched_strided(a, transA, b, transB, c, count, strideA, strideB,
                                              b.data_ptr(), transB, _dtype_code(b), strideB,
                                              c.data_ptr(), _dtype_code(c), strideC,
                                              count, na, ma, nb, mb, nc, mc, alpha, beta)
+    _check(rc)
+    return c
+
+
+def matrix_mul_batched_grid(a, transA, lda, stridesA, b, transB, ldb, stridesB, c, ldc, stridesC,
+                            count0, count1, na, ma, nb, mb, nc, mc, alpha=1.0, beta=0.0):
+    """count0 x count1 products whose matrices stand inside larger tensors: item (i0, i1) of an operand starts
+    at i0 * strides[0] + i1 * strides[1] elements and has rows ld elements apart."""
+    L = load()
+    rc = L.ntsamd_matrix_mul_batched_grid(a.device.index, _stream_ptr(a),
+                                          a.data_ptr(), transA, _dtype_code(a), lda, stridesA[0], stridesA[1],
+                                          b.data_ptr(), transB, _dtype_code(b), ldb, stridesB[0], stridesB[1],
+                                          c.data_ptr(), _dtype_code(c), ldc, stridesC[0], stridesC[1],
+                                          count0, count1, na, ma, nb, mb, nc, mc, alpha, beta)
     _check(rc)
     return c
 

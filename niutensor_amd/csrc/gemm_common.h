@@ -5,8 +5,10 @@
  * All matrices are dense and row-major. A "K-contiguous" operand stores the
  * reduction index fastest (a with X_NOTRANS, b with X_TRANS); an
  * "MN-contiguous" operand stores the output index fastest (a with X_TRANS,
- * b with X_NOTRANS). The leading dimension is always the stored column count,
- * as in the reference's BLAS calls (XTensorBLAS.cu:64-71: lda=ma, ldb=mb, ldc=mc).
+ * b with X_NOTRANS). The leading dimension is the stored column count in the
+ * reference's BLAS calls (XTensorBLAS.cu:64-71: lda=ma, ldb=mb, ldc=mc); the kernels
+ * take any leading dimension of at least that, which is how the heads of a merged
+ * [batch, length, heads * width] tensor are multiplied where they stand.
  */
 #pragma once
 #include <hip/hip_runtime.h>
@@ -50,6 +52,10 @@ struct GemmParams {
     int M, N, K;
     int lda, ldb, ldc;
     long long strideA, strideB, strideC;   /* elements between batch items; 0 = shared operand */
+    /* a batch laid out as a grid: item i stands at (i % batchInner) * stride + (i / batchInner) * stride1
+       (heads of a [batch, length, heads * width] tensor, say). batchInner == 0: items `stride` apart. */
+    int batchInner;
+    long long strideA1, strideB1, strideC1;
     float alpha, beta;
     int biasMode;                          /* BiasMode */
     int biasRowDiv, biasLen;               /* BIAS_ROW: index = (row / biasRowDiv) % biasLen */
@@ -76,6 +82,15 @@ __device__ __forceinline__ int xcd_contiguous_id(int id, int total)
     int per = total / X, rem = total % X;
     int xcd = id % X, idx = id / X;
     return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+/* first element of batch item `item` of an operand */
+__device__ __forceinline__ long long batch_offset(int item, int inner, long long stride0, long long stride1)
+{
+    if (inner <= 0)
+        return (long long)item * stride0;
+    const int outer = item / inner;
+    return (long long)(item - outer * inner) * stride0 + (long long)outer * stride1;
 }
 
 struct TileCoord {

@@ -109,9 +109,9 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         C = static_cast<OutT *>(tab.c[tc.batch]);
     }
     else {
-        A = static_cast<const half_t *>(p.a) + (long long)tc.batch * p.strideA;
-        B = static_cast<const half_t *>(p.b) + (long long)tc.batch * p.strideB;
-        C = static_cast<OutT *>(p.c) + (long long)tc.batch * p.strideC;
+        A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
+        B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
+        C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
     }
 
     const int M = p.M, N = p.N, K = p.K;
@@ -167,8 +167,8 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
 
     const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
     const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const half_t * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
-    const half_t * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+    const half_t * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
+    const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
 
     f16x8 ra[NA], rb[NB];
 

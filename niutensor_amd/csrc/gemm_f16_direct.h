@@ -104,9 +104,9 @@ gemm_f16_direct_kernel(const GemmParams p)
     __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
     const TileCoord tc = tile_of_workgroup(p);
-    const half_t * __restrict__ A = static_cast<const half_t *>(p.a) + (long long)tc.batch * p.strideA;
-    const half_t * __restrict__ B = static_cast<const half_t *>(p.b) + (long long)tc.batch * p.strideB;
-    OutT * __restrict__ C = static_cast<OutT *>(p.c) + (long long)tc.batch * p.strideC;
+    const half_t * __restrict__ A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
+    const half_t * __restrict__ B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
+    OutT * __restrict__ C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
 
     const int M = p.M, N = p.N, K = p.K;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
@@ -159,8 +159,8 @@ gemm_f16_direct_kernel(const GemmParams p)
 
     const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
     const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const half_t * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
-    const half_t * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+    const half_t * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
+    const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
 
     const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);
 

@@ -89,9 +89,9 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         C = static_cast<float *>(tab.c[tc.batch]);
     }
     else {
-        A = static_cast<const float *>(p.a) + (long long)tc.batch * p.strideA;
-        B = static_cast<const float *>(p.b) + (long long)tc.batch * p.strideB;
-        C = static_cast<float *>(p.c) + (long long)tc.batch * p.strideC;
+        A = static_cast<const float *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
+        B = static_cast<const float *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
+        C = static_cast<float *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
     }
 
     const int M = p.M, N = p.N, K = p.K;
@@ -149,8 +149,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     /* first element of the tile's operand panels, and one past the end of each matrix */
     const float * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
     const float * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const float * aEnd = A + (size_t)(AKC ? M : K) * p.lda;
-    const float * bEnd = B + (size_t)(BKC ? N : K) * p.ldb;
+    const float * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
+    const float * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
 
     f32x4 ra[NA], rb[NB];
 

@@ -206,6 +206,12 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit)
     return best;
 }
 
+/* a batch laid out as a grid of `inner` x (count / inner) items: the second set of strides */
+struct Grid {
+    int inner;
+    long long strideA1, strideB1, strideC1;
+};
+
 int run(int devID, void * stream, Kind kind, const Shape & s,
         const void * a, const void * b, void * c,
         int lda, int ldb, int ldc,
@@ -213,7 +219,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         const PtrBatch * ptrs,
         float alpha, float beta,
         const void * bias, int biasMode, int biasLen, int biasRowDiv,
-        void * colSum = NULL, float colSumBeta = 0.f, int act = ACT_NONE)
+        void * colSum = NULL, float colSumBeta = 0.f, int act = ACT_NONE, const Grid * grid = NULL)
 {
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
@@ -248,21 +254,31 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.batch = count;
     p.groupM = 8;
     p.act = act;
+    if (grid) {
+        p.batchInner = grid->inner;
+        p.strideA1 = grid->strideA1;
+        p.strideB1 = grid->strideB1;
+        p.strideC1 = grid->strideC1;
+    }
+    const int colsA = s.aKContig ? s.K : s.M, colsB = s.bKContig ? s.K : s.N;
+    const bool dense = !grid && lda == colsA && ldb == colsB && ldc == s.N;
 
     /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. It keeps a
        tile's byte offsets in 31 bits, so rows longer than 2M elements go through the generic path, like
        row-indexed bias and lists of half matrices. Float operands need no alignment beyond their own 4 bytes (a
        16-byte buffer load may start on any dword, and is range-checked dword by dword); half operands
-       travel to LDS 16 bytes at a time and must have 16-byte aligned rows. */
+       travel to LDS 16 bytes at a time and must have 16-byte aligned rows of whole 16-byte pieces. */
     bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
     if (kind != KIND_F32)
-        vec = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && aligned16(a) && aligned16(b) &&
-              strideA % 8 == 0 && strideB % 8 == 0;
+        vec = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
+              aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
+              (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
-    const Plan plan = choose_plan(s.M, s.N, s.K, count, half, kind == KIND_F32 && vec && !ptrs && act == ACT_NONE);
+    const Plan plan = choose_plan(s.M, s.N, s.K, count, half,
+                                  kind == KIND_F32 && vec && !ptrs && act == ACT_NONE && dense);
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;
@@ -660,6 +676,63 @@ int ntsamd_matrix_mul_batched_strided(int devID, void * stream,
         return fail(NTSAMD_ERR_ARGUMENT, "result matrices of the batch overlap");
     return run(devID, stream, kind, s, a, b, c, ma, mb, mc, strideA, strideB, strideC, count, NULL,
                alpha, beta, NULL, NTSAMD_BIAS_NONE, 0, 1);
+}
+
+int ntsamd_matrix_mul_batched_grid(int devID, void * stream,
+                                   const void * a, int transposedA, int dataTypeA, int lda,
+                                   long long strideA0, long long strideA1,
+                                   const void * b, int transposedB, int dataTypeB, int ldb,
+                                   long long strideB0, long long strideB1,
+                                   void * c, int dataTypeC, int ldc,
+                                   long long strideC0, long long strideC1,
+                                   int count0, int count1, int na, int ma, int nb, int mb, int nc, int mc,
+                                   float alpha, float beta)
+{
+    Kind kind;
+    Shape s;
+    int st = check_types(dataTypeA, dataTypeB, dataTypeC, kind);
+    if (st == NTSAMD_OK)
+        st = check_shape(transposedA, transposedB, na, ma, nb, mb, nc, mc, s);
+    if (st != NTSAMD_OK)
+        return st;
+    if (count0 < 0 || count1 < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative batch count");
+    if ((long long)count0 * count1 > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "too many batch items");
+    if (count0 == 0 || count1 == 0 || s.M == 0 || s.N == 0)
+        return NTSAMD_OK;
+    st = check_pointers(a, b, c);
+    if (st != NTSAMD_OK)
+        return st;
+    if (lda < ma || ldb < mb || ldc < mc)
+        return fail(NTSAMD_ERR_ARGUMENT, "leading dimension shorter than a row (lda %d for %d, ldb %d for %d, ldc %d for %d)",
+                    lda, ma, ldb, mb, ldc, mc);
+    if (strideA0 < 0 || strideA1 < 0 || strideB0 < 0 || strideB1 < 0 || strideC0 < 0 || strideC1 < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative batch stride");
+    /* results may interleave (heads side by side in one row of a merged tensor) but must not overlap:
+       rows and the two axes of the grid, taken from the shortest stride up, must each step over
+       everything the shorter ones span */
+    {
+        long long stride[3] = {ldc, strideC0, strideC1};
+        long long count[3] = {nc, count0, count1};
+        for (int i = 0; i < 3; i++)
+            for (int j = i + 1; j < 3; j++)
+                if (stride[j] < stride[i]) {
+                    long long t = stride[i]; stride[i] = stride[j]; stride[j] = t;
+                    t = count[i]; count[i] = count[j]; count[j] = t;
+                }
+        long long span = mc;
+        for (int i = 0; i < 3; i++) {
+            if (count[i] <= 1)
+                continue;
+            if (stride[i] < span)
+                return fail(NTSAMD_ERR_ARGUMENT, "result matrices of the batch overlap");
+            span += (count[i] - 1) * stride[i];
+        }
+    }
+    Grid g = {count0, strideA1, strideB1, strideC1};
+    return run(devID, stream, kind, s, a, b, c, lda, ldb, ldc, strideA0, strideB0, strideC0, count0 * count1, NULL,
+               alpha, beta, NULL, NTSAMD_BIAS_NONE, 0, 1, NULL, 0.f, ACT_NONE, &g);
 }
 
 int ntsamd_matrix_mul_batched(int devID, void * stream,

@@ -109,4 +109,51 @@ XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * 
     return probs;
 }
 
+void _AmdAttentionContext(const XTensor * probs, const XTensor * v, XTensor * out, int nhead)
+{
+    CheckNTErrors((probs && v && out), "Empty input tensors!");
+    CheckNTErrors((probs->dataType == v->dataType && probs->dataType == out->dataType), "Unmatched data types!");
+    CheckNTErrors((v->dataType == X_FLOAT || v->dataType == X_FLOAT16), "TODO!");
+    CheckNTErrors((v->order >= 2 && out->order == v->order && probs->order == v->order + 1),
+                  "Input tensors must have the same order >= 2!");
+    CheckNTErrors((v->devID >= 0), "This code must be run on GPUs!");
+    CheckNTErrors((v->devID == probs->devID && v->devID == out->devID), "The tensors must be on the same GPU!");
+
+    const int order = v->order;
+    const int hidden = v->dimSize[order - 1];
+    const int lk = v->dimSize[order - 2], lq = out->dimSize[order - 2];
+    CheckNTErrors((nhead > 0 && hidden % nhead == 0), "The hidden size must be a multiple of the number of heads!");
+    CheckNTErrors((out->dimSize[order - 1] == hidden), "Unmatched tensors in attention!");
+    int batch = 1;
+    for (int i = 0; i < order - 2; i++) {
+        CheckNTErrors((v->dimSize[i] == out->dimSize[i]), "Unmatched tensors in attention!");
+        batch *= v->dimSize[i];
+    }
+    CheckNTErrors((probs->dimSize[0] == nhead && probs->dimSize[order] == lk && probs->dimSize[order - 1] == lq &&
+                   probs->unitNum == nhead * batch * lq * lk), "Unmatched tensors in attention!");
+    const int dh = hidden / nhead;
+    /* item (b, h): probs[h][b] is dense, the heads of v and out are dh columns of rows `hidden` long */
+    int rc = ntsamd_matrix_mul_batched_grid(v->devID, NULL,
+                                            probs->data, X_NOTRANS, probs->dataType, lk, (long long)lq * lk, (long long)batch * lq * lk,
+                                            v->data, X_NOTRANS, v->dataType, hidden, (long long)lk * hidden, dh,
+                                            out->data, out->dataType, hidden, (long long)lq * hidden, dh,
+                                            batch, nhead, lq, lk, lk, dh, lq, dh, 1.0F, 0.0F);
+    if (rc != NTSAMD_OK) {
+        ShowNTErrors(ntsamd_last_error());
+    }
+}
+
+XTensor AmdAttentionContext(const XTensor & probs, const XTensor & v, int nhead)
+{
+    CheckNTErrors((v.order >= 2 && probs.order == v.order + 1), "Input tensors must have the same order >= 2!");
+    int dims[MAX_TENSOR_DIM_NUM];
+    for (int i = 0; i < v.order; i++)
+        dims[i] = v.dimSize[i];
+    dims[v.order - 2] = probs.dimSize[probs.order - 2];
+    XTensor out(v.order, dims, v.dataType, 1.0F, v.devID, v.mem);
+    out.SetTMPFlag();
+    _AmdAttentionContext(&probs, &v, &out, nhead);
+    return out;
+}
+
 }  // namespace nts

@@ -27,5 +27,12 @@ XTensor AmdAttention(const XTensor & q, const XTensor & k, const XTensor & v, co
 void _AmdAttentionProbs(const XTensor * q, const XTensor * k, const XTensor * mask, XTensor * probs, int nhead, DTYPE scale);
 XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * mask, int nhead, DTYPE scale);
 
+/* out = Merge(probs x Split(v)): the end of MakeAttention (:235-242) after Softmax and Dropout, as one batched
+   product that reads the heads of v where they stand in (batch..., lk, hidden) and writes out in merged form
+   (batch..., lq, hidden); neither Split nor Merge copies anything. probs: (nhead, batch..., lq, lk).
+   All X_FLOAT or all X_FLOAT16. */
+void _AmdAttentionContext(const XTensor * probs, const XTensor * v, XTensor * out, int nhead);
+XTensor AmdAttentionContext(const XTensor & probs, const XTensor & v, int nhead);
+
 }  // namespace nts
 #endif

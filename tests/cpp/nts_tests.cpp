@@ -715,6 +715,17 @@ static bool TestAttention()
                     fprintf(stderr, "attention probabilities case %d masked %d err=%g\n", ci, masked, pe);
                     ok = false;
                 }
+                /* ... and the product with the heads of v where they stand, written in merged form: the two
+                   calls together are the whole chain */
+                std::vector<float> cgot(B * lq * H);
+                XTensor ctx = AmdAttentionContext(probs, *gv, nh);
+                ctx.GetData(cgot.data());
+                ok = ok && ctx.order == 3 && ctx.dimSize[0] == B && ctx.dimSize[1] == lq && ctx.dimSize[2] == H;
+                float ce = MaxRelErr(cgot, ref);
+                if (!(ce < 1e-5F * sqrtf((float)(H / nh + lk)))) {
+                    fprintf(stderr, "attention context case %d masked %d err=%g\n", ci, masked, ce);
+                    ok = false;
+                }
             }
             float e = MaxRelErr(got, ref);
             if (!(e < 1e-5F * sqrtf((float)(H / nh + lk)))) {
