@@ -143,6 +143,30 @@ def test_convert_and_attention_argument_errors_need_no_device():
     assert L.ntsamd_matrix_mul_bias_act(0, None, p, 1, 2, p, 1, 2, p, 2, 8, 8, 8, 8, 8, 8, 1.0, 0.0, p, 1, 8, 1, 7) == 1
 
 
+def test_grid_batch_argument_errors_need_no_device():
+    L = nt.load()
+    p = 0x1000
+    g = L.ntsamd_matrix_mul_batched_grid
+
+    def call(lda=8, sa=(64, 0), ldb=8, sb=(64, 0), ldc=8, sc=(64, 128), counts=(2, 2), types=(2, 2, 2), a=p):
+        return g(0, None, a, 1, types[0], lda, sa[0], sa[1], p, 1, types[1], ldb, sb[0], sb[1],
+                 p, types[2], ldc, sc[0], sc[1], counts[0], counts[1], 8, 8, 8, 8, 8, 8, 1.0, 0.0)
+
+    assert call(lda=7) == 1 and "leading dimension" in L.ntsamd_last_error().decode()
+    assert call(ldc=4) == 1
+    assert call(sa=(-1, 0)) == 1 and "negative" in L.ntsamd_last_error().decode()
+    assert call(counts=(-2, 2)) == 1
+    assert call(counts=(1 << 16, 1 << 16)) == 1 and "too many" in L.ntsamd_last_error().decode()
+    assert call(counts=(0, 2)) == 0                                       # nothing to do
+    assert call(a=None) == 1
+    assert call(types=(2, 3, 2)) == 2                                     # float times half
+    # results: two items in the same place; heads side by side but rows too short for both; heads side by
+    # side with the next batch item starting inside the last row
+    assert call(sc=(0, 128)) == 1 and "overlap" in L.ntsamd_last_error().decode()
+    assert call(ldc=12, sc=(8, 128)) == 1
+    assert call(ldc=16, sc=(8, 7 * 16 + 8)) == 1
+
+
 def test_invalid_device_is_an_error():
     L = nt.load()
     rc = L.ntsamd_init(12345)
