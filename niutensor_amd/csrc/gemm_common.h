@@ -131,7 +131,11 @@ template <> struct TileShape<CFG_256x256> { static constexpr int BM = 256, BN = 
 
 int launch_f32(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,
                bool vec, int cfg, hipStream_t stream);
+/* vec: how a and b are fetched. F16_SCALAR: element by element, every bias mode; F16_DIRECT: 16 bytes per lane
+   straight to LDS (16-byte aligned rows of whole 16-byte pieces); F16_STAGED: 16 bytes per lane through
+   registers, any alignment and row length */
+enum F16Fetch { F16_SCALAR = 0, F16_DIRECT = 1, F16_STAGED = 2 };
 int launch_f16(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,
-               bool vec, bool outF32, int cfg, hipStream_t stream);
+               int vec, bool outF32, int cfg, hipStream_t stream);
 
 }  // namespace ntsamd

@@ -42,6 +42,23 @@ __device__ __forceinline__ f16x8 buffer_load_f16x8(__amdgpu_buffer_rsrc_t rsrc, 
 }
 
 /* transposing LDS read: see the header comment for what each lane receives */
+/* Eight halves from any 2-byte aligned place in a buffer of `bytes` bytes. A 16-byte buffer load may start on any
+   even address, but its range check works on whole dwords: where the eight halves hang over the end of the buffer
+   the dword that straddles the end is dropped with its valid half. Such a piece (the last of the matrix, at most)
+   is fetched half by half instead; the branch is taken by no lane almost everywhere. */
+__device__ __forceinline__ f16x8 buffer_load_f16x8_any(__amdgpu_buffer_rsrc_t rsrc, int byteOffset, int bytes)
+{
+    f16x8 v;
+    if ((unsigned)byteOffset < (unsigned)bytes && (unsigned)byteOffset + 16u > (unsigned)bytes) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            v[e] = __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(rsrc, byteOffset + 2 * e, 0, 0));
+    }
+    else
+        v = buffer_load_f16x8(rsrc, byteOffset);
+    return v;
+}
+
 __device__ __forceinline__ f16x4 lds_read_tr16(const half_t * p)
 {
     typedef __fp16 hv4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
@@ -141,8 +158,9 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             aK[s] = g / (BM / 8);
             aMN[s] = (g % (BM / 8)) * 8;
             aLds[s] = aK[s] * LDA + aMN[s];
-            int c = m0 + aMN[s] < M - 8 ? aMN[s] : M - 8 - m0;  /* 16-byte path: M % 8 == 0 */
-            aOff[s] = (aK[s] * p.lda + c) * 2;
+            /* columns past M are fetched from nowhere (zeros); a piece that straddles M runs on into the next
+               row of k, into columns of the tile that are never stored */
+            aOff[s] = m0 + aMN[s] < M ? (aK[s] * p.lda + aMN[s]) * 2 : NTSAMD_OOB_OFFSET;
         }
     }
 #pragma unroll
@@ -160,8 +178,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             bK[s] = g / (BN / 8);
             bMN[s] = (g % (BN / 8)) * 8;
             bLds[s] = bK[s] * LDB + bMN[s];
-            int c = n0 + bMN[s] < N - 8 ? bMN[s] : N - 8 - n0;
-            bOff[s] = (bK[s] * p.ldb + c) * 2;
+            bOff[s] = n0 + bMN[s] < N ? (bK[s] * p.ldb + bMN[s]) * 2 : NTSAMD_OOB_OFFSET;
         }
     }
 
@@ -177,25 +194,40 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         if constexpr (VEC) {
             const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
             const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
-            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, (long long)(aEnd - ab) * 2);
-            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, (long long)(bEnd - bb) * 2);
+            const long long aLeft = (long long)(aEnd - ab) * 2, bLeft = (long long)(bEnd - bb) * 2;
+            const int aBytes = aLeft >> 31 ? 0x7fffffff : (int)aLeft, bBytes = bLeft >> 31 ? 0x7fffffff : (int)bLeft;
+            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, aLeft);
+            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, bLeft);
             /* rows of k past the end of an MN-contiguous matrix read as zero by themselves;
                a K-contiguous row would run on into the next row, so those lanes are sent
-               out of range explicitly (last slab only) */
+               out of range explicitly, and the halves of a piece that straddles K are set to zero
+               (last slab only) */
             const bool tail = mayHangOver && k0 + BKT > K;
 #pragma unroll
             for (int s = 0; s < NA; s++) {
                 int off = aOff[s];
                 if (AKC && tail && k0 + aK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                ra[s] = buffer_load_f16x8(ar, off);
+                ra[s] = buffer_load_f16x8_any(ar, off, aBytes);
+                if constexpr (mayHangOver && AKC)
+                    if (tail) {
+#pragma unroll
+                        for (int e = 1; e < 8; e++)
+                            ra[s][e] = k0 + aK[s] + e < K ? ra[s][e] : (half_t)0;
+                    }
             }
 #pragma unroll
             for (int s = 0; s < NB; s++) {
                 int off = bOff[s];
                 if (BKC && tail && k0 + bK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                rb[s] = buffer_load_f16x8(br, off);
+                rb[s] = buffer_load_f16x8_any(br, off, bBytes);
+                if constexpr (mayHangOver && BKC)
+                    if (tail) {
+#pragma unroll
+                        for (int e = 1; e < 8; e++)
+                            rb[s][e] = k0 + bK[s] + e < K ? rb[s][e] : (half_t)0;
+                    }
             }
         }
         else {

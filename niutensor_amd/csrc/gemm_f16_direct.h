@@ -553,21 +553,30 @@ static int launch_f16_direct(const GemmParams & p0, hipStream_t stream)
     return (int)hipGetLastError();
 }
 
-template <bool AKC, bool BKC>
-static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, bool vec, bool outF32, int cfg,
-                            hipStream_t stream)
+template <typename OutT, bool AKC, bool BKC, bool VEC>
+static int launch_f16_staged(const GemmParams & p, const PtrBatch * ptrs, int cfg, hipStream_t stream)
 {
     NoPtrs none = {0};
-    if (ptrs) {
-        if (outF32)
-            return launch_f16_one<float, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
-        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, PtrBatch>(p, *ptrs, stream);
+    if constexpr (VEC) if (cfg != CFG_64x64) {
+        if (ptrs)
+            return launch_f16_one<OutT, CFG_128x128, AKC, BKC, VEC, PtrBatch>(p, *ptrs, stream);
+        return launch_f16_one<OutT, CFG_128x128, AKC, BKC, VEC, NoPtrs>(p, none, stream);
     }
-    if (!vec) {
-        if (outF32)
-            return launch_f16_one<float, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
-        return launch_f16_one<half_t, CFG_64x64, AKC, BKC, false, NoPtrs>(p, none, stream);
-    }
+    if (ptrs)
+        return launch_f16_one<OutT, CFG_64x64, AKC, BKC, VEC, PtrBatch>(p, *ptrs, stream);
+    return launch_f16_one<OutT, CFG_64x64, AKC, BKC, VEC, NoPtrs>(p, none, stream);
+}
+
+template <bool AKC, bool BKC>
+static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, int vec, bool outF32, int cfg,
+                            hipStream_t stream)
+{
+    if (vec == F16_STAGED)
+        return outF32 ? launch_f16_staged<float, AKC, BKC, true>(p, ptrs, cfg, stream)
+                      : launch_f16_staged<half_t, AKC, BKC, true>(p, ptrs, cfg, stream);
+    if (vec == F16_SCALAR || ptrs)
+        return outF32 ? launch_f16_staged<float, AKC, BKC, false>(p, ptrs, cfg, stream)
+                      : launch_f16_staged<half_t, AKC, BKC, false>(p, ptrs, cfg, stream);
     /* a float result: the same main loop, 4-byte stores from the accumulators */
     if (outF32) {
         if (cfg == CFG_256x256)

@@ -19,10 +19,10 @@ int launch_f32_nn(const GemmParams &, const PtrBatch *, bool, int, hipStream_t);
 int launch_f32_nt(const GemmParams &, const PtrBatch *, bool, int, hipStream_t);
 int launch_f32_tn(const GemmParams &, const PtrBatch *, bool, int, hipStream_t);
 int launch_f32_tt(const GemmParams &, const PtrBatch *, bool, int, hipStream_t);
-int launch_f16_nn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
-int launch_f16_nt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
-int launch_f16_tn(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
-int launch_f16_tt(const GemmParams &, const PtrBatch *, bool, bool, int, hipStream_t);
+int launch_f16_nn(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
+int launch_f16_nt(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
+int launch_f16_tn(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
+int launch_f16_tt(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
 int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
 int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream);
@@ -263,16 +263,24 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const int colsA = s.aKContig ? s.K : s.M, colsB = s.bKContig ? s.K : s.N;
     const bool dense = !grid && lda == colsA && ldb == colsB && ldc == s.N;
 
-    /* the fast path: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. It keeps a
+    /* the fast paths: 16-byte buffer loads of a and b, buffer stores of c, bias by column only. They keep a
        tile's byte offsets in 31 bits, so rows longer than 2M elements go through the generic path, like
-       row-indexed bias and lists of half matrices. Float operands need no alignment beyond their own 4 bytes (a
-       16-byte buffer load may start on any dword, and is range-checked dword by dword); half operands
-       travel to LDS 16 bytes at a time and must have 16-byte aligned rows of whole 16-byte pieces. */
+       row-indexed bias. Float operands need no alignment beyond their own 4 bytes (a 16-byte buffer load may
+       start on any dword, and is range-checked dword by dword). Half operands with 16-byte aligned rows of whole
+       16-byte pieces travel straight to LDS (the main path); all other half operands, and lists of half
+       matrices, are fetched 16 bytes at a time through registers, from any even address. */
     bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
-    if (kind != KIND_F32)
-        vec = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
-              aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
-              (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
+    int fetch16 = F16_SCALAR;
+    if (kind != KIND_F32) {
+        const bool direct = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
+                            aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
+                            (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
+        fetch16 = direct ? F16_DIRECT : (vec ? F16_STAGED : F16_SCALAR);
+        const char * e = getenv("NTSAMD_F16_FETCH");              /* 0 or 2: keep off the main path (for measurements) */
+        if (e && e[1] == 0 && (e[0] == '0' || (e[0] == '2' && vec)))
+            fetch16 = e[0] - '0';
+        vec = fetch16 == F16_DIRECT;                               /* what the column-sum by-product needs */
+    }
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
@@ -322,9 +330,9 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     else {
         bool outF32 = kind == KIND_F16_F32OUT;
         if (s.aKContig)
-            rc = s.bKContig ? launch_f16_nt(p, ptrs, vec, outF32, cfg, hs) : launch_f16_nn(p, ptrs, vec, outF32, cfg, hs);
+            rc = s.bKContig ? launch_f16_nt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_nn(p, ptrs, fetch16, outF32, cfg, hs);
         else
-            rc = s.bKContig ? launch_f16_tt(p, ptrs, vec, outF32, cfg, hs) : launch_f16_tn(p, ptrs, vec, outF32, cfg, hs);
+            rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, cfg, hs);
     }
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));

@@ -302,7 +302,7 @@ def test_backward_of_the_ragged_vocabulary_projection(gpu, oracle):
 
 def test_unaligned_operands(gpu, oracle):
     """Base pointers and leading dimensions that are not multiples of 16 bytes (float: still the main
-    path; half: the generic path)."""
+    path; half: 16-byte loads through registers from any even address)."""
     torch = torch_()
     M, N, K = 70, 52, 36
     for ta, tb in TRANS:
@@ -325,6 +325,49 @@ def test_unaligned_operands(gpu, oracle):
                 assert_fp16(c.float().cpu().numpy(), oracle.matmul2d(ah, ta, bh, tb))
             else:
                 assert_fp32(c.cpu().numpy(), ref, K)
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("out_float", [False, True])
+def test_half_rows_of_any_length_and_alignment(gpu, oracle, ta, tb, out_float):
+    """Half operands whose rows are no multiple of 16 bytes, at bases that are only 2-byte aligned, in buffers
+    that end with the matrix: they are fetched 16 bytes at a time all the same, and the piece that hangs over
+    the end of a buffer (whose last dword the range check would drop with its valid half) is fetched half by
+    half. Sizes that need the 128 x 128 tile, ragged in every dimension; the last row and column of the result
+    are checked on their own, since that is where a lost element would show."""
+    torch = torch_()
+    for (M, N, K) in ((203, 301, 77), (131, 135, 259), (9, 7, 5), (1, 300, 1)):
+        a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((M, K), ta), 31)))
+        b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((K, N), tb), 32)))
+        bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((N,), 33)))
+        ref = oracle.matmul2d(a, ta, b, tb) + bias[None, :]
+        odt = torch.float32 if out_float else torch.float16
+        for off in (0, 1):
+            # the matrices end exactly where their buffers end
+            abuf = torch.zeros(a.size + off, device=gpu, dtype=torch.float16)
+            bbuf = torch.zeros(b.size + off, device=gpu, dtype=torch.float16)
+            abuf[off:] = dev_tensor(a.ravel(), gpu, True)
+            bbuf[off:] = dev_tensor(b.ravel(), gpu, True)
+            c = torch.full((M, N), float("nan"), device=gpu, dtype=odt)
+            nt.matrix_mul(abuf[off:].view(a.shape), ta, bbuf[off:].view(b.shape), tb, c,
+                          bias=dev_tensor(bias, gpu, True).to(odt))
+            got = c.float().cpu().numpy()
+            assert_fp16(got, ref, what="%dx%dx%d offset %d" % (M, N, K, off))
+            assert_fp16(got[-1:, :], ref[-1:, :], what="last row")
+            assert_fp16(got[:, -1:], ref[:, -1:], what="last column")
+
+
+def test_lists_of_half_matrices_with_odd_rows(gpu, oracle):
+    """Pointer lists of half matrices take the same 16-byte loads (no alignment to rely on)."""
+    torch = torch_()
+    M, N, K, count = 67, 45, 131, 5
+    a = [oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((M, K), 40 + i))) for i in range(count)]
+    b = [oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((N, K), 50 + i))) for i in range(count)]
+    ad = [dev_tensor(x, gpu, True) for x in a]
+    bd = [dev_tensor(x, gpu, True) for x in b]
+    cd = [torch.full((M, N), float("nan"), device=gpu, dtype=torch.float16) for _ in range(count)]
+    nt.matrix_mul_batched(ad, X_NOTRANS, bd, X_TRANS, cd, 0.5, 0.0)
+    for i in range(count):
+        assert_fp16(cd[i].float().cpu().numpy(), oracle.matmul2d(a[i], X_NOTRANS, b[i], X_TRANS, alpha=0.5), what="item %d" % i)
 
 
 def test_beta_zero_ignores_old_contents_and_scaling_is_exact(gpu, oracle):
