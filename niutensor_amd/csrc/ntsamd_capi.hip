@@ -156,6 +156,29 @@ double tile_cost(int M, int N, int K, int count, int bm, int bn, int perCU, doub
     return (double)rounds * bm * bn * ((double)((K + splits - 1) / splits) + kFixed) / quality;
 }
 
+/* The same for fp32, in microseconds, fitted to measurements of both tile shapes with 1 to 8 pieces of k on two
+   dozen products (512^3 to 4096 x 2048 x 512, 640 x 512 x 30011): the fp32 matrix pipe of a SIMD is kept busy
+   by ONE wave, so what counts is how many workgroups the busiest CU runs one after the other (a second
+   workgroup on a CU hides latencies but takes its own turn on the pipe): rounds = ceil(workgroups / 256). A
+   workgroup's MFMAs take tile area x k x 3.48e-6 us on a 128 x 128 tile; the 64 x 64 tile (one accumulator
+   block per wave: a dependent chain) runs at 0.89 of that rate alone on its CU and at 0.965 with company. What
+   a workgroup spends before its first and after its last MFMA (4 us; 1.5 us for the small tile) is exposed
+   once and partly hidden behind the other workgroups of the CU after that. Cutting k moves c once more per piece
+   (atomic adds, about 2.7 TB/s); unless beta is 1, a pass over c applies beta first: a launch (2.5 us) and c
+   read and written. */
+double tile_cost_f32(int M, int N, int K, int count, int bm, int splits, bool betaPass)
+{
+    const bool big = bm >= 128;
+    const long long groups = (long long)((M + bm - 1) / bm) * ((N + bm - 1) / bm) * count * splits;
+    const long long rounds = (groups + 255) / 256;
+    const double rate = big ? 1.0 : (rounds > 1 ? 0.965 : 0.89);
+    const double mfma = (double)bm * bm * ((K + splits - 1) / splits) * 3.48e-6 / rate;
+    const double ends = (big ? 4.0 : 1.5) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
+    const double cBytes = 4.0 * M * N * count;
+    const double cut = splits > 1 ? cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0) : 0.0;
+    return (double)rounds * mfma + ends + cut;
+}
+
 struct Plan {
     int cfg;
     int splits;
@@ -164,11 +187,11 @@ struct Plan {
 /* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
    estimated run time. NTSAMD_TILE_CFG=0|1|2 forces a shape (128x128, 64x64, 256x256 for
    half) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
-Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit)
+Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass)
 {
     static const int bms[CFG_COUNT] = {128, 64, 256};
     static const int perCU[CFG_COUNT] = {2, 2, 1};
-    static const double q32[CFG_COUNT] = {1.0, 0.8, 0.0};
+    static const double q32[CFG_COUNT] = {1.0, 0.9, 0.0};       /* fp32: only > 0 matters, see tile_cost_f32 */
     static const double q16[CFG_COUNT] = {0.45, 0.2, 1.0};
     int forcedCfg = -1, forcedSplits = -1;
     const char * e = getenv("NTSAMD_TILE_CFG");
@@ -195,7 +218,8 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit)
                 break;
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
-            double c = tile_cost(M, N, K, count, bms[cfg], bms[cfg], perCU[cfg], q, splits);
+            double c = half ? tile_cost(M, N, K, count, bms[cfg], bms[cfg], perCU[cfg], q, splits)
+                            : tile_cost_f32(M, N, K, count, bms[cfg], splits, betaPass);
             if (bestCost < 0.0 || c < bestCost) {
                 bestCost = c;
                 best.cfg = cfg;
@@ -286,7 +310,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
     const Plan plan = choose_plan(s.M, s.N, s.K, count, half,
-                                  kind == KIND_F32 && vec && !ptrs && act == ACT_NONE && dense);
+                                  kind == KIND_F32 && vec && !ptrs && act == ACT_NONE && dense, beta != 1.f);
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;
