@@ -141,23 +141,8 @@ bool aligned16(const void * p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
-/* Relative run time of a product under a tile shape and a number of k pieces: rounds of
-   workgroups (256 CUs x the workgroups a CU holds at once) times the work of one workgroup
-   (tile area x its k range plus a fixed cost per workgroup, in units of k: fetching the first
-   slabs, storing the tile), divided by how fast the shape runs relative to the best one on a
-   product that fits it (measured: small tiles re-read operands from LDS more often per MFMA,
-   which costs fp16 far more than fp32). */
-double tile_cost(int M, int N, int K, int count, int bm, int bn, int perCU, double quality, int splits)
-{
-    long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
-    long long slots = 256LL * perCU;
-    long long rounds = (tiles + slots - 1) / slots;
-    double kFixed = splits > 1 ? 192.0 : 96.0;       /* atomics cost more than stores */
-    return (double)rounds * bm * bn * ((double)((K + splits - 1) / splits) + kFixed) / quality;
-}
-
-/* The same for fp32, in microseconds, fitted to measurements of both tile shapes with 1 to 8 pieces of k on two
-   dozen products (512^3 to 4096 x 2048 x 512, 640 x 512 x 30011): the fp32 matrix pipe of a SIMD is kept busy
+/* Estimated run time of an fp32 product under a tile shape and a number of k pieces, in microseconds, fitted to
+   graph-replayed measurements of both tile shapes with 1 to 8 pieces of k on two dozen products (512^3 to 4096 x 2048 x 512, 640 x 512 x 30011): the fp32 matrix pipe of a SIMD is kept busy
    by ONE wave, so what counts is how many workgroups the busiest CU runs one after the other (a second
    workgroup on a CU hides latencies but takes its own turn on the pipe): rounds = ceil(workgroups / 256). A
    workgroup's MFMAs take tile area x k x 3.48e-6 us on a 128 x 128 tile; the 64 x 64 tile (one accumulator
@@ -179,6 +164,28 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int splits, bool be
     return (double)rounds * mfma + ends + cut;
 }
 
+/* The same for fp16, fitted the same way (k is never cut). The 256 x 256 tile runs alone on its CU, so every round
+   pays its ends in full (11.7 us: four slabs to fetch before the first MFMA, 128 KB to store after the last);
+   the smaller tiles share a CU and hide most of theirs, but re-read their operands from LDS more often per MFMA:
+   per k, a round costs 0.0282 us (256 x 256), 0.0088 us (128 x 128; 0.011 us alone on its CU), 0.00364 us
+   (64 x 64). Short k and many rounds favour the 128 x 128 tile (4096 x 30016 x 512: 172 against 191 us), long k
+   the big one. The clock under fp16 MFMA load depends on how much of the chip is busy, which is why the same
+   tile is faster per k on a product that fills a fraction of the CUs. */
+double tile_cost_f16(int M, int N, int K, int count, int bm)
+{
+    const long long groups = (long long)((M + bm - 1) / bm) * ((N + bm - 1) / bm) * count;
+    const long long rounds = (groups + 255) / 256;
+    /* fewer workgroups than CUs: every workgroup is alone on its CU (slower per k for the small tiles, whose
+       ends nobody hides), and the part runs at a higher clock the fewer CUs are busy (down to 0.7 of the time) */
+    const bool alone = groups <= 256;
+    const double busy = alone ? (groups < 180 ? 0.7 : (double)groups / 256.0) : 1.0;
+    if (bm >= 256)
+        return (double)rounds * (0.02816 * busy * K + 11.7);
+    if (bm >= 128)
+        return (double)rounds * ((alone ? 0.011 : 0.0088) * busy * K + 1.3) + 1.5;
+    return (double)rounds * ((alone ? 0.0051 : 0.00364) * busy * K + 0.2) + 1.9;
+}
+
 struct Plan {
     int cfg;
     int splits;
@@ -190,9 +197,6 @@ struct Plan {
 Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass)
 {
     static const int bms[CFG_COUNT] = {128, 64, 256};
-    static const int perCU[CFG_COUNT] = {2, 2, 1};
-    static const double q32[CFG_COUNT] = {1.0, 0.9, 0.0};       /* fp32: only > 0 matters, see tile_cost_f32 */
-    static const double q16[CFG_COUNT] = {0.45, 0.2, 1.0};
     int forcedCfg = -1, forcedSplits = -1;
     const char * e = getenv("NTSAMD_TILE_CFG");
     if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
@@ -210,15 +214,14 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
     Plan best = {CFG_64x64, 1};
     double bestCost = -1.0;
     for (int cfg = 0; cfg < CFG_COUNT; cfg++) {
-        const double q = half ? q16[cfg] : q32[cfg];
-        if (q <= 0.0 || (forcedCfg >= 0 && cfg != forcedCfg))
+        if ((cfg == CFG_256x256 && !half) || (forcedCfg >= 0 && cfg != forcedCfg))
             continue;
         for (int splits = 1; splits <= 16; splits *= 2) {
             if (splits > 1 && (!maySplit || K / splits < 256))
                 break;
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
-            double c = half ? tile_cost(M, N, K, count, bms[cfg], bms[cfg], perCU[cfg], q, splits)
+            double c = half ? tile_cost_f16(M, N, K, count, bms[cfg])
                             : tile_cost_f32(M, N, K, count, bms[cfg], splits, betaPass);
             if (bestCost < 0.0 || c < bestCost) {
                 bestCost = c;
