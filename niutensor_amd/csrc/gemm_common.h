@@ -118,7 +118,7 @@ __device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
 }
 
 /* tile shapes the dispatcher can pick from */
-enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_256x256 = 2, CFG_COUNT = 3 };
+enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_256x256 = 2, CFG_32x128 = 3, CFG_COUNT = 4 };
 
 /* BM x BN tile per workgroup of WGM x WGN waves; BKT32: slab depth of the fp32 kernel
    (small tiles serve small, latency-bound products: a deeper slab means fewer round trips
@@ -127,6 +127,8 @@ enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_256x256 = 2, CFG_COUNT = 3 };
 template <int CFG> struct TileShape;
 template <> struct TileShape<CFG_128x128> { static constexpr int BM = 128, BN = 128, WGM = 2, WGN = 2, MINW16 = 2, BKT32 = 16; };
 template <> struct TileShape<CFG_64x64> { static constexpr int BM = 64, BN = 64, WGM = 2, WGN = 2, MINW16 = 2, BKT32 = 32; };
+/* fp32 only, for products with at most 32 rows (a decoding step): no rows of padding to multiply */
+template <> struct TileShape<CFG_32x128> { static constexpr int BM = 32, BN = 128, WGM = 1, WGN = 4, MINW16 = 2, BKT32 = 32; };
 template <> struct TileShape<CFG_256x256> { static constexpr int BM = 256, BN = 256, WGM = 2, WGN = 2, MINW16 = 1, BKT32 = 16; };
 
 int launch_f32(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,

@@ -579,6 +579,8 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
     }
     if (cfg == CFG_128x128)
         return launch_f32_one<CFG_128x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
+    if (cfg == CFG_32x128)
+        return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
     return launch_f32_one<CFG_64x64, AKC, BKC, true, false, NoPtrs>(p, none, stream);
 }
 

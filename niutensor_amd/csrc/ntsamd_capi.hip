@@ -151,13 +151,13 @@ bool aligned16(const void * p)
    once and partly hidden behind the other workgroups of the CU after that. Cutting k moves c once more per piece
    (atomic adds, about 2.7 TB/s); unless beta is 1, a pass over c applies beta first: a launch (2.5 us) and c
    read and written. */
-double tile_cost_f32(int M, int N, int K, int count, int bm, int splits, bool betaPass)
+double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits, bool betaPass)
 {
     const bool big = bm >= 128;
-    const long long groups = (long long)((M + bm - 1) / bm) * ((N + bm - 1) / bm) * count * splits;
+    const long long groups = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
     const long long rounds = (groups + 255) / 256;
     const double rate = big ? 1.0 : (rounds > 1 ? 0.965 : 0.89);
-    const double mfma = (double)bm * bm * ((K + splits - 1) / splits) * 3.48e-6 / rate;
+    const double mfma = (double)bm * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
     const double ends = (big ? 4.0 : 1.5) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
     const double cBytes = 4.0 * M * N * count;
     const double cut = splits > 1 ? cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0) : 0.0;
@@ -192,17 +192,20 @@ struct Plan {
 };
 
 /* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
-   estimated run time. NTSAMD_TILE_CFG=0|1|2 forces a shape (128x128, 64x64, 256x256 for
-   half) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
+   estimated run time. NTSAMD_TILE_CFG=0|1|2|3 forces a shape (128x128, 64x64, 256x256 for
+   half, 32x128 for float) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
 Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass)
 {
-    static const int bms[CFG_COUNT] = {128, 64, 256};
+    static const int bms[CFG_COUNT] = {128, 64, 256, 32};
+    static const int bns[CFG_COUNT] = {128, 64, 256, 128};
     int forcedCfg = -1, forcedSplits = -1;
     const char * e = getenv("NTSAMD_TILE_CFG");
     if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
         forcedCfg = e[0] - '0';
         if (forcedCfg == CFG_256x256 && !half)
             forcedCfg = CFG_128x128;
+        if (forcedCfg == CFG_32x128 && half)
+            forcedCfg = CFG_64x64;
     }
     e = getenv("NTSAMD_SPLIT_K");
     if (e && atoi(e) >= 1)
@@ -214,7 +217,7 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
     Plan best = {CFG_64x64, 1};
     double bestCost = -1.0;
     for (int cfg = 0; cfg < CFG_COUNT; cfg++) {
-        if ((cfg == CFG_256x256 && !half) || (forcedCfg >= 0 && cfg != forcedCfg))
+        if ((cfg == CFG_256x256 && !half) || (cfg == CFG_32x128 && (half || M > 32)) || (forcedCfg >= 0 && cfg != forcedCfg))
             continue;
         for (int splits = 1; splits <= 16; splits *= 2) {
             if (splits > 1 && (!maySplit || K / splits < 128))
@@ -222,7 +225,7 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
             double c = half ? tile_cost_f16(M, N, K, count, bms[cfg])
-                            : tile_cost_f32(M, N, K, count, bms[cfg], splits, betaPass);
+                            : tile_cost_f32(M, N, K, count, bms[cfg], bns[cfg], splits, betaPass);
             if (bestCost < 0.0 || c < bestCost) {
                 bestCost = c;
                 best.cfg = cfg;

@@ -153,13 +153,14 @@ def test_compiled_reference_fixture(gpu, generated):
 # ---- seeded inputs against the oracle ------------------------------------------
 
 SHAPES = [(1, 1, 1), (5, 7, 3), (37, 29, 53), (64, 64, 16), (63, 65, 17), (127, 129, 31), (128, 128, 64),
-          (130, 70, 33), (200, 24, 100), (256, 384, 128), (300, 260, 101), (1, 300, 40), (300, 1, 40), (96, 96, 1)]
+          (130, 70, 33), (200, 24, 100), (256, 384, 128), (300, 260, 101), (1, 300, 40), (300, 1, 40), (96, 96, 1),
+          (32, 300, 70), (17, 515, 129)]
 
 
 @pytest.mark.parametrize("ta,tb", TRANS)
 def test_fp32_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
-    for cfg in ("0", "1"):
+    for cfg in ("0", "1", "3"):                          # 128 x 128, 64 x 64, 32 x 128 (at most 32 rows; else the rule's choice)
         os.environ["NTSAMD_TILE_CFG"] = cfg
         for i, (M, N, K) in enumerate(SHAPES):
             a = oracle.uniform(stored((M, K), ta), 1000 + i)
