@@ -261,6 +261,12 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     if (scope.status != NTSAMD_OK)
         return scope.status;
 
+    /* the kernels number their workgroups with 32-bit integers: the finest tiling of the largest batch,
+       with k cut into the most pieces, must fit */
+    if ((long long)((s.M + 31) / 32) * ((s.N + 63) / 64) * count * 16 > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "the product has too many tiles for one launch (%d x %d x %d matrices)",
+                    s.M, s.N, count);
+
     GemmParams p;
     memset(&p, 0, sizeof(p));
     p.a = a;

@@ -648,3 +648,13 @@ def test_config5_ragged_vocab_projection(gpu, oracle):
     nt.matrix_mul(gh, X_NOTRANS, gw, X_TRANS, c, 1.0, 1.0)
     want2 = 2 * sampled_f64(h, X_NOTRANS, w, X_TRANS, rows) + c0[rows]
     assert_fp32(c.cpu().numpy()[rows], want2, 512)
+
+
+def test_a_batch_with_too_many_tiles_is_refused(gpu):
+    """Workgroups are numbered with 32-bit integers: a batch that would not fit is an argument error, found
+    before anything is launched (the strides below lie about the size of the tensors; nothing reads them)."""
+    torch = torch_()
+    t = torch.zeros(1024, device=gpu)
+    with pytest.raises(nt.NtsAmdError, match="too many tiles"):
+        nt.matrix_mul_batched_strided(t, X_NOTRANS, t, X_NOTRANS, t, 1 << 27, 0, 0, 1024, 32, 32, 32, 32, 32, 32)
+
