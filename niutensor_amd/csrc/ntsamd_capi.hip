@@ -165,7 +165,8 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
 }
 
 /* The same for fp16, fitted the same way (k is never cut). The 256 x 256 tile runs alone on its CU, so every round
-   pays its ends in full (11.7 us: four slabs to fetch before the first MFMA, 128 KB to store after the last);
+   pays its ends in full (11.7 us: four slabs to fetch before the first MFMA, 128 KB to store after the last;
+   8.5 us on eight waves, which is how it runs up to k = 2048);
    the smaller tiles share a CU and hide most of theirs, but re-read their operands from LDS more often per MFMA:
    per k, a round costs 0.0282 us (256 x 256), 0.0088 us (128 x 128; 0.011 us alone on its CU), 0.00364 us
    (64 x 64). Short k and many rounds favour the 128 x 128 tile (4096 x 30016 x 512: 172 against 191 us), long k
@@ -180,7 +181,7 @@ double tile_cost_f16(int M, int N, int K, int count, int bm)
     const bool alone = groups <= 256;
     const double busy = alone ? (groups < 180 ? 0.7 : (double)groups / 256.0) : 1.0;
     if (bm >= 256)
-        return (double)rounds * (0.02816 * busy * K + 11.7);
+        return (double)rounds * (K <= 2048 ? 0.0275 * busy * K + 8.5 : 0.02816 * busy * K + 11.7);   /* eight waves / four */
     if (bm >= 128)
         return (double)rounds * ((alone ? 0.011 : 0.0088) * busy * K + 1.3) + 1.5;
     return (double)rounds * ((alone ? 0.0051 : 0.00364) * busy * K + 0.2) + 1.9;

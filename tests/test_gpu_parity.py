@@ -177,9 +177,10 @@ def test_fp32_against_oracle(gpu, oracle, ta, tb):
 @pytest.mark.parametrize("ta,tb", TRANS)
 def test_fp16_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
-    for cfg in ("0", "1"):
+    # 128 x 128, 64 x 64, 256 x 256 (eight waves up to k = 2048, four beyond: the last shape)
+    for cfg in ("0", "1", "2"):
         os.environ["NTSAMD_TILE_CFG"] = cfg
-        for i, (M, N, K) in enumerate(SHAPES):
+        for i, (M, N, K) in enumerate(SHAPES + [(264, 520, 2304)]):
             # round the inputs to half first; the oracle then runs in fp32 on those values
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 4000 + i, 0, 0.5)))
             b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 5000 + i, 0, 0.5)))
