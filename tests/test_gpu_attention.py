@@ -251,3 +251,29 @@ def test_bad_arguments_are_refused(gpu):
     assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 0, 1, 8, 8, 8, st, 1.0) == 0           # nothing to do
     bad = (C.c_longlong * 12)(*([8, 64, 6] * 4))
     assert L.ntsamd_attention(0, None, p, p, p, None, p, 2, 1, 1, 8, 8, 8, bad, 1.0) != 0          # unaligned rows
+
+
+def test_probabilities_at_the_benchmark_shape(gpu, oracle):
+    """32 sentences x 8 heads, 128 x 128 scores per head: every row sums to 1, the probabilities times v equal
+    the one-kernel attention (two independent kernels for the same chain), and one head against the oracle."""
+    torch = torch_()
+    B, L, H, nh = 32, 128, 512, 8
+    q, k, v = oracle.normal((B, L, H), 91), oracle.normal((B, L, H), 92), oracle.normal((B, L, H), 93)
+    qd, kd, vd = dev(q, gpu), dev(k, gpu), dev(v, gpu)
+    probs = torch.full((nh, B, L, L), float("nan"), device=gpu)
+    nt.attention_probs(qd, kd, probs, nh, 0.125)
+    torch.cuda.synchronize()
+    p = probs.cpu().numpy()
+    assert np.isfinite(p).all() and (p >= 0).all()
+    assert np.abs(p.sum(-1) - 1.0).max() <= 1e-5
+    out = torch.empty((B, L, H), device=gpu)
+    nt.attention(qd, kd, vd, out, nh, 0.125)
+    ctx = torch.empty((B, L, H), device=gpu)
+    dh = H // nh
+    nt.matrix_mul_batched_grid(probs, nt.X_NOTRANS, L, (L * L, B * L * L), vd, nt.X_NOTRANS, H, (L * H, dh),
+                               ctx, H, (L * H, dh), B, nh, L, L, L, dh, L, dh)
+    torch.cuda.synchronize()
+    assert_fp32(ctx.cpu().numpy(), out.cpu().numpy(), dh + L, what="probabilities x v against the one kernel")
+    ref = oracle.attention_probs(q[3:4], k[3:4], nh, 0.125)
+    assert_fp32(p[:, 3:4], ref, dh, what="sentence 3")
+

@@ -192,3 +192,28 @@ def test_argument_errors(gpu):
     # nothing to do is no error
     nt.matrix_mul_batched_grid(t, X_NOTRANS, 8, (64, 0), t, X_NOTRANS, 8, (64, 0), t, 8, (64, 128),
                                0, 2, 8, 8, 8, 8, 8, 8)
+
+
+def test_benchmark_shape_against_split_product_merge(gpu, oracle):
+    """32 sentences x 8 heads at full size: the product on merged tensors equals, bit for bit, the same kernels
+    run on tensors that were split and merged by copies (same tiles, same order of accumulation: only the
+    addressing differs), and one head of one sentence against the oracle."""
+    torch = torch_()
+    B, nh, L, dh = 32, 8, 128, 64
+    H = nh * dh
+    probs = dev(oracle.uniform((nh, B, L, L), 81, 0.0, 1.0), gpu)
+    probs /= probs.sum(-1, keepdim=True)
+    v = dev(oracle.normal((B, L, H), 82), gpu)
+    out = torch.full((B, L, H), float("nan"), device=gpu)
+    nt.matrix_mul_batched_grid(probs, X_NOTRANS, L, (L * L, B * L * L), v, X_NOTRANS, H, (L * H, dh),
+                               out, H, (L * H, dh), B, nh, L, L, L, dh, L, dh)
+    vs = v.view(B, L, nh, dh).permute(2, 0, 1, 3).contiguous()
+    os_ = torch.empty((nh, B, L, dh), device=gpu)
+    nt.matrix_mul_batched_strided(probs, X_NOTRANS, vs, X_NOTRANS, os_, nh * B, L * L, L * dh, L * dh,
+                                  L, L, L, dh, L, dh)
+    torch.cuda.synchronize()
+    assert torch.equal(out, os_.permute(1, 2, 0, 3).reshape(B, L, H))
+    b, h = 17, 5
+    ref = oracle.matmul2d(probs[h, b].cpu().numpy(), X_NOTRANS,
+                          np.ascontiguousarray(v[b, :, h * dh:(h + 1) * dh].cpu().numpy()), X_NOTRANS)
+    assert_fp32(out[b, :, h * dh:(h + 1) * dh].cpu().numpy(), ref, L, what="sentence 17, head 5")

@@ -659,3 +659,19 @@ def test_a_batch_with_too_many_tiles_is_refused(gpu):
     with pytest.raises(nt.NtsAmdError, match="too many tiles"):
         nt.matrix_mul_batched_strided(t, X_NOTRANS, t, X_NOTRANS, t, 1 << 27, 0, 0, 1024, 32, 32, 32, 32, 32, 32)
 
+
+def test_rectified_linear_layer_at_full_size(gpu, oracle):
+    """Configuration 2's layer with the activation in the epilogue: bit for bit the maximum of zero and the
+    layer without it (the activation is applied to the same fp32 value the plain epilogue stores)."""
+    torch = torch_()
+    x = dev_tensor(oracle.uniform((4096, 512), 1), gpu)
+    w = dev_tensor(oracle.normal((512, 2048), 2, 0, 0.02), gpu)
+    b = dev_tensor(oracle.normal((2048,), 3, 0, 0.02), gpu)
+    plain = torch.empty((4096, 2048), device=gpu)
+    rect = torch.full((4096, 2048), float("nan"), device=gpu)
+    nt.matrix_mul(x, X_NOTRANS, w, X_NOTRANS, plain, bias=b)
+    nt.matrix_mul(x, X_NOTRANS, w, X_NOTRANS, rect, bias=b, act=nt.ACT_RECTIFY)
+    torch.cuda.synchronize()
+    assert torch.equal(rect, torch.clamp_min(plain, 0.0))
+    assert 0.3 < (rect == 0).float().mean().item() < 0.7
+
