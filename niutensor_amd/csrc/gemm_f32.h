@@ -33,6 +33,8 @@
  */
 #pragma once
 #include "gemm_common.h"
+#include <stdlib.h>
+#include <type_traits>
 
 namespace ntsamd {
 
@@ -59,14 +61,23 @@ __device__ __forceinline__ f32x4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t rsrc, 
     return __builtin_bit_cast(f32x4, v);
 }
 
-template <int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, bool CS, typename PT>
+/* R16 (products with at most 16 rows, on the 32 x 128 tile): a wave multiplies only the first 16 rows of the
+   tile, as two 16 x 16 blocks of v_mfma_f32_16x16x4_f32 side by side (lane l feeds row/column l % 16 at k slot
+   l / 16; step t of a group of 16 k takes k = 4 * (l / 16) + t, so a K-contiguous operand is still one 16-byte
+   read per group): half the MFMA work of 32 padded rows, and a chain of dependent MFMAs half as long. */
+template <int BM, int BN, int BKT, int WGM, int WGN, bool AKC, bool BKC, bool VEC, bool CS, typename PT, bool R16 = false>
 __global__ void __launch_bounds__(WGM * WGN * 64, 2)
 gemm_f32_kernel(const GemmParams p, const PT tab)
 {
+    static_assert(!R16 || (BM == 32 && WGM == 1 && VEC && !CS), "16-row MFMAs: one row of waves on a 32-row tile");
     constexpr int NT = WGM * WGN * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
-    constexpr int TI = WM / 32, TJ = WN / 32;
-    constexpr int KK = BKT / 2;           /* MFMA steps per slab */
+    constexpr int BS = R16 ? 16 : 32;                      /* rows and columns of an accumulator block */
+    constexpr int TI = R16 ? 1 : WM / 32, TJ = WN / BS;
+    constexpr int KPM = R16 ? 4 : 2;                       /* k per MFMA */
+    constexpr int KG = 4 * KPM;                            /* k per group of four MFMA steps */
+    constexpr int ACCN = R16 ? 4 : 16;                     /* accumulator registers per block */
+    constexpr int KK = BKT / KPM;         /* MFMA steps per slab */
     constexpr int LDK = BKT + 4;          /* row pitch of a K-contiguous operand in LDS */
     constexpr int NA = BM * BKT / 4 / NT;
     constexpr int NB = BN * BKT / 4 / NT;
@@ -99,7 +110,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
-    const int l32 = lane & 31, lh = lane >> 5;
+    const int l32 = R16 ? (lane & 15) : (lane & 31);      /* row / column inside a block */
+    const int lh = R16 ? (lane >> 4) : (lane >> 5);        /* k slot */
 
     /* ---- staging slots: which 4 elements of the slab each thread moves ------ */
     int aOff[NA], bOff[NB];        /* 16-byte path: byte offset from the slab base */
@@ -274,7 +286,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int q = 0; q < KK / 4; q++)
 #pragma unroll
                 for (int i = 0; i < TI; i++)
-                    fa4[set][q][i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * LDK + 8 * q);
+                    fa4[set][q][i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * LDK + KG * q);
         }
         else {
             const float * as = &As[buf][4 * lh * BM + wm0 + l32];
@@ -282,7 +294,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int t = 0; t < KK; t++)
 #pragma unroll
                 for (int i = 0; i < TI; i++)
-                    fa1[set][t][i] = as[(8 * (t / 4) + (t % 4)) * BM + i * 32];
+                    fa1[set][t][i] = as[(KG * (t / 4) + (t % 4)) * BM + i * 32];
         }
         if constexpr (BKC) {
             const float * bs = &Bs[buf][(wn0 + l32) * LDK + 4 * lh];
@@ -290,7 +302,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int q = 0; q < KK / 4; q++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
-                    fb4[set][q][j] = *reinterpret_cast<const f32x4 *>(bs + j * 32 * LDK + 8 * q);
+                    fb4[set][q][j] = *reinterpret_cast<const f32x4 *>(bs + j * BS * LDK + KG * q);
         }
         else {
             const float * bs = &Bs[buf][4 * lh * BN + wn0 + l32];
@@ -298,17 +310,18 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             for (int t = 0; t < KK; t++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
-                    fb1[set][t][j] = bs[(8 * (t / 4) + (t % 4)) * BN + j * 32];
+                    fb1[set][t][j] = bs[(KG * (t / 4) + (t % 4)) * BN + j * BS];
         }
     };
 
-    f32x16 acc[TI][TJ];
+    typedef typename std::conditional<R16, f32x4, f32x16>::type Acc;
+    Acc acc[TI][TJ];
 #pragma unroll
     for (int i = 0; i < TI; i++)
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++)
+            for (int r = 0; r < ACCN; r++)
                 acc[i][j][r] = 0.f;
 
     /* CS: every lane also adds up the op(b) values that pass through its fragments: lane
@@ -329,7 +342,10 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                 for (int j = 0; j < TJ; j++) {
                     float av = AKC ? fa4[set][t / 4][i][t % 4] : fa1[set][t][i];
                     float bv = BKC ? fb4[set][t / 4][j][t % 4] : fb1[set][t][j];
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                    if constexpr (R16)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[i][j], 0, 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
                     if constexpr (CS)
                         if (i == 0)
                             colSum[j] += bv;
@@ -408,7 +424,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 
     /* ---- epilogue: accumulator register r of lane l is element
        (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block, so a store covers
-       two rows of 32 consecutive floats and needs no alignment of ldc ---------- */
+       two rows of 32 consecutive floats and needs no alignment of ldc
+       (16x16 blocks: element (4*(l/16) + r, l%16), four rows of 16 floats) ---------- */
     const float alpha = p.alpha, beta = p.beta;
     const float * __restrict__ bias = static_cast<const float *>(p.bias);
     const int biasMode = p.biasMode;
@@ -427,7 +444,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         float bcol[TJ];
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const int col = n0 + wn0 + j * 32 + l32;
+            const int col = n0 + wn0 + j * BS + l32;
             cOff[j] = col < N ? (unsigned)(4 * lh * p.ldc + col) * 4u : (unsigned)NTSAMD_OOB_OFFSET;
             bcol[j] = biasMode == BIAS_COL && col < N ? bias[col] : 0.f;
         }
@@ -438,7 +455,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 #pragma unroll
                 for (int j = 0; j < TJ; j++) {
                     const float v = colSum[j] + __shfl_xor(colSum[j], 32);
-                    const int col = n0 + wn0 + j * 32 + l32;
+                    const int col = n0 + wn0 + j * BS + l32;
                     if (lh == 0 && col < N) {
                         if (p.splits > 1)
                             unsafeAtomicAdd(cs + col, v);      /* the caller has applied colSumBeta */
@@ -456,14 +473,14 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                does not rely on the same for atomics and uses plain global atomics). */
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
-                const int col = n0 + wn0 + j * 32 + l32;
+                const int col = n0 + wn0 + j * BS + l32;
                 if (col < N) {
                     const float bj = tc.split == 0 ? bcol[j] : 0.f;
 #pragma unroll
                     for (int i = 0; i < TI; i++)
 #pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                        for (int r = 0; r < ACCN; r++) {
+                            const int row = m0 + wm0 + i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4)) + 4 * lh;
                             if (row < M)
                                 unsafeAtomicAdd(C + (size_t)row * p.ldc + col, alpha * acc[i][j][r] + bj);
                         }
@@ -474,14 +491,14 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         /* beta is tested once, outside the loops: inside them the test would fence every
            load of c off in a block of its own, one memory round trip after the other */
         if (beta != 0.f) {
-            float old[TI][TJ][16];
+            float old[TI][TJ][ACCN];
 #pragma unroll
             for (int i = 0; i < TI; i++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    for (int r = 0; r < ACCN; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
                         old[i][j][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
                     }
 #pragma unroll
@@ -489,8 +506,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    for (int r = 0; r < ACCN; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
                         const float v = activate(alpha * acc[i][j][r] + bcol[j] + beta * old[i][j][r], act);
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
                     }
@@ -501,8 +518,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + 8 * (r / 4) + (r % 4)) * rowPitch;
+                    for (int r = 0; r < ACCN; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
                         const float v = activate(alpha * acc[i][j][r] + bcol[j], act);
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
                     }
@@ -512,7 +529,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
         /* generic path: plain pointers, per-element bounds, every bias mode */
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
-            const int col = n0 + wn0 + j * 32 + l32;
+            const int col = n0 + wn0 + j * BS + l32;
             if (col >= N)
                 continue;
             float bcol = 0.f;
@@ -523,8 +540,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                 const int rowBase = m0 + wm0 + i * 32 + 4 * lh;
                 float * cb = C + (size_t)rowBase * p.ldc + col;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int dr = 8 * (r / 4) + (r % 4);
+                for (int r = 0; r < ACCN; r++) {
+                    const int dr = R16 ? r : 8 * (r / 4) + (r % 4);
                     if (rowBase + dr < M) {
                         float * cp = cb + (size_t)dr * p.ldc;
                         float v = alpha * acc[i][j][r];
@@ -542,7 +559,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     }
 }
 
-template <int CFG, bool AKC, bool BKC, bool VEC, bool CS, typename PT>
+template <int CFG, bool AKC, bool BKC, bool VEC, bool CS, typename PT, bool R16 = false>
 static int launch_f32_one(const GemmParams & p0, const PT & tab, hipStream_t stream)
 {
     typedef TileShape<CFG> S;
@@ -552,7 +569,7 @@ static int launch_f32_one(const GemmParams & p0, const PT & tab, hipStream_t str
     if (p.splits < 1 || !VEC)
         p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
-    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, S::BKT32, S::WGM, S::WGN, AKC, BKC, VEC, CS, PT>),
+    hipLaunchKernelGGL((gemm_f32_kernel<S::BM, S::BN, S::BKT32, S::WGM, S::WGN, AKC, BKC, VEC, CS, PT, R16>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();
 }
@@ -579,8 +596,13 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
     }
     if (cfg == CFG_128x128)
         return launch_f32_one<CFG_128x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
-    if (cfg == CFG_32x128)
+    if (cfg == CFG_32x128) {
+        /* at most 16 rows: 16-row MFMAs on the same tile (NTSAMD_F32_R16=0 keeps the 32-row ones: for measurements) */
+        const char * e = getenv("NTSAMD_F32_R16");
+        if (p.M <= 16 && !(e && e[0] == '0'))
+            return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs, true>(p, none, stream);
         return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
+    }
     return launch_f32_one<CFG_64x64, AKC, BKC, true, false, NoPtrs>(p, none, stream);
 }
 
