@@ -157,7 +157,8 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
     const long long rounds = (groups + 255) / 256;
     const double rate = big ? 1.0 : (rounds > 1 ? 0.965 : 0.89);
-    const double mfma = (double)bm * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
+    /* the 32-row tile multiplies only 16 rows when there are no more (16-row MFMAs) */
+    const double mfma = (double)(bm == 32 && M <= 16 ? 16 : bm) * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
     const double ends = (big ? 4.0 : 1.5) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
     const double cBytes = 4.0 * M * N * count;
     const double cut = splits > 1 ? cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0) : 0.0;
