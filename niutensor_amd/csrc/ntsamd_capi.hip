@@ -214,7 +214,7 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
         forcedSplits = atoi(e);
     if (forcedSplits != 1 && forcedSplits != 2 && forcedSplits != 4 && forcedSplits != 8 && forcedSplits != 16)
         forcedSplits = -1;
-    if (forcedSplits > 1 && (!maySplit || K / forcedSplits < 128))
+    if (forcedSplits > 1 && (!maySplit || K / forcedSplits < 64))
         forcedSplits = 1;
     Plan best = {CFG_64x64, 1};
     double bestCost = -1.0;
@@ -222,7 +222,7 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
         if ((cfg == CFG_256x256 && !half) || (cfg == CFG_32x128 && (half || M > 32)) || (forcedCfg >= 0 && cfg != forcedCfg))
             continue;
         for (int splits = 1; splits <= 16; splits *= 2) {
-            if (splits > 1 && (!maySplit || K / splits < 128))
+            if (splits > 1 && (!maySplit || K / splits < 64))
                 break;
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
