@@ -26,6 +26,10 @@ struct AttnParams {
 
 int launch_attention_f32(const AttnParams & p, hipStream_t stream);
 int launch_attention_f16(const AttnParams & p, hipStream_t stream);
+/* a handful of query rows per head (a decoding step): every key and value read once, no MFMA tiles of padding.
+   attention_rows_lds: the LDS that kernel would need for the problem, 0 if it does not take it */
+size_t attention_rows_lds(const AttnParams & p, bool half);
+int launch_attention_rows(const AttnParams & p, bool half, hipStream_t stream);
 /* probabilities only: out is the dense [heads][batch][lq][lk] tensor, v is not used */
 int launch_attention_probs_f32(const AttnParams & p, hipStream_t stream);
 

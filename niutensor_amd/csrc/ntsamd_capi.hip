@@ -622,8 +622,17 @@ int ntsamd_attention(int devID, void * stream,
     p.vH = strides[6]; p.vB = strides[7]; p.vL = strides[8];
     p.oH = strides[9]; p.oB = strides[10]; p.oL = strides[11];
     p.scale = scale;
-    int rc = dataType == NTSAMD_X_FLOAT ? launch_attention_f32(p, static_cast<hipStream_t>(stream))
-                                        : launch_attention_f16(p, static_cast<hipStream_t>(stream));
+    /* up to eight query rows per head (a decoding step) go to the kernel that reads k and v once and multiplies
+       in the vector ALU, as long as its scores fit in LDS; NTSAMD_ATTN_ROWS=0 keeps them on the MFMA kernels */
+    const bool halfType = dataType == NTSAMD_X_FLOAT16;
+    const size_t rowsLds = attention_rows_lds(p, halfType);
+    const char * env = getenv("NTSAMD_ATTN_ROWS");
+    int rc;
+    if (rowsLds > 0 && rowsLds <= 60 * 1024 && !(env && env[0] == '0'))
+        rc = launch_attention_rows(p, halfType, static_cast<hipStream_t>(stream));
+    else
+        rc = halfType ? launch_attention_f16(p, static_cast<hipStream_t>(stream))
+                      : launch_attention_f32(p, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

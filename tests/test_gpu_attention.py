@@ -277,3 +277,31 @@ def test_probabilities_at_the_benchmark_shape(gpu, oracle):
     ref = oracle.attention_probs(q[3:4], k[3:4], nh, 0.125)
     assert_fp32(p[:, 3:4], ref, dh, what="sentence 3")
 
+
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
+    (16, 1, 100, 512, 8, False),       # one new position against 100 cached ones
+    (5, 1, 1, 64, 2, False),           # the first step: one key
+    (3, 8, 77, 96, 3, True),           # eight rows (the most this kernel takes), ragged keys, masked
+    (2, 4, 700, 256, 2, True),         # head size 128, more keys than lanes
+    (7, 3, 33, 24, 2, False),          # head size 12: lanes without columns
+])
+def test_a_handful_of_query_rows(gpu, oracle, B, lq, lk, H, nh, masked):
+    """Up to eight query rows per head (a decoding step) run on the kernel that reads k and v once and
+    multiplies in the vector ALU; the same inputs through the MFMA kernel (NTSAMD_ATTN_ROWS=0) must meet
+    the same limit against the oracle."""
+    import os
+    q, k, v = oracle.normal((B, lq, H), 61), oracle.normal((B, lk, H), 62), oracle.normal((B, lk, H), 63)
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 64, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., 0] = 0.0
+    scale = 1.0 / np.sqrt(H // nh)
+    ref = oracle.attention(q, k, v, nh, scale, mask)
+    for rows in ("1", "0"):
+        os.environ["NTSAMD_ATTN_ROWS"] = rows
+        try:
+            got = run(gpu, q, k, v, nh, scale, mask)
+        finally:
+            os.environ.pop("NTSAMD_ATTN_ROWS", None)
+        assert_fp32(got, ref, H // nh + lk, what="rows kernel" if rows == "1" else "MFMA kernel")
+
