@@ -27,10 +27,17 @@
  * Every function returns 0 on success and a non-zero code on failure; the
  * message of the last failure on the calling thread is available from
  * ntsamd_last_error(). Nothing is thrown across this boundary. The library
- * keeps no mutable global state, allocates no device memory, restores the
- * caller's current device before returning, and issues its work on `stream`
- * (NULL = the default stream, which is what the reference uses) without
- * synchronising.
+ * restores the caller's current device before returning and issues its work
+ * on `stream` (NULL = the default stream, which is what the reference uses)
+ * without synchronising. Its only state beyond a per-device flag, and the only
+ * device memory it allocates, is a 32 MiB workspace per device and stream for
+ * half products with few tiles and a long k, which are cut along k (partial
+ * products in fp32, added up by a second kernel): allocated at the first such
+ * product on that stream, kept until the process ends. Launches on one stream
+ * share it; kernels recorded into a graph keep the workspace of the stream
+ * they were captured on, so graphs captured on one stream and that stream's
+ * own launches must not run concurrently. NTSAMD_SPLIT_K=1 in the environment
+ * keeps every product in one piece and the library from allocating.
  */
 #ifndef NTSAMD_GEMM_H
 #define NTSAMD_GEMM_H

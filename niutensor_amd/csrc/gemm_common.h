@@ -66,10 +66,13 @@ struct GemmParams {
        (NULL = none); written by the workgroups of the first tile row */
     void * colSum;
     float colSumBeta;
-    /* fp32 only: the k range is cut into `splits` pieces of kPerSplit (a multiple of every slab
-       depth), one workgroup each, which ADD alpha * (their partial product) to c with atomics;
-       the caller has already applied beta to c. 1 = one workgroup per tile, plain stores. */
+    /* The k range is cut into `splits` pieces of kPerSplit (a multiple of every slab depth), one workgroup
+       each; 1 = one workgroup per tile, plain stores. fp32: the pieces ADD alpha * (their partial product) to
+       c with atomics, the caller has already applied beta to c. fp16 (16-byte path, 64 x 64 and 128 x 128
+       tiles): the pieces go to splitWork (splits x batch dense M x N fp32 matrices) as plain products, and
+       launch_split_reduce adds them up and writes c. */
     int splits, kPerSplit;
+    float * splitWork;
     int act;                               /* Activation of the epilogue */
 };
 
@@ -139,5 +142,7 @@ int launch_f32(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool 
 enum F16Fetch { F16_SCALAR = 0, F16_DIRECT = 1, F16_STAGED = 2 };
 int launch_f16(const GemmParams & p, const PtrBatch * ptrs, bool aKContig, bool bKContig,
                int vec, bool outF32, int cfg, hipStream_t stream);
+/* c = f(alpha * (sum of the p.splits partial products in p.splitWork) + bias + beta * c) */
+int launch_split_reduce(const GemmParams & p, bool outF32, hipStream_t stream);
 
 }  // namespace ntsamd

@@ -76,11 +76,16 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
                  : "memory");
 }
 
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS>
+/* SPLIT: the k range is cut into p.splits pieces, one workgroup each, and every workgroup leaves its partial tile
+   as plain fp32 (no alpha, beta, bias or activation) in p.splitWork, which holds p.splits x p.batch dense M x N
+   matrices; split_reduce.hip adds the pieces up and does what the epilogue would have done. */
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
     static_assert(!CS || std::is_same<OutT, half_t>::value, "column sums have the type of b and of c");
+    static_assert(!(CS && SPLIT), "column sums are not gathered from pieces of k");
+    static_assert(!SPLIT || std::is_same<OutT, float>::value, "partial tiles are fp32");
     constexpr int BKT = 32, KS = 2, NSTAGE = 4;
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -106,9 +111,16 @@ gemm_f16_direct_kernel(const GemmParams p)
     const TileCoord tc = tile_of_workgroup(p);
     const half_t * __restrict__ A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
     const half_t * __restrict__ B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
-    OutT * __restrict__ C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
+    OutT * __restrict__ C;
+    if constexpr (SPLIT)
+        C = reinterpret_cast<OutT *>(p.splitWork) + ((size_t)tc.split * p.batch + tc.batch) * p.M * p.N;
+    else
+        C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
 
-    const int M = p.M, N = p.N, K = p.K;
+    /* K: the k range of this workgroup, which starts at kBeg (p.kPerSplit is a multiple of the slab depth, so only
+       the last piece has a ragged end, and that is where the operands end too) */
+    const int kBeg = SPLIT ? tc.split * p.kPerSplit : 0;
+    const int M = p.M, N = p.N, K = SPLIT && kBeg + p.kPerSplit < p.K ? p.kPerSplit : p.K - kBeg;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -157,10 +169,10 @@ gemm_f16_direct_kernel(const GemmParams p)
         }
     }
 
-    const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
-    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const half_t * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
-    const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
+    const half_t * aTile = AKC ? A + (size_t)m0 * p.lda + kBeg : A + m0 + (size_t)kBeg * p.lda;
+    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb + kBeg : B + n0 + (size_t)kBeg * p.ldb;
+    const half_t * aEnd = A + (size_t)((AKC ? M : p.K) - 1) * p.lda + (AKC ? p.K : M);
+    const half_t * bEnd = B + (size_t)((BKC ? N : p.K) - 1) * p.ldb + (BKC ? p.K : N);
 
     const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);
 
@@ -386,12 +398,13 @@ gemm_f16_direct_kernel(const GemmParams p)
        would otherwise have to stay in a register (or be spilled) across the whole main loop */
     const int laneE = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     const int l32E = laneE & 31, lhE = laneE >> 5;
-    const float alpha = p.alpha, beta = p.beta;
+    const float alpha = SPLIT ? 1.f : p.alpha, beta = SPLIT ? 0.f : p.beta;
     const OutT * __restrict__ bias = static_cast<const OutT *>(p.bias);     /* the bias has the type of c */
-    const int biasMode = p.biasMode;
-    const int act = p.act;
-    OutT * cw = C + (size_t)(m0 + wm0) * p.ldc;
-    const unsigned rowPitch = (unsigned)p.ldc * (unsigned)sizeof(OutT);
+    const int biasMode = SPLIT ? (int)BIAS_NONE : p.biasMode;
+    const int act = SPLIT ? (int)ACT_NONE : p.act;
+    const int ldc = SPLIT ? N : p.ldc;
+    OutT * cw = C + (size_t)(m0 + wm0) * ldc;
+    const unsigned rowPitch = (unsigned)ldc * (unsigned)sizeof(OutT);
 
     if constexpr (CS) {
         /* the first tile row's first wave row has seen every k of its columns */
@@ -503,13 +516,13 @@ gemm_f16_direct_kernel(const GemmParams p)
        inside them every load of c would sit in a block of its own, one memory round trip after the other. */
     if (m0 + wm0 >= M)
         return;
-    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * p.ldc * (long long)sizeof(OutT));
+    __amdgpu_buffer_rsrc_t cr = make_rsrc(cw, (long long)(M - m0 - wm0) * ldc * (long long)sizeof(OutT));
     auto narrow = [&](auto BETAC) {
         constexpr bool useOld = decltype(BETAC)::value != 0;
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = n0 + wn0 + j * 32 + l32E;
-            const unsigned cOff = col < N ? (unsigned)(4 * lhE * p.ldc + col) * (unsigned)sizeof(OutT)
+            const unsigned cOff = col < N ? (unsigned)(4 * lhE * ldc + col) * (unsigned)sizeof(OutT)
                                           : (unsigned)NTSAMD_OOB_OFFSET;
             float bcol = 0.f;
             if (biasMode == BIAS_COL && col < N)
@@ -539,15 +552,16 @@ gemm_f16_direct_kernel(const GemmParams p)
         narrow(IntC<0>());
 }
 
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false>
 static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
 {
     GemmParams p = p0;
     p.tilesM = (p.M + BM - 1) / BM;
     p.tilesN = (p.N + BN - 1) / BN;
-    p.splits = 1;
-    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS>),
+    if (!SPLIT)
+        p.splits = 1;
+    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT>),
                        grid, dim3(WGM * WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -562,6 +576,11 @@ static int launch_f16_direct(const GemmParams & p, hipStream_t stream)
            15-20 % faster at k = 512, 3-8 % at k = 1024, level at k = 4096 and 0-4 % slower at k = 8192. */
         if (p.K <= 2048)
             return launch_f16_direct_shape<OutT, S::BM, S::BN, 2, 4, 1, AKC, BKC, CS>(p, stream);
+    }
+    else if constexpr (!CS) {
+        /* pieces of k leave fp32 partial tiles, whatever the type of c */
+        if (p.splits > 1 && p.splitWork != NULL)
+            return launch_f16_direct_shape<float, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS, true>(p, stream);
     }
     return launch_f16_direct_shape<OutT, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>(p, stream);
 }

@@ -9,6 +9,9 @@
 #include "attention.h"
 
 #include <atomic>
+#include <map>
+#include <mutex>
+#include <utility>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -165,33 +168,89 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     return (double)rounds * mfma + ends + cut;
 }
 
-/* The same for fp16, fitted the same way (k is never cut). The 256 x 256 tile runs alone on its CU, so every round
-   pays its ends in full (11.7 us: four slabs to fetch before the first MFMA, 128 KB to store after the last;
-   8.5 us on eight waves, which is how it runs up to k = 2048);
-   the smaller tiles share a CU and hide most of theirs, but re-read their operands from LDS more often per MFMA:
-   per k, a round costs 0.0282 us (256 x 256), 0.0088 us (128 x 128; 0.011 us alone on its CU), 0.00364 us
-   (64 x 64). Short k and many rounds favour the 128 x 128 tile (4096 x 30016 x 512: 172 against 191 us), long k
-   the big one. The clock under fp16 MFMA load depends on how much of the chip is busy, which is why the same
-   tile is faster per k on a product that fills a fraction of the CUs. */
-double tile_cost_f16(int M, int N, int K, int count, int bm)
+/* The same for fp16, fitted to graph-replayed measurements of each tile shape on 8 to 4096 workgroups with k from
+   256 to 4096. Up to 256 workgroups every workgroup has a CU to itself and the time is one workgroup's chain of
+   slabs, nearly whatever their number; beyond, what counts is how many the busiest CU runs (rounds), and the
+   workgroups that share a CU hide each other's waits: per k and round 0.00368 us (64 x 64, against 0.0051 us
+   alone), 0.0086 us (128 x 128, against 0.0078 to 0.0094 us alone), 0.0275 us (256 x 256, which always runs
+   alone on its CU: four slabs to fetch before the first MFMA, 128 KB to store after the last, paid every round:
+   7.2 us on eight waves, which is how it runs up to k = 2048, 3.4 us on four). Short k and many rounds favour
+   the 128 x 128 tile, long k the big one. The clock under fp16 MFMA
+   load depends on how much of the chip is busy, which is why the big tile is faster per k on a product that
+   fills a fraction of the CUs.
+   Cutting k into pieces (few tiles, long k: weight gradients, the few rows of a decoding step) makes as many
+   products of a shorter k, whose fp32 results cross memory once (about 5 TB/s, much of it behind the
+   multiplications) on their way to a second launch (2.3 us) that adds them up. */
+constexpr double SPLIT16_FIXED_US = 2.3, SPLIT16_BYTES_PER_US = 5.0e6;
+
+double tile_cost_f16(int M, int N, int K, int count, int bm, int splits)
 {
+    if (splits > 1) {
+        const int kPiece = ((K + splits - 1) / splits + 31) / 32 * 32;
+        return tile_cost_f16(M, N, kPiece, count * splits, bm, 1) + SPLIT16_FIXED_US +
+               8.0 * M * N * count * splits / SPLIT16_BYTES_PER_US;
+    }
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bm - 1) / bm) * count;
     const long long rounds = (groups + 255) / 256;
-    /* fewer workgroups than CUs: every workgroup is alone on its CU (slower per k for the small tiles, whose
-       ends nobody hides), and the part runs at a higher clock the fewer CUs are busy (down to 0.7 of the time) */
     const bool alone = groups <= 256;
-    const double busy = alone ? (groups < 180 ? 0.7 : (double)groups / 256.0) : 1.0;
-    if (bm >= 256)
-        return (double)rounds * (K <= 2048 ? 0.0275 * busy * K + 8.5 : 0.02816 * busy * K + 11.7);   /* eight waves / four */
-    if (bm >= 128)
-        return (double)rounds * ((alone ? 0.011 : 0.0088) * busy * K + 1.3) + 1.5;
-    return (double)rounds * ((alone ? 0.0051 : 0.00364) * busy * K + 0.2) + 1.9;
+    if (bm >= 256) {
+        /* the fewer CUs are busy, the higher the clock (down to 0.7 of the time) */
+        const double busy = alone ? (groups < 180 ? 0.7 : (double)groups / 256.0) : 1.0;
+        return K <= 2048 ? (double)rounds * (0.0275 * busy * K + 7.2) + 3.0        /* eight waves */
+                         : (double)rounds * (0.02816 * busy * K + 3.4) + 4.0;      /* four */
+    }
+    if (bm >= 128) {
+        if (alone) {
+            const double full = groups <= 128 ? 0.0 : (double)(groups - 128) / 128.0;
+            return (0.0078 + 0.0016 * full) * K + 4.5 + 0.6 * full;
+        }
+        return (double)rounds * 0.0086 * K + 4.3 + 1.4 * (double)(rounds - 1);
+    }
+    if (alone)
+        return 0.0051 * K + (groups <= 128 ? 3.1 : 3.5);
+    return (double)rounds * 0.00368 * K + 3.5 + 0.47 * (double)(rounds - 1);
 }
 
 struct Plan {
     int cfg;
     int splits;
 };
+
+/* Where the pieces of a half product whose k is cut meet: one workspace per device and stream (launches on one
+   stream run one after the other, so they can share; launches on different streams may overlap, so they must
+   not), allocated at the first product that wants it and kept until the process ends. A kernel recorded into a
+   graph keeps the workspace of the stream it was captured on: graphs captured on one stream, and that stream's
+   own launches, must not run at the same time. */
+constexpr size_t SPLIT_WORK_BYTES = (size_t)32 << 20;
+constexpr size_t SPLIT_STREAMS_MAX = 64;            /* per process, over all devices */
+std::mutex g_splitMutex;
+std::map<std::pair<int, hipStream_t>, float *> g_splitWork;
+
+/* NULL: none to be had (no memory, too many streams) and the product runs in one piece. Device devID is current. */
+float * split_work_for(int devID, hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(g_splitMutex);
+    const std::pair<int, hipStream_t> key(devID, stream);
+    std::map<std::pair<int, hipStream_t>, float *>::iterator it = g_splitWork.find(key);
+    if (it != g_splitWork.end())
+        return it->second;
+    if (g_splitWork.size() >= SPLIT_STREAMS_MAX)
+        return NULL;
+    /* the stream may be recording a graph: allocating is allowed then only in the relaxed mode, which is how
+       allocators that serve captures do it; the allocation itself is no part of the graph */
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    void * mem = NULL;
+    const hipError_t err = hipMalloc(&mem, SPLIT_WORK_BYTES);
+    if (exchanged)
+        (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (err != hipSuccess || mem == NULL) {
+        (void)hipGetLastError();
+        return NULL;
+    }
+    g_splitWork[key] = static_cast<float *>(mem);
+    return static_cast<float *>(mem);
+}
 
 /* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
    estimated run time. NTSAMD_TILE_CFG=0|1|2|3 forces a shape (128x128, 64x64, 256x256 for
@@ -218,15 +277,25 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
         forcedSplits = 1;
     Plan best = {CFG_64x64, 1};
     double bestCost = -1.0;
+    /* a forced number of pieces that no shape can take gives way: second turn */
+    for (int turn = 0; turn < 2 && bestCost < 0.0; turn++) {
+    if (turn == 1)
+        forcedSplits = 1;
     for (int cfg = 0; cfg < CFG_COUNT; cfg++) {
         if ((cfg == CFG_256x256 && !half) || (cfg == CFG_32x128 && (half || M > 32)) || (forcedCfg >= 0 && cfg != forcedCfg))
             continue;
         for (int splits = 1; splits <= 16; splits *= 2) {
             if (splits > 1 && (!maySplit || K / splits < 64))
                 break;
+            if (splits > 1 && half) {
+                /* the big tile has no such kernel; the partial products must fit the workspace */
+                if (cfg == CFG_256x256 || K / splits < 128 ||
+                    (long long)M * N * count * splits * 4 > (long long)SPLIT_WORK_BYTES)
+                    break;
+            }
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
-            double c = half ? tile_cost_f16(M, N, K, count, bms[cfg])
+            double c = half ? tile_cost_f16(M, N, K, count, bms[cfg], splits)
                             : tile_cost_f32(M, N, K, count, bms[cfg], bns[cfg], splits, betaPass);
             if (bestCost < 0.0 || c < bestCost) {
                 bestCost = c;
@@ -234,6 +303,7 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
                 best.splits = splits;
             }
         }
+    }
     }
     return best;
 }
@@ -323,8 +393,16 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const bool half = kind != KIND_F32;
     /* cutting k into pieces pays when the result has few tiles and k is long (weight
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
-    const Plan plan = choose_plan(s.M, s.N, s.K, count, half,
-                                  kind == KIND_F32 && vec && !ptrs && act == ACT_NONE && dense, beta != 1.f);
+    /* ... and for half products on the 16-byte path, whose pieces meet in a workspace and leave the ordinary way
+       (any beta, bias, activation, leading dimensions; no column sums) */
+    const bool maySplit = half ? fetch16 == F16_DIRECT && !ptrs && colSum == NULL
+                               : vec && !ptrs && act == ACT_NONE && dense;
+    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f);
+    if (half && plan.splits > 1) {
+        p.splitWork = split_work_for(devID, hs);
+        if (p.splitWork == NULL)
+            plan = choose_plan(s.M, s.N, s.K, count, half, false, beta != 1.f);
+    }
     const int cfg = plan.cfg;
     int rc = 0;
     p.splits = 1;
@@ -332,7 +410,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 31) / 32 * 32;
         p.splits = (s.K + p.kPerSplit - 1) / p.kPerSplit;
     }
-    if (p.splits > 1 && beta != 1.f) {
+    if (!half && p.splits > 1 && beta != 1.f) {
         /* c is dense: count matrices of M x N, strideC apart */
         if (count == 1 || strideC == (long long)s.M * s.N)
             rc = launch_scale(false, c, (long long)s.M * s.N * count, beta, hs);
@@ -347,7 +425,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             /* by-product of the product kernel */
             p.colSum = colSum;
             p.colSumBeta = colSumBeta;
-            if (p.splits > 1)
+            if (!half && p.splits > 1)
                 rc = launch_scale(false, colSum, s.N, colSumBeta, hs);
         }
         else {
@@ -372,6 +450,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         else
             rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, cfg, hs);
     }
+    if (rc == 0 && half && p.splits > 1)
+        rc = launch_split_reduce(p, kind == KIND_F16_F32OUT, hs);
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

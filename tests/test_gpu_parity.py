@@ -51,8 +51,10 @@ def name_the_case(request):
     # a GPU fault can take the box with it: say which test is running first
     print("\n[gpu-case] %s" % request.node.nodeid, flush=True)
     os.environ.pop("NTSAMD_TILE_CFG", None)
+    os.environ.pop("NTSAMD_SPLIT_K", None)
     yield
     os.environ.pop("NTSAMD_TILE_CFG", None)
+    os.environ.pop("NTSAMD_SPLIT_K", None)
 
 
 # ---- fixtures held by the reference and by the compiled reference ------------
@@ -190,6 +192,68 @@ def test_fp16_against_oracle(gpu, oracle, ta, tb):
                 c = dev_tensor(c0, gpu, True) if beta != 0 else torch.full((M, N), float("nan"), device=gpu).half()
                 nt.matrix_mul(dev_tensor(a, gpu, True), ta, dev_tensor(b, gpu, True), tb, c, alpha, beta)
                 assert_fp16(c.float().cpu().numpy(), ref, what="cfg%s %dx%dx%d alpha=%g beta=%g" % (cfg, M, N, K, alpha, beta))
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_products_cut_along_k(gpu, oracle, ta, tb):
+    """Few tiles and a long k (weight gradients, the few rows of a decoding step): k is cut into pieces whose fp32
+    partial products a second kernel adds up and finishes (alpha, beta, bias by column, rectifier, either result
+    type). Forced here on both tile shapes with 2 and 16 pieces, ragged edges and a ragged last piece; the last
+    two shapes are cut by the dispatcher's own choice as well (no forcing: the first turn of the loop)."""
+    torch = torch_()
+    shapes = [(8, 8, 264), (72, 136, 1000), (200, 24, 4096), (16, 512, 2048), (256, 256, 2304)]
+    for cfg, pieces in ((None, None), ("0", "2"), ("0", "16"), ("1", "2"), ("1", "16")):
+        for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces)):
+            if val is None:
+                os.environ.pop(key, None)
+            else:
+                os.environ[key] = val
+        for i, (M, N, K) in enumerate(shapes if cfg else shapes[-2:]):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 8000 + i, 0, 0.5)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 8100 + i, 0, 0.5)))
+            bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((N,), 8300 + i)))
+            for out_float in (False, True):
+                c0 = oracle.uniform((M, N), 8200 + i)
+                if not out_float:
+                    c0 = oracle.from_f16_bits(oracle.to_f16_bits(c0))
+                for alpha, beta, with_bias, act in ((1.0, 0.0, False, nt.ACT_NONE), (0.5, 1.0, False, nt.ACT_NONE),
+                                                    (1.0, 0.0, True, nt.ACT_NONE), (1.0, 0.5, True, nt.ACT_RECTIFY)):
+                    ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                    if with_bias:
+                        ref = ref + bias[None, :]
+                    if act == nt.ACT_RECTIFY:
+                        ref = np.maximum(ref, 0)
+                    c = dev_tensor(c0, gpu, not out_float) if beta != 0 else \
+                        torch.full((M, N), float("nan"), device=gpu, dtype=torch.float32 if out_float else torch.float16)
+                    nt.matrix_mul(dev_tensor(a, gpu, True), ta, dev_tensor(b, gpu, True), tb, c, alpha, beta,
+                                  bias=dev_tensor(bias, gpu, not out_float) if with_bias else None, act=act)
+                    what = "cfg%s pieces=%s %dx%dx%d alpha=%g beta=%g bias=%s act=%d float=%s" % (
+                        cfg, pieces, M, N, K, alpha, beta, with_bias, act, out_float)
+                    if out_float:
+                        assert_fp32(c.cpu().numpy(), ref, K, what=what)
+                    else:
+                        assert_fp16(c.float().cpu().numpy(), ref, what=what)
+
+
+def test_batches_of_half_products_cut_along_k(gpu, oracle):
+    """Three products with their own strides between them and rows of c longer than the result is wide (the heads
+    of a merged tensor): every piece of every item finds its place in the workspace and in c, and what lies
+    between the rows of c stays as it was. Twice in a row on one stream: the second call reuses the workspace."""
+    torch = torch_()
+    os.environ["NTSAMD_TILE_CFG"] = "1"
+    os.environ["NTSAMD_SPLIT_K"] = "4"
+    M, N, K, count = 40, 72, 1536, 3
+    ldc, between = 3 * N, N
+    a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((count, M, K), 8400, 0, 0.5)))
+    b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((count, K, N), 8401, 0, 0.5)))
+    for turn in range(2):
+        whole = torch.full((M, ldc), -7.0, device=gpu, dtype=torch.float16)
+        nt.matrix_mul_batched_grid(dev_tensor(a, gpu, True), X_NOTRANS, K, (M * K, 0), dev_tensor(b, gpu, True), X_NOTRANS, N, (K * N, 0),
+                                   whole, ldc, (between, 0), count, 1, M, K, K, N, M, N, 1.0 + turn, 0.0)
+        got = whole.float().cpu().numpy()
+        for i in range(count):
+            ref = oracle.matmul2d(a[i], X_NOTRANS, b[i], X_NOTRANS, None, 1.0 + turn, 0.0)
+            assert_fp16(got[:, i * between:i * between + N], ref, what="item %d turn %d" % (i, turn))
 
 
 def test_fp16_bits_match_the_oracle_conversion(gpu, oracle):
