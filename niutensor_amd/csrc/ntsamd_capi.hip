@@ -255,7 +255,7 @@ float * split_work_for(int devID, hipStream_t stream)
 /* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
    estimated run time. NTSAMD_TILE_CFG=0|1|2|3 forces a shape (128x128, 64x64, 256x256 for
    half, 32x128 for float) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
-Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass)
+Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass, double cutExtra = 0.0)
 {
     static const int bms[CFG_COUNT] = {128, 64, 256, 32};
     static const int bns[CFG_COUNT] = {128, 64, 256, 128};
@@ -297,6 +297,8 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
                 continue;
             double c = half ? tile_cost_f16(M, N, K, count, bms[cfg], splits)
                             : tile_cost_f32(M, N, K, count, bms[cfg], bns[cfg], splits, betaPass);
+            if (splits > 1)
+                c += cutExtra;
             if (bestCost < 0.0 || c < bestCost) {
                 bestCost = c;
                 best.cfg = cfg;
@@ -395,9 +397,13 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
        gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
     /* ... and for half products on the 16-byte path, whose pieces meet in a workspace and leave the ordinary way
        (any beta, bias, activation, leading dimensions; no column sums) */
-    const bool maySplit = half ? fetch16 == F16_DIRECT && !ptrs && colSum == NULL
+    const bool maySplit = half ? fetch16 == F16_DIRECT && !ptrs
                                : vec && !ptrs && act == ACT_NONE && dense;
-    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f);
+    /* the pieces of a half product gather no column sums: cutting costs a pass of its own over b then (a launch,
+       b read once more) */
+    const bool colSumAside = half && colSum != NULL && vec && count == 1;
+    const double cutExtra = colSumAside ? 2.3 + 2.0 * s.K * s.N / 4.0e6 : 0.0;
+    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, cutExtra);
     if (half && plan.splits > 1) {
         p.splitWork = split_work_for(devID, hs);
         if (p.splitWork == NULL)
@@ -421,7 +427,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
     if (colSum != NULL) {
-        if (vec && count == 1) {
+        if (vec && count == 1 && !(half && plan.splits > 1)) {
             /* by-product of the product kernel */
             p.colSum = colSum;
             p.colSumBeta = colSumBeta;

@@ -163,6 +163,29 @@ def test_colsum_with_split_k_and_without_a_product(gpu, oracle):
     assert_fp32(s.cpu().numpy(), s0 + oracle.reduce_sum(b, 0), K)
 
 
+def test_half_colsum_with_k_cut(gpu, oracle):
+    """The half weight gradient with its bias gradient: cut along k the product leaves the sums to a pass of its
+    own over b (the pieces gather none); both ways give the same sums and a product within the half limit."""
+    M, N, K = 128, 256, 4096
+    a, b = halfed(oracle, oracle.normal((K, M), 1, 0, 0.5)), halfed(oracle, oracle.normal((K, N), 2, 0, 0.5))
+    c0, s0 = halfed(oracle, oracle.uniform((M, N), 3)), halfed(oracle, oracle.uniform((N,), 4))
+    ref = oracle.matmul2d(a, X_TRANS, b, X_NOTRANS, c0.copy(), 1.0, 1.0)
+    for splits in ("1", "8", None):
+        if splits is None:
+            os.environ.pop("NTSAMD_SPLIT_K", None)
+        else:
+            os.environ["NTSAMD_SPLIT_K"] = splits
+        for sbeta in (1.0, 0.0):
+            c, s = dev(c0, gpu, True), dev(s0, gpu, True)
+            nt.matrix_mul_colsum(dev(a, gpu, True), X_TRANS, dev(b, gpu, True), X_NOTRANS, c, s, 1.0, 1.0, sbeta)
+            what = "pieces %s sbeta %g" % (splits, sbeta)
+            assert_fp16(c.float().cpu().numpy(), ref, what=what)
+            sref = sbeta * s0 + oracle.reduce_sum(b, 0)
+            smag = np.abs(sbeta * s0) + oracle.reduce_sum(np.abs(b), 0)
+            assert np.abs(s.float().cpu().numpy() - sref).max() <= 2.0 ** -10 * smag.max() + 1e-6, what
+    os.environ.pop("NTSAMD_SPLIT_K", None)
+
+
 # ---- the reduction ------------------------------------------------------------------------
 
 @pytest.mark.parametrize("half", (False, True))
