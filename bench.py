@@ -56,6 +56,9 @@ def configs():
         12: dict(name="cfg12 fp32 attention context on merged tensors: Merge(BMMul(att[8x32x128x128], Split(v[32x128x512]))) as one "
                       "batched product that reads the heads of v and writes the merged result where they stand",
                  dtype="f32", M=128, N=64, K=128, batch=256),
+        13: dict(name="cfg13 fp16 weight gradient of a 512x512 projection over 4096 positions: dW += X^T.dY (TN, beta=1), k cut into "
+                      "pieces whose fp32 partial products a second kernel adds up",
+                 dtype="f16", M=512, N=512, K=4096, batch=1),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -107,6 +110,15 @@ class Workload:
             self.flops = 2.0 * 8192 * 4096 * 1024
             self.bytes = 2.0 * (1024 * 8192 + 1024 * 4096 + 8192 * 4096)
             self.launches = 1
+        elif idx == 13:
+            self.x = g(oracle.normal((4096, 512), 1)).half()
+            self.dy = g(oracle.normal((4096, 512), 2, 0, 0.02)).half()
+            self.dw = torch.zeros((512, 512), device=dev, dtype=torch.float16)
+            self.run = lambda: nt.matrix_mul(self.x, T, self.dy, NT, self.dw, 1.0, 1.0)
+            self.flops = 2.0 * 512 * 512 * 4096
+            # x and dY read once, dW read and written; the partial products (workspace) are no part of the algorithm
+            self.bytes = 2.0 * (2 * 4096 * 512 + 2 * 512 * 512)
+            self.launches = 2
         elif idx == 5:
             self.h = g(oracle.uniform((4096, 512), 1))
             self.w = g(oracle.normal((30011, 512), 2, 0, 0.02))
@@ -222,7 +234,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 13: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -293,12 +305,13 @@ def cpu_baseline(idx, budget_s=12.0):
             else:
                 o.rectify(o.mulandshift(a.reshape(1, rows, K), b, bias)[0])
             dt = time.perf_counter() - t0
-        elif idx == 4:
+        elif idx in (4, 13):
             # fp32 arithmetic on the half-rounded values: the reference has no CPU half product
             a = o.from_f16_bits(o.to_f16_bits(o.normal((K, rows), 1, 0, 0.02)))
             b = o.from_f16_bits(o.to_f16_bits(o.normal((K, N), 2, 0, 0.02)))
+            c = np.zeros((rows, N), np.float32)
             t0 = time.perf_counter()
-            o.matmul2d(a, X_TRANS, b, X_NOTRANS)
+            o.matmul2d(a, X_TRANS, b, X_NOTRANS, c, 1.0, 1.0 if idx == 13 else 0.0)
             dt = time.perf_counter() - t0
         else:
             a, b = o.uniform((rows, K), 1), o.normal((N, K), 2, 0, 0.02)
@@ -411,7 +424,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-12 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-13 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -439,7 +452,7 @@ def main():
         return
     oracle = Oracle()
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13):
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
             print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
                                        not args.no_cpu)), flush=True)

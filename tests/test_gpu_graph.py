@@ -1,8 +1,10 @@
-"""The entry points allocate nothing and never synchronise, so a caller may record them into a HIP graph
-on its own stream and replay it: a linear layer with Rectify, the two attention products, the attention
-in one kernel, a product cut along k (atomics after a scaling pass) and a conversion are captured once
-and replayed with new inputs; every replay must reproduce the eager results bit for bit (the product
-cut along k, whose additions are unordered: within the fp32 limit)."""
+"""The entry points never synchronise, so a caller may record them into a HIP graph on its own stream and
+replay it: a linear layer with Rectify, the two attention products, the attention in one kernel, a float
+product cut along k (atomics after a scaling pass), a half product cut along k (partial products in the
+library's workspace, which the capturing stream does not have yet: the one allocation the library makes,
+in the relaxed capture mode) and a conversion are captured once and replayed with new inputs; every
+replay must reproduce the eager results bit for bit (the float product cut along k, whose additions are
+unordered: within the fp32 limit)."""
 import os
 
 import numpy as np
@@ -29,6 +31,8 @@ def test_replays_match_eager(gpu, oracle):
     att = torch.empty((4, 70, 64), device=dev)
     cut = torch.empty((64, 64), device=dev)
     h16 = torch.empty((256, 160), device=dev, dtype=torch.float16)
+    big_a16, big_b16 = big_a.half(), big_b.half()
+    cut16 = torch.empty((64, 64), device=dev, dtype=torch.float16)
 
     def step():
         nt.matrix_mul(x, X_NOTRANS, w, X_NOTRANS, h, 1.0, 0.0, bias=b, act=nt.ACT_RECTIFY)
@@ -37,6 +41,7 @@ def test_replays_match_eager(gpu, oracle):
         nt.attention(q, k, v, att, 2, 0.25)
         nt.matrix_mul(big_a, X_NOTRANS, big_b, X_NOTRANS, cut, 1.0, 0.0)
         nt.convert_data_type(h, h16)
+        nt.matrix_mul(big_a16, X_NOTRANS, big_b16, X_NOTRANS, cut16, 1.0, 0.0)
 
     os.environ["NTSAMD_SPLIT_K"] = "4"                  # the product with the long k goes out in four pieces
     try:
@@ -53,15 +58,16 @@ def test_replays_match_eager(gpu, oracle):
             # new inputs in place, eager results first
             for t, seed in ((x, 10), (q, 11), (k, 12), (v, 13), (big_a, 14)):
                 t.copy_(g(oracle.uniform(tuple(t.shape), seed + 10 * rep)))
+            big_a16.copy_(big_a)
             step()
             torch.cuda.synchronize()
-            want = [t.clone() for t in (h, s, o, att, cut, h16)]
-            for t in (h, s, o, att, cut, h16):
+            want = [t.clone() for t in (h, s, o, att, cut, h16, cut16)]
+            for t in (h, s, o, att, cut, h16, cut16):
                 t.fill_(float("nan"))
             graph.replay()
             torch.cuda.synchronize()
-            for name, got, ref in zip(("linear layer", "scores", "context", "attention", "cut along k", "conversion"),
-                                      (h, s, o, att, cut, h16), want):
+            for name, got, ref in zip(("linear layer", "scores", "context", "attention", "cut along k", "conversion",
+                                       "half, cut along k"), (h, s, o, att, cut, h16, cut16), want):
                 if name == "cut along k":
                     assert_fp32(got.cpu().numpy(), ref.cpu().numpy(), 2048, what="replay %d: %s" % (rep, name))
                 else:
