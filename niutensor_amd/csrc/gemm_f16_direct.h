@@ -79,14 +79,14 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
 /* SPLIT: the k range is cut into p.splits pieces, one workgroup each, and every workgroup leaves its partial tile
    as plain fp32 (no alpha, beta, bias or activation) in p.splitWork, which holds p.splits x p.batch dense M x N
    matrices; split_reduce.hip adds the pieces up and does what the epilogue would have done. */
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
     static_assert(!CS || std::is_same<OutT, half_t>::value, "column sums have the type of b and of c");
     static_assert(!(CS && SPLIT), "column sums are not gathered from pieces of k");
     static_assert(!SPLIT || std::is_same<OutT, float>::value, "partial tiles are fp32");
-    constexpr int BKT = 32, KS = 2, NSTAGE = 4;
+    constexpr int BKT = 32, KS = 2;
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TI = WM / 32, TJ = WN / 32;
@@ -347,7 +347,124 @@ gemm_f16_direct_kernel(const GemmParams p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    if (nk > 0) {
+    /* A wave with one accumulator block (the 64 x 64 tile) has one MFMA per k step to wait behind, and an LDS
+       read takes four times as long to come back: with its fragments requested one k step ahead, as below, such a
+       wave spends its time waiting for them (0.16 us per slab for a workgroup alone on its CU). It asks for the
+       fragments of a whole slab at once instead, one slab ahead, into a second set of registers (0.14 us per slab).
+       The loop is written for any number of stages; eight instead of four gain nothing (measured: a lone
+       workgroup is not waiting for memory either), and four leave room for four workgroups on a CU. */
+    constexpr bool DEEP = TI == 1 && TJ == 1;
+    if constexpr (DEEP) {
+        f16x8 da[2][KS], db[2][KS];                  /* [set][k step] */
+        auto read_set = [&](auto SETC, const char * stage) {
+            constexpr int S = decltype(SETC)::value;
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++) {
+                if constexpr (AKC)
+                    da[S][kk] = *reinterpret_cast<const f16x8 *>(stage + aFrag[kk]);
+                else {
+                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][0]));
+                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][1]));
+                    da[S][kk] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+                if constexpr (BKC)
+                    db[S][kk] = *reinterpret_cast<const f16x8 *>(stage + bFrag[kk]);
+                else {
+                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][0]));
+                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][1]));
+                    db[S][kk] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+            }
+        };
+        /* Slab kt, whose fragments are in set S. AHEAD = how many later slabs exist (capped at NSTAGE). */
+        auto deep_slab = [&](auto SETC, auto AHEADC, auto TAILC, int kt) {
+            constexpr int S = decltype(SETC)::value;
+            constexpr int ahead = decltype(AHEADC)::value;
+            if constexpr (ahead >= 1) {
+                /* slab kt+1 must have landed: at most the loads of slabs kt+2 .. kt+NSTAGE-1 stay in flight. Every
+                   wave's reads of this slab's stage have come back by the barrier (they are what the MFMAs below
+                   wait for anyway), so the stage is free after it. */
+                wait_vmcnt<((ahead < NSTAGE - 1 ? ahead : NSTAGE - 1) - 1) * NL>();
+                wait_lgkmcnt0();
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                read_set(IntC<S ^ 1>(), lds + ((kt + 1) % NSTAGE) * STAGE);
+                if constexpr (ahead >= NSTAGE)
+                    issue_loads(TAILC, kt + NSTAGE);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++) {
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(da[S][kk], db[S][kk], acc[0][0], 0, 0, 0);
+                if constexpr (CS) {
+                    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                    const h2 ones = {(_Float16)1, (_Float16)1};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const h2 pr = {db[S][kk][2 * e], db[S][kk][2 * e + 1]};
+                        colSum[0] = __builtin_amdgcn_fdot2(pr, ones, colSum[0], false);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        static_assert((NSTAGE - 1) * NL < 64, "the wait counter has six bits");
+        if (nk > 0) {
+            /* prologue: every stage in flight, then wait for the first */
+            auto issue_first = [&](auto self, auto NC) {
+                constexpr int n = decltype(NC)::value;
+                if constexpr (n < NSTAGE) {
+                    if (nk > n) {
+                        issue_loads(IntC<1>(), n);
+                        self(self, IntC<n + 1>());
+                    }
+                }
+            };
+            issue_first(issue_first, IntC<0>());
+            auto wait_first = [&](auto self, auto NC) {
+                constexpr int n = decltype(NC)::value;          /* slabs in flight besides the first */
+                if (nk > n)
+                    wait_vmcnt<n * NL>();
+                else if constexpr (n > 0)
+                    self(self, IntC<n - 1>());
+            };
+            wait_first(wait_first, IntC<NSTAGE - 1>());
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            read_set(IntC<0>(), lds);
+
+            /* two slabs per turn, so that the register sets have fixed names; kt stays even */
+            const int nkFull = K / BKT;
+            int kt = 0;
+            for (; kt + NSTAGE + 1 < nkFull; kt += 2) {  /* the slabs to fetch are complete: no tail handling */
+                deep_slab(IntC<0>(), IntC<NSTAGE>(), IntC<0>(), kt);
+                deep_slab(IntC<1>(), IntC<NSTAGE>(), IntC<0>(), kt + 1);
+            }
+            for (; kt + NSTAGE + 1 < nk; kt += 2) {
+                deep_slab(IntC<0>(), IntC<NSTAGE>(), IntC<1>(), kt);
+                deep_slab(IntC<1>(), IntC<NSTAGE>(), IntC<1>(), kt + 1);
+            }
+            /* one to NSTAGE + 1 slabs are left, the first of them in set 0: the one with R slabs to go (itself
+               included) is in set (left - R) & 1 */
+            const int left = nk - kt;
+            auto rest = [&](auto self, auto RC, auto PARC) {
+                constexpr int R = decltype(RC)::value, P = decltype(PARC)::value;
+                if constexpr (R >= 1) {
+                    if (nk - kt == R) {
+                        deep_slab(IntC<((P + R) & 1)>(), IntC<(R - 1 < NSTAGE ? R - 1 : NSTAGE)>(), IntC<1>(), kt);
+                        kt++;
+                    }
+                    self(self, IntC<R - 1>(), PARC);
+                }
+            };
+            if (left & 1)
+                rest(rest, IntC<NSTAGE + 1>(), IntC<1>());
+            else
+                rest(rest, IntC<NSTAGE + 1>(), IntC<0>());
+        }
+    }
+    else if (nk > 0) {
+        static_assert(DEEP || NSTAGE == 4, "this loop is written for four stages");
         /* prologue: all four stages in flight, then wait for the first */
         issue_loads(IntC<1>(), 0);
         if (nk > 1)
@@ -552,7 +669,7 @@ gemm_f16_direct_kernel(const GemmParams p)
         narrow(IntC<0>());
 }
 
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4>
 static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
 {
     GemmParams p = p0;
@@ -561,7 +678,7 @@ static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
     if (!SPLIT)
         p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT>),
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT, NSTAGE>),
                        grid, dim3(WGM * WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }

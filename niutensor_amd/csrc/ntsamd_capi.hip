@@ -171,7 +171,7 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
 /* The same for fp16, fitted to graph-replayed measurements of each tile shape on 8 to 4096 workgroups with k from
    256 to 4096. Up to 256 workgroups every workgroup has a CU to itself and the time is one workgroup's chain of
    slabs, nearly whatever their number; beyond, what counts is how many the busiest CU runs (rounds), and the
-   workgroups that share a CU hide each other's waits: per k and round 0.00368 us (64 x 64, against 0.0051 us
+   workgroups that share a CU hide each other's waits: per k and round 0.00368 us (64 x 64, against 0.0045 us
    alone), 0.0086 us (128 x 128, against 0.0078 to 0.0094 us alone), 0.0275 us (256 x 256, which always runs
    alone on its CU: four slabs to fetch before the first MFMA, 128 KB to store after the last, paid every round:
    7.2 us on eight waves, which is how it runs up to k = 2048, 3.4 us on four). Short k and many rounds favour
@@ -207,7 +207,7 @@ double tile_cost_f16(int M, int N, int K, int count, int bm, int splits)
         return (double)rounds * 0.0086 * K + 4.3 + 1.4 * (double)(rounds - 1);
     }
     if (alone)
-        return 0.0051 * K + (groups <= 128 ? 3.1 : 3.5);
+        return 0.0045 * K + (groups <= 128 ? 3.15 : 3.45);
     return (double)rounds * 0.00368 * K + 3.5 + 0.47 * (double)(rounds - 1);
 }
 
