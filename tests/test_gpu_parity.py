@@ -201,7 +201,9 @@ def test_half_products_cut_along_k(gpu, oracle, ta, tb):
     type). Forced here on both tile shapes with 2 and 16 pieces, ragged edges and a ragged last piece; the last
     two shapes are cut by the dispatcher's own choice as well (no forcing: the first turn of the loop)."""
     torch = torch_()
-    shapes = [(8, 8, 264), (72, 136, 1000), (200, 24, 4096), (16, 512, 2048), (256, 256, 2304)]
+    # 51 columns: rows of c that the adding kernel cannot take four elements at a time (cut only where b is stored
+    # n x k: the 16-byte path needs whole 16-byte pieces along the rows of b)
+    shapes = [(8, 8, 264), (72, 136, 1000), (40, 51, 1024), (200, 24, 4096), (16, 512, 2048), (256, 256, 2304)]
     for cfg, pieces in ((None, None), ("0", "2"), ("0", "16"), ("1", "2"), ("1", "16")):
         for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces)):
             if val is None:
