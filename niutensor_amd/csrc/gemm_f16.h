@@ -22,9 +22,15 @@
  *       keeps the four rows of one read in different bank groups.
  *
  * Pipeline per slab of BKT values of k, as in the fp32 kernel: all fragments of
- * the current slab sit in registers; the next slab goes global -> registers (one
- * slab ahead) -> the other LDS stage -> one barrier -> the second register set,
- * and every one of those instructions is interleaved between MFMAs.
+ * the current slab sit in registers; a later slab goes global -> registers ->
+ * the other LDS stage -> one barrier -> the second register set, and every one
+ * of those instructions is interleaved between MFMAs. The registers between
+ * global memory and LDS are a ring of RING slabs: a slab is requested RING
+ * slabs before its turn and written to LDS one slab before it, so RING - 1
+ * slabs are on their way at any time (a trip to memory takes several slabs'
+ * worth of MFMAs, and nothing else covers it where a workgroup has its CU to
+ * itself: 4096 x 512 x 30011 with rows of 30011 halves took 642 us with one slab
+ * on its way).
  */
 #pragma once
 #include "gemm_common.h"
@@ -42,23 +48,6 @@ __device__ __forceinline__ f16x8 buffer_load_f16x8(__amdgpu_buffer_rsrc_t rsrc, 
 }
 
 /* transposing LDS read: see the header comment for what each lane receives */
-/* Eight halves from any 2-byte aligned place in a buffer of `bytes` bytes. A 16-byte buffer load may start on any
-   even address, but its range check works on whole dwords: where the eight halves hang over the end of the buffer
-   the dword that straddles the end is dropped with its valid half. Such a piece (the last of the matrix, at most)
-   is fetched half by half instead; the branch is taken by no lane almost everywhere. */
-__device__ __forceinline__ f16x8 buffer_load_f16x8_any(__amdgpu_buffer_rsrc_t rsrc, int byteOffset, int bytes)
-{
-    f16x8 v;
-    if ((unsigned)byteOffset < (unsigned)bytes && (unsigned)byteOffset + 16u > (unsigned)bytes) {
-#pragma unroll
-        for (int e = 0; e < 8; e++)
-            v[e] = __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(rsrc, byteOffset + 2 * e, 0, 0));
-    }
-    else
-        v = buffer_load_f16x8(rsrc, byteOffset);
-    return v;
-}
-
 __device__ __forceinline__ f16x4 lds_read_tr16(const half_t * p)
 {
     typedef __fp16 hv4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
@@ -106,6 +95,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     constexpr int NB = BN * BKT / 8 / NT;
     constexpr int ASIZE = AKC ? BM * LDK : BKT * LDA;
     constexpr int BSIZE = BKC ? BN * LDK : BKT * LDB;
+    constexpr int RING = 4;               /* slabs between global memory and LDS, in registers */
     constexpr int NMFMA = KS * TI * TJ;   /* MFMAs per slab */
     constexpr int PRE = NMFMA / 4;        /* MFMAs issued before the slab's barrier */
     constexpr int PREG = PRE > 0 ? PRE : 1;
@@ -187,18 +177,23 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     const half_t * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
     const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
 
-    f16x8 ra[NA], rb[NB];
+    f16x8 ra[RING][NA], rb[RING][NB];
 
-    auto load_global = [&](auto TAIL, int k0) {
+    auto load_global = [&](auto RINGC, auto TAIL, int k0) {
+        constexpr int rg = decltype(RINGC)::value;
         constexpr bool mayHangOver = decltype(TAIL)::value != 0;
         if constexpr (VEC) {
             const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
             const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
-            const long long aLeft = (long long)(aEnd - ab) * 2, bLeft = (long long)(bEnd - bb) * 2;
-            const int aBytes = aLeft >> 31 ? 0x7fffffff : (int)aLeft, bBytes = bLeft >> 31 ? 0x7fffffff : (int)bLeft;
-            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, aLeft);
-            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, bLeft);
-            /* rows of k past the end of an MN-contiguous matrix read as zero by themselves;
+            /* A 16-byte buffer load may start on any even address, but its range check works on whole dwords: where
+               the eight halves hang over the end of the buffer (the last piece of the matrix, at most), the dword
+               that straddles the end would be dropped with its valid half. Two bytes more on the descriptor let it
+               through: the other half of that dword is read, from the same aligned dword that holds the last
+               element (so from the same page), and lands where nothing looks: a column past M or N, or a k that
+               the masks below set to zero. A dword that starts at the end or beyond is still out of range. */
+            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, (long long)(aEnd - ab) * 2 + 2);
+            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, (long long)(bEnd - bb) * 2 + 2);
+            /* Rows of k past the end of an MN-contiguous matrix read as zero by themselves;
                a K-contiguous row would run on into the next row, so those lanes are sent
                out of range explicitly, and the halves of a piece that straddles K are set to zero
                (last slab only) */
@@ -208,12 +203,12 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 int off = aOff[s];
                 if (AKC && tail && k0 + aK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                ra[s] = buffer_load_f16x8_any(ar, off, aBytes);
+                ra[rg][s] = buffer_load_f16x8(ar, off);
                 if constexpr (mayHangOver && AKC)
                     if (tail) {
 #pragma unroll
                         for (int e = 1; e < 8; e++)
-                            ra[s][e] = k0 + aK[s] + e < K ? ra[s][e] : (half_t)0;
+                            ra[rg][s][e] = k0 + aK[s] + e < K ? ra[rg][s][e] : (half_t)0;
                     }
             }
 #pragma unroll
@@ -221,12 +216,12 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 int off = bOff[s];
                 if (BKC && tail && k0 + bK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                rb[s] = buffer_load_f16x8_any(br, off, bBytes);
+                rb[rg][s] = buffer_load_f16x8(br, off);
                 if constexpr (mayHangOver && BKC)
                     if (tail) {
 #pragma unroll
                         for (int e = 1; e < 8; e++)
-                            rb[s][e] = k0 + bK[s] + e < K ? rb[s][e] : (half_t)0;
+                            rb[rg][s][e] = k0 + bK[s] + e < K ? rb[rg][s][e] : (half_t)0;
                     }
             }
         }
@@ -251,7 +246,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                         v[e] = rp[c];
                     }
                 }
-                ra[s] = v;
+                ra[rg][s] = v;
             }
 #pragma unroll
             for (int s = 0; s < NB; s++) {
@@ -272,18 +267,19 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                         v[e] = rp[c];
                     }
                 }
-                rb[s] = v;
+                rb[rg][s] = v;
             }
         }
     };
 
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](auto RINGC, int buf) {
+        constexpr int rg = decltype(RINGC)::value;
 #pragma unroll
         for (int s = 0; s < NA; s++)
-            *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = ra[s];
+            *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = ra[rg][s];
 #pragma unroll
         for (int s = 0; s < NB; s++)
-            *reinterpret_cast<f16x8 *>(&Bs[buf][bLds[s]]) = rb[s];
+            *reinterpret_cast<f16x8 *>(&Bs[buf][bLds[s]]) = rb[rg][s];
     };
 
     /* ---- fragments: two register sets, [set][k step][block] ------------------- */
@@ -356,13 +352,16 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
 
     const int nk = (K + BKT - 1) / BKT;
 
-    /* One slab: fragments of slab kt are in register set SET and came from LDS stage SET.
-       FULL: slabs kt+1 and kt+2 exist and are complete, so the slab is straight-line code. */
-    auto slab = [&](auto SET, auto FULL, int kt) {
-        constexpr int set = decltype(SET)::value;
+    /* One slab, number kt = SLOT mod RING: its fragments are in register set SLOT % 2 and came from LDS stage
+       SLOT % 2. FULL: slabs kt+1 .. kt+RING exist and are complete, so the slab is straight-line code. */
+    auto slab = [&](auto SLOT, auto FULL, int kt) {
+        constexpr int slot = decltype(SLOT)::value;
+        constexpr int set = slot & 1;
+        typedef IntC<set> SET_T;
+        const SET_T SET = SET_T();
         constexpr bool full = decltype(FULL)::value != 0;
         if (full || kt + 1 < nk)
-            store_lds(set ^ 1);                  /* slab kt+1, fetched during slab kt-1 */
+            store_lds(IntC<(slot + 1) % RING>(), set ^ 1);     /* slab kt+1, requested during slab kt+1-RING */
         mfma_range(SET, 0, PRE);
         if constexpr (full) {
 #pragma unroll
@@ -375,10 +374,11 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();                         /* stage set^1 complete; stage set no longer read by anyone */
         __builtin_amdgcn_sched_barrier(0);
+        /* slab kt+RING into the registers that slab kt left for LDS one slab ago */
         if (full)
-            load_global(IntC<0>(), (kt + 2) * BKT);
-        else if (kt + 2 < nk)
-            load_global(IntC<1>(), (kt + 2) * BKT);
+            load_global(IntC<slot>(), IntC<0>(), (kt + RING) * BKT);
+        else if (kt + RING < nk)
+            load_global(IntC<slot>(), IntC<1>(), (kt + RING) * BKT);
         if (full || kt + 1 < nk)
             read_frags(IntC<set ^ 1>(), set ^ 1);
         mfma_range(SET, PRE, NMFMA);
@@ -396,24 +396,40 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         }
     };
 
+    static_assert(RING >= 2 && RING % 2 == 0, "the ring and the two LDS stages turn together");
     if (nk > 0) {
-        load_global(IntC<1>(), 0);
-        store_lds(0);
-        if (nk > 1)
-            load_global(IntC<1>(), BKT);
+        /* slabs 0 .. RING-1 requested, slab 0 on to LDS (slab 0's turn then asks for slab RING) */
+        auto first = [&](auto self, auto SLOT) {
+            constexpr int slot = decltype(SLOT)::value;
+            if constexpr (slot < RING) {
+                if (slot < nk) {
+                    load_global(SLOT, IntC<1>(), slot * BKT);
+                    self(self, IntC<slot + 1>());
+                }
+            }
+        };
+        first(first, IntC<0>());
+        store_lds(IntC<0>(), 0);
         __syncthreads();
         read_frags(IntC<0>(), 0);
         const int nkFull = K / BKT;
+        /* RING slabs per turn, so that registers and stages have fixed names; kt stays a multiple of RING */
+        auto turn = [&](auto self, auto SLOT, auto FULL, int kt) {
+            constexpr int slot = decltype(SLOT)::value;
+            constexpr bool full = decltype(FULL)::value != 0;
+            if constexpr (slot < RING) {
+                if (full || kt + slot < nk) {
+                    slab(SLOT, FULL, kt + slot);
+                    self(self, IntC<slot + 1>(), FULL, kt);
+                }
+            }
+        };
         int kt = 0;
-        for (; kt + 3 < nkFull; kt += 2) {
-            slab(IntC<0>(), IntC<1>(), kt);
-            slab(IntC<1>(), IntC<1>(), kt + 1);
-        }
-        for (; kt < nk; kt += 2) {
-            slab(IntC<0>(), IntC<0>(), kt);
-            if (kt + 1 < nk)
-                slab(IntC<1>(), IntC<0>(), kt + 1);
-        }
+        /* straight-line turns: every slab they ask for is complete */
+        for (; kt + 2 * RING - 1 < nkFull; kt += RING)
+            turn(turn, IntC<0>(), IntC<1>(), kt);
+        for (; kt < nk; kt += RING)
+            turn(turn, IntC<0>(), IntC<0>(), kt);
     }
 
     /* ---- epilogue: accumulator register r of lane l is element
