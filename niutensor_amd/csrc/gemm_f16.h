@@ -47,6 +47,24 @@ __device__ __forceinline__ f16x8 buffer_load_f16x8(__amdgpu_buffer_rsrc_t rsrc, 
     return __builtin_bit_cast(f16x8, v);
 }
 
+/* Eight halves from any 2-byte aligned place in a buffer of `bytes` bytes. A 16-byte buffer load may start on any
+   even address, but its range check works on whole dwords: where the eight halves hang over the end of the buffer
+   the dword that straddles the end is dropped with its valid half. Such a piece (the last of the matrix, at most)
+   is fetched half by half instead. The test is a branch around the load, and a loop body cut up by branches waits
+   for ALL loads in flight at every turn: only the loads of the last slabs go through here. */
+__device__ __forceinline__ f16x8 buffer_load_f16x8_any(__amdgpu_buffer_rsrc_t rsrc, int byteOffset, int bytes)
+{
+    f16x8 v;
+    if ((unsigned)byteOffset < (unsigned)bytes && (unsigned)byteOffset + 16u > (unsigned)bytes) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            v[e] = __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(rsrc, byteOffset + 2 * e, 0, 0));
+    }
+    else
+        v = buffer_load_f16x8(rsrc, byteOffset);
+    return v;
+}
+
 /* transposing LDS read: see the header comment for what each lane receives */
 __device__ __forceinline__ f16x4 lds_read_tr16(const half_t * p)
 {
@@ -185,15 +203,14 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         if constexpr (VEC) {
             const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
             const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
-            /* A 16-byte buffer load may start on any even address, but its range check works on whole dwords: where
-               the eight halves hang over the end of the buffer (the last piece of the matrix, at most), the dword
-               that straddles the end would be dropped with its valid half. Two bytes more on the descriptor let it
-               through: the other half of that dword is read, from the same aligned dword that holds the last
-               element (so from the same page), and lands where nothing looks: a column past M or N, or a k that
-               the masks below set to zero. A dword that starts at the end or beyond is still out of range. */
-            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, (long long)(aEnd - ab) * 2 + 2);
-            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, (long long)(bEnd - bb) * 2 + 2);
-            /* Rows of k past the end of an MN-contiguous matrix read as zero by themselves;
+            const long long aLeft = (long long)(aEnd - ab) * 2, bLeft = (long long)(bEnd - bb) * 2;
+            const int aBytes = aLeft >> 31 ? 0x7fffffff : (int)aLeft, bBytes = bLeft >> 31 ? 0x7fffffff : (int)bLeft;
+            __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, aLeft);
+            __amdgpu_buffer_rsrc_t br = make_rsrc(bb, bLeft);
+            /* The one piece that can hang over the end of a buffer lies in the last slab (the last row of k of an
+               MN-contiguous operand, the end of the last row of a K-contiguous one): only the loads of the last
+               slabs (mayHangOver) look for it.
+               Rows of k past the end of an MN-contiguous matrix read as zero by themselves;
                a K-contiguous row would run on into the next row, so those lanes are sent
                out of range explicitly, and the halves of a piece that straddles K are set to zero
                (last slab only) */
@@ -203,7 +220,10 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 int off = aOff[s];
                 if (AKC && tail && k0 + aK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                ra[rg][s] = buffer_load_f16x8(ar, off);
+                if constexpr (mayHangOver)
+                    ra[rg][s] = buffer_load_f16x8_any(ar, off, aBytes);
+                else
+                    ra[rg][s] = buffer_load_f16x8(ar, off);
                 if constexpr (mayHangOver && AKC)
                     if (tail) {
 #pragma unroll
@@ -216,7 +236,10 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 int off = bOff[s];
                 if (BKC && tail && k0 + bK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                rb[rg][s] = buffer_load_f16x8(br, off);
+                if constexpr (mayHangOver)
+                    rb[rg][s] = buffer_load_f16x8_any(br, off, bBytes);
+                else
+                    rb[rg][s] = buffer_load_f16x8(br, off);
                 if constexpr (mayHangOver && BKC)
                     if (tail) {
 #pragma unroll
@@ -353,7 +376,8 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     const int nk = (K + BKT - 1) / BKT;
 
     /* One slab, number kt = SLOT mod RING: its fragments are in register set SLOT % 2 and came from LDS stage
-       SLOT % 2. FULL: slabs kt+1 .. kt+RING exist and are complete, so the slab is straight-line code. */
+       SLOT % 2. FULL: slabs kt+1 .. kt+RING exist, are complete and are followed by another, so the slab is
+       straight-line code with plain loads. */
     auto slab = [&](auto SLOT, auto FULL, int kt) {
         constexpr int slot = decltype(SLOT)::value;
         constexpr int set = slot & 1;
@@ -425,8 +449,8 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             }
         };
         int kt = 0;
-        /* straight-line turns: every slab they ask for is complete */
-        for (; kt + 2 * RING - 1 < nkFull; kt += RING)
+        /* straight-line turns: every slab they ask for is complete and is not the last one */
+        for (; kt + 2 * RING < nkFull; kt += RING)
             turn(turn, IntC<0>(), IntC<1>(), kt);
         for (; kt < nk; kt += RING)
             turn(turn, IntC<0>(), IntC<0>(), kt);
