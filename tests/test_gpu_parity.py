@@ -403,7 +403,10 @@ def test_half_rows_of_any_length_and_alignment(gpu, oracle, ta, tb, out_float):
     half. Sizes that need the 128 x 128 tile, ragged in every dimension; the last row and column of the result
     are checked on their own, since that is where a lost element would show."""
     torch = torch_()
-    for (M, N, K) in ((203, 301, 77), (131, 135, 259), (9, 7, 5), (1, 300, 1)):
+    # the two long ones run many turns of the straight-line loop (a ring of four slabs in registers between memory
+    # and LDS), with a ragged last slab after a complete one and with a last slab that is complete
+    for (M, N, K) in ((203, 301, 77), (131, 135, 259), (9, 7, 5), (1, 300, 1), (70, 67, 1003), (33, 141, 1056)):
+        os.environ["NTSAMD_TILE_CFG"] = "1" if K == 1056 else "0"
         a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((M, K), ta), 31)))
         b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((K, N), tb), 32)))
         bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((N,), 33)))
