@@ -78,7 +78,14 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     constexpr int KG = 4 * KPM;                            /* k per group of four MFMA steps */
     constexpr int ACCN = R16 ? 4 : 16;                     /* accumulator registers per block */
     constexpr int KK = BKT / KPM;         /* MFMA steps per slab */
-    constexpr int LDK = BKT + 4;          /* row pitch of a K-contiguous operand in LDS */
+    /* K-contiguous operand in LDS. Slab of 32: rows BKT + 4 floats apart. Slab of 16: rows of 64 bytes with no
+       padding, four to a 256-byte line of the 64 banks, and the four 16-byte pieces of row r stored permuted,
+       piece u at position u ^ ((r >> 2) & 3): rows r, r+4, r+8, r+12 share their 64 bytes of the line, and both the
+       sixteen lanes that write four rows and the sixteen that read one piece of sixteen rows cover the whole line
+       (the 80-byte pitch this replaces made the writes of a fourth row wrap into the first: 17 % of the LDS
+       cycles were bank conflicts) */
+    constexpr bool SWZ = BKT == 16;
+    constexpr int LDK = SWZ ? BKT : BKT + 4;
     constexpr int NA = BM * BKT / 4 / NT;
     constexpr int NB = BN * BKT / 4 / NT;
     constexpr int ASIZE = AKC ? BM * LDK : BKT * BM;
@@ -125,7 +132,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             int row = g / (BKT / 4);
             aK[s] = (g % (BKT / 4)) * 4;
             aMN[s] = row;
-            aLds[s] = row * LDK + aK[s];
+            aLds[s] = SWZ ? row * LDK + (((aK[s] >> 2) ^ ((row >> 2) & 3)) << 2) : row * LDK + aK[s];
             int r = m0 + row < M - 1 ? row : M - 1 - m0;        /* rows past the edge repeat the last one */
             aOff[s] = (r * p.lda + aK[s]) * 4;
         }
@@ -146,7 +153,7 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             int row = g / (BKT / 4);
             bK[s] = (g % (BKT / 4)) * 4;
             bMN[s] = row;
-            bLds[s] = row * LDK + bK[s];
+            bLds[s] = SWZ ? row * LDK + (((bK[s] >> 2) ^ ((row >> 2) & 3)) << 2) : row * LDK + bK[s];
             int r = n0 + row < N - 1 ? row : N - 1 - n0;
             bOff[s] = (r * p.ldb + bK[s]) * 4;
         }
@@ -281,12 +288,13 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     auto read_frags = [&](auto SET, int buf) {
         constexpr int set = decltype(SET)::value;
         if constexpr (AKC) {
-            const float * as = &As[buf][(wm0 + l32) * LDK + 4 * lh];
+            const float * as = &As[buf][(wm0 + l32) * LDK + (SWZ ? 0 : 4 * lh)];
 #pragma unroll
             for (int q = 0; q < KK / 4; q++)
 #pragma unroll
                 for (int i = 0; i < TI; i++)
-                    fa4[set][q][i] = *reinterpret_cast<const f32x4 *>(as + i * 32 * LDK + KG * q);
+                    fa4[set][q][i] = *reinterpret_cast<const f32x4 *>(
+                        as + i * 32 * LDK + (SWZ ? (((lh + (KG / 4) * q) ^ ((l32 >> 2) & 3)) << 2) : KG * q));
         }
         else {
             const float * as = &As[buf][4 * lh * BM + wm0 + l32];
@@ -297,12 +305,13 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                     fa1[set][t][i] = as[(KG * (t / 4) + (t % 4)) * BM + i * 32];
         }
         if constexpr (BKC) {
-            const float * bs = &Bs[buf][(wn0 + l32) * LDK + 4 * lh];
+            const float * bs = &Bs[buf][(wn0 + l32) * LDK + (SWZ ? 0 : 4 * lh)];
 #pragma unroll
             for (int q = 0; q < KK / 4; q++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
-                    fb4[set][q][j] = *reinterpret_cast<const f32x4 *>(bs + j * BS * LDK + KG * q);
+                    fb4[set][q][j] = *reinterpret_cast<const f32x4 *>(
+                        bs + j * BS * LDK + (SWZ ? (((lh + (KG / 4) * q) ^ ((l32 >> 2) & 3)) << 2) : KG * q));
         }
         else {
             const float * bs = &Bs[buf][4 * lh * BN + wn0 + l32];
