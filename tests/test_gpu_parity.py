@@ -258,6 +258,34 @@ def test_batches_of_half_products_cut_along_k(gpu, oracle):
             assert_fp16(got[:, i * between:i * between + N], ref, what="item %d turn %d" % (i, turn))
 
 
+def test_half_products_cut_along_k_on_two_streams(gpu, oracle):
+    """The partial products of a cut product live in a workspace that belongs to the stream: two streams that run
+    such products at the same time must not see each other's. The sums are added in a fixed order, so each result
+    must equal, bit for bit, what the same product gives on its own."""
+    torch = torch_()
+    os.environ["NTSAMD_TILE_CFG"] = "1"
+    os.environ["NTSAMD_SPLIT_K"] = "8"
+    M, N, K = 64, 512, 4096
+    ops = []
+    for i in range(2):
+        a = dev_tensor(oracle.normal((M, K), 8500 + i, 0, 0.5), gpu, True)
+        b = dev_tensor(oracle.normal((K, N), 8510 + i, 0, 0.5), gpu, True)
+        alone = torch.empty((M, N), device=gpu, dtype=torch.float16)
+        nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, alone)
+        ops.append((a, b, alone, torch.empty_like(alone)))
+    torch.cuda.synchronize()
+    ref = oracle.matmul2d(ops[0][0].float().cpu().numpy(), X_NOTRANS, ops[0][1].float().cpu().numpy(), X_NOTRANS)
+    assert_fp16(ops[0][2].float().cpu().numpy(), ref, what="alone")
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for turn in range(30):
+        for (a, b, alone, c), st in zip(ops, streams):
+            with torch.cuda.stream(st):
+                nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c)
+    torch.cuda.synchronize()
+    for i, (a, b, alone, c) in enumerate(ops):
+        assert torch.equal(c, alone), "stream %d" % i
+
+
 def test_fp16_bits_match_the_oracle_conversion(gpu, oracle):
     """Small integers: every product and sum is exact in fp32 and representable in half,
     so the half result must equal the oracle's result bit for bit (RNE store)."""
