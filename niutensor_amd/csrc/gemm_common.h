@@ -121,7 +121,8 @@ __device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
 }
 
 /* tile shapes the dispatcher can pick from */
-enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_256x256 = 2, CFG_32x128 = 3, CFG_COUNT = 4 };
+/* CFG_16x128 (float): the 32 x 128 tile's kernel on 16-row MFMAs, one workgroup per 16 rows of c */
+enum TileCfg { CFG_128x128 = 0, CFG_64x64 = 1, CFG_256x256 = 2, CFG_32x128 = 3, CFG_16x128 = 4, CFG_COUNT = 5 };
 
 /* BM x BN tile per workgroup of WGM x WGN waves; BKT32: slab depth of the fp32 kernel
    (small tiles serve small, latency-bound products: a deeper slab means fewer round trips

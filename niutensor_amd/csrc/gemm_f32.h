@@ -113,7 +113,8 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     }
 
     const int M = p.M, N = p.N, K = p.K;
-    const int m0 = tc.tm * BM, n0 = tc.tn * BN;
+    /* R16: a workgroup multiplies the first 16 rows of what it stages, and the workgroups stand 16 rows apart */
+    const int m0 = tc.tm * (R16 ? 16 : BM), n0 = tc.tn * BN;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
@@ -573,7 +574,7 @@ static int launch_f32_one(const GemmParams & p0, const PT & tab, hipStream_t str
 {
     typedef TileShape<CFG> S;
     GemmParams p = p0;
-    p.tilesM = (p.M + S::BM - 1) / S::BM;
+    p.tilesM = R16 ? (p.M + 15) / 16 : (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
     if (p.splits < 1 || !VEC)
         p.splits = 1;
@@ -605,10 +606,11 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
     }
     if (cfg == CFG_128x128)
         return launch_f32_one<CFG_128x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
-    if (cfg == CFG_32x128) {
-        /* at most 16 rows: 16-row MFMAs on the same tile (NTSAMD_F32_R16=0 keeps the 32-row ones: for measurements) */
+    if (cfg == CFG_32x128 || cfg == CFG_16x128) {
+        /* at most 16 rows, or 16 rows per workgroup asked for: 16-row MFMAs on the same tile (NTSAMD_F32_R16=0
+           keeps the 32-row ones for products of at most 16 rows: for measurements) */
         const char * e = getenv("NTSAMD_F32_R16");
-        if (p.M <= 16 && !(e && e[0] == '0'))
+        if (cfg == CFG_16x128 || (p.M <= 16 && !(e && e[0] == '0')))
             return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs, true>(p, none, stream);
         return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
     }

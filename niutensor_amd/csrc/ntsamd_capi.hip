@@ -159,10 +159,12 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     const bool big = bm >= 128;
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
     const long long rounds = (groups + 255) / 256;
-    const double rate = big ? 1.0 : (rounds > 1 ? 0.965 : 0.89);
+    /* 16 rows per workgroup: every workgroup stages 128 columns of b for 16 rows of c, twice what the others move
+       per MFMA (measured: 0.7 of the rate, and a longer start) */
+    const double rate = big ? 1.0 : (bm == 16 ? 0.7 : (rounds > 1 ? 0.965 : 0.89));
     /* the 32-row tile multiplies only 16 rows when there are no more (16-row MFMAs) */
     const double mfma = (double)(bm == 32 && M <= 16 ? 16 : bm) * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
-    const double ends = (big ? 4.0 : 1.5) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
+    const double ends = (big ? 4.0 : (bm == 16 ? 2.5 : 1.5)) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
     const double cBytes = 4.0 * M * N * count;
     const double cut = splits > 1 ? cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0) : 0.0;
     return (double)rounds * mfma + ends + cut;
@@ -253,19 +255,20 @@ float * split_work_for(int devID, hipStream_t stream)
 }
 
 /* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
-   estimated run time. NTSAMD_TILE_CFG=0|1|2|3 forces a shape (128x128, 64x64, 256x256 for
-   half, 32x128 for float) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
-Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass, double cutExtra = 0.0)
+   estimated run time. NTSAMD_TILE_CFG=0|1|2|3|4 forces a shape (128x128, 64x64, 256x256 for
+   half, 32x128 and 16x128 for float) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
+Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass, double cutExtra = 0.0,
+                 bool fast32 = false)
 {
-    static const int bms[CFG_COUNT] = {128, 64, 256, 32};
-    static const int bns[CFG_COUNT] = {128, 64, 256, 128};
+    static const int bms[CFG_COUNT] = {128, 64, 256, 32, 16};
+    static const int bns[CFG_COUNT] = {128, 64, 256, 128, 128};
     int forcedCfg = -1, forcedSplits = -1;
     const char * e = getenv("NTSAMD_TILE_CFG");
     if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
         forcedCfg = e[0] - '0';
         if (forcedCfg == CFG_256x256 && !half)
             forcedCfg = CFG_128x128;
-        if (forcedCfg == CFG_32x128 && half)
+        if ((forcedCfg == CFG_32x128 || forcedCfg == CFG_16x128) && half)
             forcedCfg = CFG_64x64;
     }
     e = getenv("NTSAMD_SPLIT_K");
@@ -282,7 +285,8 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
     if (turn == 1)
         forcedSplits = 1;
     for (int cfg = 0; cfg < CFG_COUNT; cfg++) {
-        if ((cfg == CFG_256x256 && !half) || (cfg == CFG_32x128 && (half || M > 32)) || (forcedCfg >= 0 && cfg != forcedCfg))
+        if ((cfg == CFG_256x256 && !half) || (cfg == CFG_32x128 && (half || M > 32)) ||
+            (cfg == CFG_16x128 && (half || !fast32 || M <= 16)) || (forcedCfg >= 0 && cfg != forcedCfg))
             continue;
         for (int splits = 1; splits <= 16; splits *= 2) {
             if (splits > 1 && (!maySplit || K / splits < 64))
@@ -337,7 +341,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
 
     /* the kernels number their workgroups with 32-bit integers: the finest tiling of the largest batch,
        with k cut into the most pieces, must fit */
-    if ((long long)((s.M + 31) / 32) * ((s.N + 63) / 64) * count * 16 > 0x7fffffffLL)
+    if ((long long)((s.M + 15) / 16) * ((s.N + 63) / 64) * count * 16 > 0x7fffffffLL)
         return fail(NTSAMD_ERR_ARGUMENT, "the product has too many tiles for one launch (%d x %d x %d matrices)",
                     s.M, s.N, count);
 
@@ -403,7 +407,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
        b read once more) */
     const bool colSumAside = half && colSum != NULL && vec && count == 1;
     const double cutExtra = colSumAside ? 2.3 + 2.0 * s.K * s.N / 4.0e6 : 0.0;
-    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, cutExtra);
+    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, cutExtra,
+                            kind == KIND_F32 && vec && !ptrs && colSum == NULL);
     if (half && plan.splits > 1) {
         p.splitWork = split_work_for(devID, hs);
         if (p.splitWork == NULL)

@@ -162,7 +162,8 @@ SHAPES = [(1, 1, 1), (5, 7, 3), (37, 29, 53), (64, 64, 16), (63, 65, 17), (127, 
 @pytest.mark.parametrize("ta,tb", TRANS)
 def test_fp32_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
-    for cfg in ("0", "1", "3"):                          # 128 x 128, 64 x 64, 32 x 128 (at most 32 rows; else the rule's choice)
+    # 128 x 128, 64 x 64, 32 x 128 (at most 32 rows; else the rule's choice), 16 rows per workgroup on the same kernel
+    for cfg in ("0", "1", "3", "4"):
         os.environ["NTSAMD_TILE_CFG"] = cfg
         for i, (M, N, K) in enumerate(SHAPES):
             a = oracle.uniform(stored((M, K), ta), 1000 + i)
