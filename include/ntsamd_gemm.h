@@ -31,13 +31,21 @@
  * on `stream` (NULL = the default stream, which is what the reference uses)
  * without synchronising. Its only state beyond a per-device flag, and the only
  * device memory it allocates, is a 32 MiB workspace per device and stream for
- * half products with few tiles and a long k, which are cut along k (partial
- * products in fp32, added up by a second kernel): allocated at the first such
- * product on that stream, kept until the process ends. Launches on one stream
- * share it; kernels recorded into a graph keep the workspace of the stream
- * they were captured on, so graphs captured on one stream and that stream's
- * own launches must not run concurrently. NTSAMD_SPLIT_K=1 in the environment
- * keeps every product in one piece and the library from allocating.
+ * products with few tiles and a long k, which are cut along k (partial
+ * products in fp32, added up in a fixed order by a second kernel, so results
+ * are the same bits on every run): allocated at the first such product on that
+ * stream, kept until ntsamd_release_workspaces or the end of the process.
+ *
+ * Threads and streams: every entry point may be called from any host thread.
+ * Calls that use a workspace hold its lock from before their first launch
+ * until after their last, so two host threads that issue to ONE stream (every
+ * caller of the NULL stream does) get their kernels queued call by call and
+ * cannot read each other's partial products. Launches on different streams
+ * have different workspaces. Kernels recorded into a graph keep the workspace
+ * of the stream they were captured on, so graphs captured on one stream and
+ * that stream's own launches must not run concurrently. NTSAMD_SPLIT_K=1 in
+ * the environment (read once, at the library's first call) keeps every product
+ * in one piece and the library from allocating.
  */
 #ifndef NTSAMD_GEMM_H
 #define NTSAMD_GEMM_H
@@ -276,6 +284,14 @@ int ntsamd_attention_probs(int devID, void * stream,
  */
 int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS, void * t, int typeT,
                              long long size);
+
+/*
+ * Frees the workspaces the library allocated on `devID` (every device if devID < 0): one of 32 MiB per stream on
+ * which a product was ever cut along k. Waits for the device's work first; the next product that wants a
+ * workspace allocates it again. Has no counterpart among the reference's cuBLAS calls (cuBLAS keeps its own
+ * workspace inside the handle, released by cublasDestroy, which the reference never calls: XDevice.cpp:100-108).
+ */
+int ntsamd_release_workspaces(int devID);
 
 #ifdef __cplusplus
 }

@@ -34,6 +34,7 @@ EXPORTS = (
     "ntsamd_attention",
     "ntsamd_attention_probs",
     "ntsamd_convert_data_type",
+    "ntsamd_release_workspaces",
 )
 
 
@@ -76,6 +77,10 @@ def load():
     L.ntsamd_attention.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     L.ntsamd_attention_probs.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     L.ntsamd_convert_data_type.argtypes = [ci, vp, vp, ci, vp, ci, ll]
+    L.ntsamd_release_workspaces.argtypes = [ci]
+    # measurement knobs: exported, but no part of the interface include/ntsamd_gemm.h documents
+    L.ntsamd_tuning_set.argtypes = [C.c_char_p, ci]
+    L.ntsamd_tuning_set.restype = ci
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
     _lib = L
@@ -128,6 +133,18 @@ def matrix_mul(a, transA, b, transB, c, alpha=1.0, beta=0.0, bias=None, bias_mod
                                           bias.data_ptr(), bias_mode, bias.numel(), bias_row_div, act)
     _check(rc)
     return c
+
+
+def release_workspaces(device=-1):
+    """Free the workspaces of products cut along k (every device if device < 0)."""
+    _check(load().ntsamd_release_workspaces(device))
+
+
+def tuning_set(name, value):
+    """Set a measurement knob ("NTSAMD_TILE_CFG", "NTSAMD_SPLIT_K", ...) in the running library; None or a negative
+    value hands the decision back to the library. For tests and measurements only."""
+    v = -1 if value is None else int(value)
+    _check(load().ntsamd_tuning_set(name.encode(), v))
 
 
 def matrix_mul_batched_strided(a, transA, b, transB, c, count, strideA, strideB, strideC,

@@ -67,13 +67,15 @@ struct GemmParams {
     void * colSum;
     float colSumBeta;
     /* The k range is cut into `splits` pieces of kPerSplit (a multiple of every slab depth), one workgroup
-       each; 1 = one workgroup per tile, plain stores. fp32: the pieces ADD alpha * (their partial product) to
-       c with atomics, the caller has already applied beta to c. fp16 (16-byte path, 64 x 64 and 128 x 128
-       tiles): the pieces go to splitWork (splits x batch dense M x N fp32 matrices) as plain products, and
-       launch_split_reduce adds them up and writes c. */
+       each; 1 = one workgroup per tile, plain stores. The pieces go to splitWork (splits x batch dense M x N
+       fp32 matrices) as plain products, and launch_split_reduce adds them up in their order and writes c
+       (fp16: 16-byte path, 64 x 64 and 128 x 128 tiles). fp32 with splitWork == NULL: the pieces ADD alpha *
+       (their partial product) to c with atomics, in no fixed order, and the caller has already applied beta
+       to c. */
     int splits, kPerSplit;
     float * splitWork;
     int act;                               /* Activation of the epilogue */
+    int wideRowsOnly;                      /* fp32, measurements: no 16-row MFMAs for products of at most 16 rows */
 };
 
 /* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and

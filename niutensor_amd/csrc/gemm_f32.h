@@ -33,7 +33,6 @@
  */
 #pragma once
 #include "gemm_common.h"
-#include <stdlib.h>
 #include <type_traits>
 
 namespace ntsamd {
@@ -475,8 +474,29 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
                 }
             }
         }
+        if (p.splits > 1 && p.splitWork != NULL) {
+            /* one of several workgroups that share this tile, and a workspace for them to meet in: the partial
+               tile goes there as it is (splits x batch dense M x N matrices), and split_reduce.hip adds the pieces
+               in their order, the same bits on every run, and applies alpha, beta, bias and activation */
+            float * w = p.splitWork + ((size_t)tc.split * p.batch + tc.batch) * M * N;
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const int col = n0 + wn0 + j * BS + l32;
+                if (col < N) {
+#pragma unroll
+                    for (int i = 0; i < TI; i++)
+#pragma unroll
+                        for (int r = 0; r < ACCN; r++) {
+                            const int row = m0 + wm0 + i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4)) + 4 * lh;
+                            if (row < M)
+                                w[(size_t)row * N + col] = acc[i][j][r];
+                        }
+                }
+            }
+            return;
+        }
         if (p.splits > 1) {
-            /* one of several workgroups that share this tile: add the partial product to c,
+            /* no workspace: add the partial product to c,
                which already holds beta * c; the bias rides on the first piece. Every add is
                predicated on its own row and column: an atomic must never be issued out of range
                (loads and stores past the end of a buffer are dropped by the hardware; this path
@@ -607,10 +627,9 @@ static int launch_f32_trans(const GemmParams & p, const PtrBatch * ptrs, bool ve
     if (cfg == CFG_128x128)
         return launch_f32_one<CFG_128x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
     if (cfg == CFG_32x128 || cfg == CFG_16x128) {
-        /* at most 16 rows, or 16 rows per workgroup asked for: 16-row MFMAs on the same tile (NTSAMD_F32_R16=0
+        /* at most 16 rows, or 16 rows per workgroup asked for: 16-row MFMAs on the same tile (p.wideRowsOnly
            keeps the 32-row ones for products of at most 16 rows: for measurements) */
-        const char * e = getenv("NTSAMD_F32_R16");
-        if (cfg == CFG_16x128 || (p.M <= 16 && !(e && e[0] == '0')))
+        if (cfg == CFG_16x128 || (p.M <= 16 && !p.wideRowsOnly))
             return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs, true>(p, none, stream);
         return launch_f32_one<CFG_32x128, AKC, BKC, true, false, NoPtrs>(p, none, stream);
     }

@@ -12,6 +12,7 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -27,7 +28,8 @@ int launch_f16_nt(const GemmParams &, const PtrBatch *, int, bool, int, hipStrea
 int launch_f16_tn(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
 int launch_f16_tt(const GemmParams &, const PtrBatch *, int, bool, int, hipStream_t);
 int launch_scale(bool half, void * v, long long n, float beta, hipStream_t stream);
-int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream);
+int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream,
+                         float * work, size_t workFloats);
 int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream);
 }
 
@@ -151,10 +153,14 @@ bool aligned16(const void * p)
    workgroup's MFMAs take tile area x k x 3.48e-6 us on a 128 x 128 tile; the 64 x 64 tile (one accumulator
    block per wave: a dependent chain) runs at 0.89 of that rate alone on its CU and at 0.965 with company. What
    a workgroup spends before its first and after its last MFMA (4 us; 1.5 us for the small tile) is exposed
-   once and partly hidden behind the other workgroups of the CU after that. Cutting k moves c once more per piece
-   (atomic adds, about 2.7 TB/s); unless beta is 1, a pass over c applies beta first: a launch (2.5 us) and c
+   once and partly hidden behind the other workgroups of the CU after that. Cutting k sends the fp32 partial
+   products across memory once (about 5 TB/s, much of it behind the multiplications) on their way to a second
+   launch (2.3 us) that adds them up in a fixed order. Without a workspace the pieces add to c with atomics
+   instead (about 2.7 TB/s) and, unless beta is 1, a pass over c applies beta first: a launch (2.5 us) and c
    read and written. */
-double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits, bool betaPass)
+constexpr double SPLIT_FIXED_US = 2.3, SPLIT_BYTES_PER_US = 5.0e6;
+
+double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits, bool betaPass, bool viaWork)
 {
     const bool big = bm >= 128;
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
@@ -166,7 +172,11 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     const double mfma = (double)(bm == 32 && M <= 16 ? 16 : bm) * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
     const double ends = (big ? 4.0 : (bm == 16 ? 2.5 : 1.5)) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
     const double cBytes = 4.0 * M * N * count;
-    const double cut = splits > 1 ? cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0) : 0.0;
+    double cut = 0.0;
+    if (splits > 1 && viaWork)
+        cut = SPLIT_FIXED_US + 2.0 * cBytes * splits / SPLIT_BYTES_PER_US;
+    else if (splits > 1)
+        cut = cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0);
     return (double)rounds * mfma + ends + cut;
 }
 
@@ -183,14 +193,13 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
    Cutting k into pieces (few tiles, long k: weight gradients, the few rows of a decoding step) makes as many
    products of a shorter k, whose fp32 results cross memory once (about 5 TB/s, much of it behind the
    multiplications) on their way to a second launch (2.3 us) that adds them up. */
-constexpr double SPLIT16_FIXED_US = 2.3, SPLIT16_BYTES_PER_US = 5.0e6;
 
 double tile_cost_f16(int M, int N, int K, int count, int bm, int splits)
 {
     if (splits > 1) {
         const int kPiece = ((K + splits - 1) / splits + 31) / 32 * 32;
-        return tile_cost_f16(M, N, kPiece, count * splits, bm, 1) + SPLIT16_FIXED_US +
-               8.0 * M * N * count * splits / SPLIT16_BYTES_PER_US;
+        return tile_cost_f16(M, N, kPiece, count * splits, bm, 1) + SPLIT_FIXED_US +
+               8.0 * M * N * count * splits / SPLIT_BYTES_PER_US;
     }
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bm - 1) / bm) * count;
     const long long rounds = (groups + 255) / 256;
@@ -218,62 +227,131 @@ struct Plan {
     int splits;
 };
 
-/* Where the pieces of a half product whose k is cut meet: one workspace per device and stream (launches on one
-   stream run one after the other, so they can share; launches on different streams may overlap, so they must
-   not), allocated at the first product that wants it and kept until the process ends. A kernel recorded into a
-   graph keeps the workspace of the stream it was captured on: graphs captured on one stream, and that stream's
-   own launches, must not run at the same time. */
-constexpr size_t SPLIT_WORK_BYTES = (size_t)32 << 20;
-constexpr size_t SPLIT_STREAMS_MAX = 64;            /* per process, over all devices */
-std::mutex g_splitMutex;
-std::map<std::pair<int, hipStream_t>, float *> g_splitWork;
+/* Knobs for measurements and tests, none of them part of the documented interface: the environment is read ONCE,
+   at the first call that looks (never again on the way to a launch), and ntsamd_tuning_set changes a knob in a
+   running process. -1 = the library decides.
+     NTSAMD_TILE_CFG=0|1|2|3|4   force a tile shape (128x128, 64x64, 256x256 for half, 32x128 and 16x128 for float)
+     NTSAMD_SPLIT_K=n            force the number of pieces k is cut into (1 = never cut, and never a workspace)
+     NTSAMD_F16_FETCH=0|2        keep half products off the main path (element-wise / register-staged fetch)
+     NTSAMD_ATTN_ROWS=0          keep attention with a handful of query rows on the MFMA kernels
+     NTSAMD_F32_R16=0            no 16-row MFMAs for float products of at most 16 rows
+     NTSAMD_F32_SPLIT_ATOMIC=1   float pieces of k add to c with atomics (no workspace, no fixed order) */
+struct Tuning {
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic;
+};
+Tuning g_tuning;
+std::once_flag g_tuningOnce;
 
-/* NULL: none to be had (no memory, too many streams) and the product runs in one piece. Device devID is current. */
-float * split_work_for(int devID, hipStream_t stream)
+struct Knob {
+    const char * name;
+    std::atomic<int> Tuning::* field;
+};
+const Knob g_knobs[] = {
+    {"NTSAMD_TILE_CFG", &Tuning::tileCfg},   {"NTSAMD_SPLIT_K", &Tuning::splitK},
+    {"NTSAMD_F16_FETCH", &Tuning::f16Fetch}, {"NTSAMD_ATTN_ROWS", &Tuning::attnRows},
+    {"NTSAMD_F32_R16", &Tuning::f32R16},     {"NTSAMD_F32_SPLIT_ATOMIC", &Tuning::f32SplitAtomic},
+};
+
+const Tuning & tuning()
 {
-    std::lock_guard<std::mutex> lock(g_splitMutex);
-    const std::pair<int, hipStream_t> key(devID, stream);
-    std::map<std::pair<int, hipStream_t>, float *>::iterator it = g_splitWork.find(key);
-    if (it != g_splitWork.end())
-        return it->second;
-    if (g_splitWork.size() >= SPLIT_STREAMS_MAX)
-        return NULL;
-    /* the stream may be recording a graph: allocating is allowed then only in the relaxed mode, which is how
-       allocators that serve captures do it; the allocation itself is no part of the graph */
-    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
-    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
-    void * mem = NULL;
-    const hipError_t err = hipMalloc(&mem, SPLIT_WORK_BYTES);
-    if (exchanged)
-        (void)hipThreadExchangeStreamCaptureMode(&mode);
-    if (err != hipSuccess || mem == NULL) {
-        (void)hipGetLastError();
-        return NULL;
-    }
-    g_splitWork[key] = static_cast<float *>(mem);
-    return static_cast<float *>(mem);
+    std::call_once(g_tuningOnce, [] {
+        for (const Knob & k : g_knobs) {
+            const char * e = getenv(k.name);
+            (g_tuning.*(k.field)).store(e && e[0] >= '0' && e[0] <= '9' ? atoi(e) : -1, std::memory_order_relaxed);
+        }
+    });
+    return g_tuning;
 }
 
-/* The tile shape and (fp32, 16-byte path only) the number of k pieces with the lowest
-   estimated run time. NTSAMD_TILE_CFG=0|1|2|3|4 forces a shape (128x128, 64x64, 256x256 for
-   half, 32x128 and 16x128 for float) and NTSAMD_SPLIT_K=n a number of pieces (1 = never split): for measurements. */
-Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass, double cutExtra = 0.0,
-                 bool fast32 = false)
+/* Where the pieces of a product whose k is cut meet: one workspace per device and stream (launches on one
+   stream run one after the other, so they can share; launches on different streams may overlap, so they must
+   not), allocated at the first product that wants it and kept until ntsamd_release_workspaces or the end of the
+   process. A call holds its workspace's mutex from before its first launch until after its last: two host
+   threads that issue to one stream (every caller of the NULL stream does) cannot interleave their product and
+   summing kernels. A kernel recorded into a graph keeps the workspace of the stream it was captured on: graphs
+   captured on one stream, and that stream's own launches, must not run at the same time. */
+constexpr size_t SPLIT_WORK_BYTES = (size_t)32 << 20;
+constexpr int SPLIT_STREAMS_MAX = 64;               /* workspaces alive per process, over all devices */
+struct SplitWork {
+    float * mem;
+    std::mutex inUse;
+};
+std::mutex g_splitMutex;                            /* guards the map, not the workspaces */
+std::map<std::pair<int, hipStream_t>, SplitWork *> g_splitWork;   /* entries are never removed */
+std::atomic<int> g_splitAlive;
+
+/* A workspace held for the launches of one call; released when the call returns. */
+struct WorkHold {
+    float * mem;
+    size_t bytes;
+    std::mutex * held;
+    WorkHold() : mem(NULL), bytes(0), held(NULL) {}
+    ~WorkHold()
+    {
+        if (held)
+            held->unlock();
+    }
+    /* the workspace of (devID, stream), allocated now if need be; mem stays NULL if there is none to be had (no
+       memory, too many streams): the product then runs in one piece. Device devID is current. */
+    void take_stream(int devID, hipStream_t stream)
+    {
+        if (mem != NULL)
+            return;
+        SplitWork * w;
+        {
+            std::lock_guard<std::mutex> lock(g_splitMutex);
+            SplitWork *& slot = g_splitWork[std::make_pair(devID, stream)];
+            if (slot == NULL) {
+                slot = new SplitWork;
+                slot->mem = NULL;
+            }
+            w = slot;
+        }
+        w->inUse.lock();
+        if (w->mem == NULL && g_splitAlive.load() < SPLIT_STREAMS_MAX) {
+            /* the stream may be recording a graph: allocating is allowed then only in the relaxed mode, which is
+               how allocators that serve captures do it; the allocation itself is no part of the graph */
+            hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+            const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+            void * got = NULL;
+            const hipError_t err = hipMalloc(&got, SPLIT_WORK_BYTES);
+            if (exchanged)
+                (void)hipThreadExchangeStreamCaptureMode(&mode);
+            if (err == hipSuccess && got != NULL) {
+                w->mem = static_cast<float *>(got);
+                g_splitAlive.fetch_add(1);
+            }
+            else
+                (void)hipGetLastError();
+        }
+        if (w->mem == NULL) {
+            w->inUse.unlock();
+            return;
+        }
+        mem = w->mem;
+        bytes = SPLIT_WORK_BYTES;
+        held = &w->inUse;
+    }
+};
+
+/* The tile shape and the number of k pieces with the lowest estimated run time. workBytes: what the partial
+   products of a cut k may take (0: no limit, the float pieces add to c with atomics). forcedSplits >= 1: that many
+   pieces or, where no shape can take them, one; otherwise the NTSAMD_SPLIT_K knob, otherwise the estimate. */
+Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool betaPass, size_t workBytes,
+                 double cutExtra = 0.0, bool fast32 = false, int forcedSplits = -1)
 {
     static const int bms[CFG_COUNT] = {128, 64, 256, 32, 16};
     static const int bns[CFG_COUNT] = {128, 64, 256, 128, 128};
-    int forcedCfg = -1, forcedSplits = -1;
-    const char * e = getenv("NTSAMD_TILE_CFG");
-    if (e && e[0] >= '0' && e[0] < '0' + CFG_COUNT && e[1] == 0) {
-        forcedCfg = e[0] - '0';
-        if (forcedCfg == CFG_256x256 && !half)
-            forcedCfg = CFG_128x128;
-        if ((forcedCfg == CFG_32x128 || forcedCfg == CFG_16x128) && half)
-            forcedCfg = CFG_64x64;
-    }
-    e = getenv("NTSAMD_SPLIT_K");
-    if (e && atoi(e) >= 1)
-        forcedSplits = atoi(e);
+    const Tuning & tn = tuning();
+    int forcedCfg = tn.tileCfg.load(std::memory_order_relaxed);
+    if (forcedCfg < 0 || forcedCfg >= CFG_COUNT)
+        forcedCfg = -1;
+    if (forcedCfg == CFG_256x256 && !half)
+        forcedCfg = CFG_128x128;
+    if ((forcedCfg == CFG_32x128 || forcedCfg == CFG_16x128) && half)
+        forcedCfg = CFG_64x64;
+    if (forcedSplits < 1)
+        forcedSplits = tn.splitK.load(std::memory_order_relaxed);
     if (forcedSplits != 1 && forcedSplits != 2 && forcedSplits != 4 && forcedSplits != 8 && forcedSplits != 16)
         forcedSplits = -1;
     if (forcedSplits > 1 && (!maySplit || K / forcedSplits < 64))
@@ -291,16 +369,16 @@ Plan choose_plan(int M, int N, int K, int count, bool half, bool maySplit, bool 
         for (int splits = 1; splits <= 16; splits *= 2) {
             if (splits > 1 && (!maySplit || K / splits < 64))
                 break;
-            if (splits > 1 && half) {
-                /* the big tile has no such kernel; the partial products must fit the workspace */
-                if (cfg == CFG_256x256 || K / splits < 128 ||
-                    (long long)M * N * count * splits * 4 > (long long)SPLIT_WORK_BYTES)
-                    break;
-            }
+            /* the partial products must fit the workspace */
+            if (splits > 1 && workBytes > 0 && (long long)M * N * count * splits * 4 > (long long)workBytes)
+                break;
+            /* half: the big tile has no such kernel */
+            if (splits > 1 && half && (cfg == CFG_256x256 || K / splits < 128))
+                break;
             if (forcedSplits >= 1 && splits != forcedSplits)
                 continue;
             double c = half ? tile_cost_f16(M, N, K, count, bms[cfg], splits)
-                            : tile_cost_f32(M, N, K, count, bms[cfg], bns[cfg], splits, betaPass);
+                            : tile_cost_f32(M, N, K, count, bms[cfg], bns[cfg], splits, betaPass, workBytes > 0);
             if (splits > 1)
                 c += cutExtra;
             if (bestCost < 0.0 || c < bestCost) {
@@ -345,6 +423,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         return fail(NTSAMD_ERR_ARGUMENT, "the product has too many tiles for one launch (%d x %d x %d matrices)",
                     s.M, s.N, count);
 
+    const Tuning & tn = tuning();
     GemmParams p;
     memset(&p, 0, sizeof(p));
     p.a = a;
@@ -368,6 +447,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.batch = count;
     p.groupM = 8;
     p.act = act;
+    p.wideRowsOnly = tn.f32R16.load(std::memory_order_relaxed) == 0;
     if (grid) {
         p.batchInner = grid->inner;
         p.strideA1 = grid->strideA1;
@@ -390,29 +470,35 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                             aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
                             (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
         fetch16 = direct ? F16_DIRECT : (vec ? F16_STAGED : F16_SCALAR);
-        const char * e = getenv("NTSAMD_F16_FETCH");              /* 0 or 2: keep off the main path (for measurements) */
-        if (e && e[1] == 0 && (e[0] == '0' || (e[0] == '2' && vec)))
-            fetch16 = e[0] - '0';
+        const int knob = tn.f16Fetch.load(std::memory_order_relaxed);   /* 0 or 2: keep off the main path */
+        if (knob == F16_SCALAR || (knob == F16_STAGED && vec))
+            fetch16 = knob;
         vec = fetch16 == F16_DIRECT;                               /* what the column-sum by-product needs */
     }
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
-    /* cutting k into pieces pays when the result has few tiles and k is long (weight
-       gradients); the pieces add to c with fp32 atomics, so c gets its beta first */
-    /* ... and for half products on the 16-byte path, whose pieces meet in a workspace and leave the ordinary way
-       (any beta, bias, activation, leading dimensions; no column sums) */
-    const bool maySplit = half ? fetch16 == F16_DIRECT && !ptrs
-                               : vec && !ptrs && act == ACT_NONE && dense;
-    /* the pieces of a half product gather no column sums: cutting costs a pass of its own over b then (a launch,
-       b read once more) */
-    const bool colSumAside = half && colSum != NULL && vec && count == 1;
-    const double cutExtra = colSumAside ? 2.3 + 2.0 * s.K * s.N / 4.0e6 : 0.0;
-    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, cutExtra,
-                            kind == KIND_F32 && vec && !ptrs && colSum == NULL);
-    if (half && plan.splits > 1) {
-        p.splitWork = split_work_for(devID, hs);
-        if (p.splitWork == NULL)
-            plan = choose_plan(s.M, s.N, s.K, count, half, false, beta != 1.f);
+    /* Cutting k into pieces pays when the result has few tiles and k is long (weight gradients, the few rows of a
+       decoding step). The pieces of a product on the 16-byte path meet in a workspace and leave the ordinary way
+       (any beta, bias, activation, leading dimensions; no column sums): the same bits on every run. Float pieces
+       can add to c with atomics instead (in no fixed order; dense results without activation only, and c gets
+       its beta first): only if the knob asks for it, or when there is no workspace to be had. */
+    const bool atomicAble = !half && vec && !ptrs && act == ACT_NONE && dense;
+    const bool atomicAsked = atomicAble && tn.f32SplitAtomic.load(std::memory_order_relaxed) > 0;
+    const bool maySplit = atomicAsked || ((half ? fetch16 == F16_DIRECT : vec) && !ptrs);
+    const size_t workBytes = atomicAsked ? 0 : SPLIT_WORK_BYTES;
+    /* pieces that meet in a workspace gather no column sums: cutting costs a pass of its own over b then (a
+       launch, b read once more) */
+    const bool colSumAside = colSum != NULL && vec && count == 1 && !atomicAsked;
+    const double cutExtra = colSumAside ? 2.3 + (half ? 2.0 : 4.0) * s.K * s.N / 4.0e6 : 0.0;
+    const bool fast32 = kind == KIND_F32 && vec && !ptrs && colSum == NULL;
+    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, workBytes, cutExtra, fast32);
+    WorkHold work;
+    bool viaWork = false;
+    if (plan.splits > 1 && !atomicAsked) {
+        work.take_stream(devID, hs);
+        viaWork = work.mem != NULL;
+        if (!viaWork && !atomicAble)
+            plan = choose_plan(s.M, s.N, s.K, count, half, false, beta != 1.f, 0, 0.0, fast32);
     }
     const int cfg = plan.cfg;
     int rc = 0;
@@ -420,9 +506,10 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     if (plan.splits > 1) {
         p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 31) / 32 * 32;
         p.splits = (s.K + p.kPerSplit - 1) / p.kPerSplit;
+        p.splitWork = viaWork ? work.mem : NULL;
     }
-    if (!half && p.splits > 1 && beta != 1.f) {
-        /* c is dense: count matrices of M x N, strideC apart */
+    if (p.splits > 1 && !viaWork && beta != 1.f) {
+        /* float pieces that add to c: c is dense, count matrices of M x N, strideC apart */
         if (count == 1 || strideC == (long long)s.M * s.N)
             rc = launch_scale(false, c, (long long)s.M * s.N * count, beta, hs);
         else
@@ -432,17 +519,20 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
     if (colSum != NULL) {
-        if (vec && count == 1 && !(half && plan.splits > 1)) {
+        if (vec && count == 1 && !(p.splits > 1 && viaWork)) {
             /* by-product of the product kernel */
             p.colSum = colSum;
             p.colSumBeta = colSumBeta;
-            if (!half && p.splits > 1)
+            if (p.splits > 1)
                 rc = launch_scale(false, colSum, s.N, colSumBeta, hs);
         }
         else {
-            /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS */
-            rc = s.bKContig ? launch_reduce_sum_xz(half, b, 1, s.N, s.K, colSum, colSumBeta, hs)
-                            : launch_reduce_sum_xz(half, b, s.K, s.N, 1, colSum, colSumBeta, hs);
+            /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS. It runs before the product
+               on the same stream, so the two can share the workspace. */
+            if (!half && !s.bKContig)
+                work.take_stream(devID, hs);
+            rc = s.bKContig ? launch_reduce_sum_xz(half, b, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
+                            : launch_reduce_sum_xz(half, b, s.K, s.N, 1, colSum, colSumBeta, hs, work.mem, work.bytes / 4);
         }
         if (rc != 0)
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -461,8 +551,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         else
             rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, cfg, hs);
     }
-    if (rc == 0 && half && p.splits > 1)
-        rc = launch_split_reduce(p, kind == KIND_F16_F32OUT, hs);
+    if (rc == 0 && p.splits > 1 && viaWork)
+        rc = launch_split_reduce(p, kind != KIND_F16, hs);
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;
@@ -497,7 +587,52 @@ int ntsamd_init(int devID)
     DeviceScope scope(devID);
     if (scope.status != NTSAMD_OK)
         return scope.status;
+    (void)tuning();
     return NTSAMD_OK;
+}
+
+int ntsamd_release_workspaces(int devID)
+{
+    if (devID >= MAX_DEVICES)
+        return fail(NTSAMD_ERR_DEVICE, "invalid device id %d", devID);
+    std::vector<std::pair<int, SplitWork *> > mine;
+    {
+        std::lock_guard<std::mutex> lock(g_splitMutex);
+        for (std::map<std::pair<int, hipStream_t>, SplitWork *>::iterator it = g_splitWork.begin();
+             it != g_splitWork.end(); ++it)
+            if (devID < 0 || it->first.first == devID)
+                mine.push_back(std::make_pair(it->first.first, it->second));
+    }
+    for (size_t i = 0; i < mine.size(); i++) {
+        SplitWork * w = mine[i].second;
+        std::lock_guard<std::mutex> lock(w->inUse);
+        if (w->mem == NULL)
+            continue;
+        DeviceScope scope(mine[i].first);
+        if (scope.status != NTSAMD_OK)
+            return scope.status;
+        /* hipFree waits for the device's work, the kernels that still use the workspace included */
+        const hipError_t err = hipFree(w->mem);
+        if (err != hipSuccess)
+            return fail(NTSAMD_ERR_DEVICE, "cannot free a workspace on device %d: %s", mine[i].first,
+                        hipGetErrorString(err));
+        w->mem = NULL;
+        g_splitAlive.fetch_sub(1);
+    }
+    return NTSAMD_OK;
+}
+
+int ntsamd_tuning_set(const char * name, int value)
+{
+    if (!name)
+        return fail(NTSAMD_ERR_ARGUMENT, "no knob named");
+    (void)tuning();                      /* the environment first, so that it cannot overwrite this later */
+    for (const Knob & k : g_knobs)
+        if (strcmp(name, k.name) == 0 || strcmp(name, k.name + 7) == 0) {
+            (g_tuning.*(k.field)).store(value < 0 ? -1 : value, std::memory_order_relaxed);
+            return NTSAMD_OK;
+        }
+    return fail(NTSAMD_ERR_ARGUMENT, "no knob named %s", name);
 }
 
 int ntsamd_matrix_mul_bias(int devID, void * stream,
@@ -581,8 +716,12 @@ int ntsamd_matrix_mul_colsum(int devID, void * stream,
         if (scope.status != NTSAMD_OK)
             return scope.status;
         hipStream_t hs = static_cast<hipStream_t>(stream);
-        int rc = s.bKContig ? launch_reduce_sum_xz(kind != KIND_F32, b, 1, s.N, s.K, colSum, colSumBeta, hs)
-                            : launch_reduce_sum_xz(kind != KIND_F32, b, s.K, s.N, 1, colSum, colSumBeta, hs);
+        WorkHold work;
+        if (kind == KIND_F32 && !s.bKContig && s.K >= 128)
+            work.take_stream(devID, hs);
+        int rc = s.bKContig ? launch_reduce_sum_xz(kind != KIND_F32, b, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
+                            : launch_reduce_sum_xz(kind != KIND_F32, b, s.K, s.N, 1, colSum, colSumBeta, hs,
+                                                   work.mem, work.bytes / 4);
         if (rc != 0)
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
         return NTSAMD_OK;
@@ -610,8 +749,12 @@ int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType
     DeviceScope scope(devID);
     if (scope.status != NTSAMD_OK)
         return scope.status;
+    /* float column sums over many rows are cut into pieces of the rows, which meet in the stream's workspace */
+    WorkHold work;
+    if (dataType == NTSAMD_X_FLOAT && z == 1 && x >= 128)
+        work.take_stream(devID, static_cast<hipStream_t>(stream));
     int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,
-                                  static_cast<hipStream_t>(stream));
+                                  static_cast<hipStream_t>(stream), work.mem, work.bytes / 4);
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;
@@ -714,12 +857,12 @@ int ntsamd_attention(int devID, void * stream,
     p.oH = strides[9]; p.oB = strides[10]; p.oL = strides[11];
     p.scale = scale;
     /* up to eight query rows per head (a decoding step) go to the kernel that reads k and v once and multiplies
-       in the vector ALU, as long as its scores fit in LDS; NTSAMD_ATTN_ROWS=0 keeps them on the MFMA kernels */
+       in the vector ALU, as long as its scores fit in LDS; the NTSAMD_ATTN_ROWS=0 knob keeps them on the MFMA
+       kernels */
     const bool halfType = dataType == NTSAMD_X_FLOAT16;
     const size_t rowsLds = attention_rows_lds(p, halfType);
-    const char * env = getenv("NTSAMD_ATTN_ROWS");
     int rc;
-    if (rowsLds > 0 && rowsLds <= 60 * 1024 && !(env && env[0] == '0'))
+    if (rowsLds > 0 && rowsLds <= 60 * 1024 && tuning().attnRows.load(std::memory_order_relaxed) != 0)
         rc = launch_attention_rows(p, halfType, static_cast<hipStream_t>(stream));
     else
         rc = halfType ? launch_attention_f16(p, static_cast<hipStream_t>(stream))

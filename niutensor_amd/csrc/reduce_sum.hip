@@ -8,7 +8,10 @@
  * produce the same column sums as a by-product when they can; these kernels
  * serve the shapes and layouts where they cannot. Also here: the scaling pass
  * that applies beta ahead of kernels that add to their result with atomics.
- * Memory-bound, fp32 accumulation for both data types.
+ * Memory-bound, fp32 accumulation for both data types. Float column sums over
+ * many rows are cut into pieces of the rows: with a workspace the pieces leave
+ * their sums there and split_reduce.hip adds them in their order (the same bits
+ * on every run); without one they add to the result with atomics.
  */
 #include "gemm_common.h"
 #include "gemm_f16.h"       /* half_t */
@@ -17,7 +20,9 @@ namespace ntsamd {
 
 /* Z == 1. A workgroup owns 64 columns and one piece of the rows: 16 threads side by side
    read 4 columns each (256 contiguous bytes of a row for fp32), 16 such rows per step. */
-template <typename T, bool ATOMIC>
+enum { SUM_WHOLE = 0, SUM_ATOMIC = 1, SUM_PIECE = 2 };   /* what a workgroup does with its sums */
+
+template <typename T, int MODE>
 __global__ void __launch_bounds__(256)
 column_sum_kernel(const T * __restrict__ in, int X, int Y, int rowsPerPiece, T * __restrict__ out, float beta)
 {
@@ -56,8 +61,10 @@ column_sum_kernel(const T * __restrict__ in, int X, int Y, int rowsPerPiece, T *
             v += part[r][threadIdx.x];
         const int col = blockIdx.x * 64 + threadIdx.x;
         if (col < Y) {
-            if constexpr (ATOMIC)
+            if constexpr (MODE == SUM_ATOMIC)
                 unsafeAtomicAdd(reinterpret_cast<float *>(out) + col, v);     /* beta already applied */
+            else if constexpr (MODE == SUM_PIECE)
+                reinterpret_cast<float *>(out)[(size_t)blockIdx.y * Y + col] = v;   /* out: pieces x Y partial sums */
             else
                 out[col] = (T)(beta != 0.f ? beta * (float)out[col] + v : v);
         }
@@ -110,7 +117,10 @@ int launch_scale(bool half, void * v, long long n, float beta, hipStream_t strea
     return (int)hipGetLastError();
 }
 
-int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream)
+/* work: NULL, or workFloats floats of device memory that this stream's launches may use until the call's last
+   kernel has run */
+int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream,
+                         float * work, size_t workFloats)
 {
     if (Y <= 0)
         return 0;
@@ -126,7 +136,7 @@ int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void *
     const int colGroups = (Y + 63) / 64;
     if (half) {
         /* one piece: half sums are rounded once, from the fp32 total */
-        hipLaunchKernelGGL((column_sum_kernel<half_t, false>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
+        hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_WHOLE>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
                            static_cast<const half_t *>(in), X, Y, X > 0 ? X : 1, static_cast<half_t *>(out), beta);
         return (int)hipGetLastError();
     }
@@ -135,16 +145,40 @@ int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void *
     if (pieces > (X + 63) / 64)
         pieces = (X + 63) / 64;
     if (pieces <= 1) {
-        hipLaunchKernelGGL((column_sum_kernel<float, false>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
+        hipLaunchKernelGGL((column_sum_kernel<float, SUM_WHOLE>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
                            static_cast<const float *>(in), X, Y, X > 0 ? X : 1, static_cast<float *>(out), beta);
         return (int)hipGetLastError();
+    }
+    if (work != NULL && (size_t)Y * 2 <= workFloats) {
+        /* the pieces meet in the workspace and are added in their order */
+        const int most = (size_t)Y * 16 <= workFloats ? 16 : (int)(workFloats / (size_t)Y);
+        if (pieces > most)
+            pieces = most;
+        const int rows = (X + pieces - 1) / pieces;
+        pieces = (X + rows - 1) / rows;
+        hipLaunchKernelGGL((column_sum_kernel<float, SUM_PIECE>), dim3((unsigned)colGroups, (unsigned)pieces), dim3(256), 0,
+                           stream, static_cast<const float *>(in), X, Y, rows, reinterpret_cast<float *>(work), 1.f);
+        int rc = (int)hipGetLastError();
+        if (rc != 0)
+            return rc;
+        GemmParams p = {};
+        p.c = out;
+        p.M = 1;
+        p.N = Y;
+        p.ldc = Y;
+        p.batch = 1;
+        p.alpha = 1.f;
+        p.beta = beta;
+        p.splits = pieces;
+        p.splitWork = work;
+        return launch_split_reduce(p, true, stream);
     }
     int rc = launch_scale(false, out, Y, beta, stream);
     if (rc != 0)
         return rc;
     const int rowsPerPiece = (X + pieces - 1) / pieces;
     pieces = (X + rowsPerPiece - 1) / rowsPerPiece;
-    hipLaunchKernelGGL((column_sum_kernel<float, true>), dim3((unsigned)colGroups, (unsigned)pieces), dim3(256), 0, stream,
+    hipLaunchKernelGGL((column_sum_kernel<float, SUM_ATOMIC>), dim3((unsigned)colGroups, (unsigned)pieces), dim3(256), 0, stream,
                        static_cast<const float *>(in), X, Y, rowsPerPiece, static_cast<float *>(out), 1.f);
     return (int)hipGetLastError();
 }

@@ -24,11 +24,26 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 14
+    assert len(names) == 15
     assert sorted(nt.EXPORTS) == names
     lib = C.CDLL(nt.LIB_PATH)
     for name in names:
         assert hasattr(lib, name), name
+
+
+def test_measurement_knobs_are_set_by_name_and_not_declared_in_the_header():
+    """The knobs for measurements and tests are exported but no part of the documented interface; they are read
+    from the environment once and changed by name afterwards (no getenv on the way to a launch)."""
+    assert "ntsamd_tuning_set" not in declared_functions()
+    nt.tuning_set("NTSAMD_SPLIT_K", 4)
+    nt.tuning_set("SPLIT_K", None)
+    with pytest.raises(nt.NtsAmdError, match="no knob named"):
+        nt.tuning_set("NTSAMD_NO_SUCH_KNOB", 1)
+    src = open(os.path.join(ROOT, "niutensor_amd", "csrc", "ntsamd_capi.hip")).read()
+    assert src.count("getenv(") == 1          # the one inside the call_once
+    for name in os.listdir(os.path.join(ROOT, "niutensor_amd", "csrc")):
+        if name.endswith((".h", ".hip")) and name != "ntsamd_capi.hip":
+            assert "getenv" not in open(os.path.join(ROOT, "niutensor_amd", "csrc", name)).read(), name
 
 
 def test_no_vendor_blas_is_linked():
@@ -66,6 +81,8 @@ def test_argument_errors_need_no_device():
     assert call_mm(L, ta=nt.X_TRANS, dims=(2, 3, 3, 2, 2, 2)) == 1
     assert call_mm(L, dims=(2, 3, 3, 2, 2, 3)) == 1
     assert call_mm(L, dims=(-2, 3, 3, 2, 2, 2)) == 1
+    assert L.ntsamd_release_workspaces(1000) == 3
+    assert L.ntsamd_release_workspaces(-1) == 0                                        # none allocated: nothing to do
     # null pointers
     assert call_mm(L, ptr=None) == 1
     assert L.ntsamd_last_error().decode() == "Empty matrices in multiplication!"

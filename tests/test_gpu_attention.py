@@ -289,7 +289,6 @@ def test_a_handful_of_query_rows(gpu, oracle, B, lq, lk, H, nh, masked):
     """Up to eight query rows per head (a decoding step) run on the kernel that reads k and v once and
     multiplies in the vector ALU; the same inputs through the MFMA kernel (NTSAMD_ATTN_ROWS=0) must meet
     the same limit against the oracle."""
-    import os
     q, k, v = oracle.normal((B, lq, H), 61), oracle.normal((B, lk, H), 62), oracle.normal((B, lk, H), 63)
     mask = None
     if masked:
@@ -298,10 +297,10 @@ def test_a_handful_of_query_rows(gpu, oracle, B, lq, lk, H, nh, masked):
     scale = 1.0 / np.sqrt(H // nh)
     ref = oracle.attention(q, k, v, nh, scale, mask)
     for rows in ("1", "0"):
-        os.environ["NTSAMD_ATTN_ROWS"] = rows
+        nt.tuning_set("NTSAMD_ATTN_ROWS", rows)
         try:
             got = run(gpu, q, k, v, nh, scale, mask)
         finally:
-            os.environ.pop("NTSAMD_ATTN_ROWS", None)
+            nt.tuning_set("NTSAMD_ATTN_ROWS", None)
         assert_fp32(got, ref, H // nh + lk, what="rows kernel" if rows == "1" else "MFMA kernel")
 

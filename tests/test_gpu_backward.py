@@ -1,11 +1,11 @@
 """Parity of the backward-side entry points with the CPU oracle, through the C ABI:
-products whose k range is cut into pieces that add to c with atomics, products that return
+products whose k range is cut into pieces (which meet in a workspace and are added in a fixed order,
+or add to c with atomics when the knob asks for that), products that return
 the column sums of op(b) on the side, the [x][y][z] reduction, and the three gradient
 steps (MatrixMul, MatrixMulBatched, MulAndShift) assembled from them the way the nts::
 layer assembles them, against the oracle and the compiled reference's fixtures.
 Limits are in tests/tolerance.py."""
 import itertools
-import os
 
 import numpy as np
 import pytest
@@ -17,7 +17,7 @@ from tolerance import assert_fp16, assert_fp32
 pytestmark = pytest.mark.gpu
 
 TRANS = list(itertools.product((X_NOTRANS, X_TRANS), repeat=2))
-ENV = ("NTSAMD_TILE_CFG", "NTSAMD_SPLIT_K")
+ENV = ("NTSAMD_TILE_CFG", "NTSAMD_SPLIT_K", "NTSAMD_F32_SPLIT_ATOMIC")
 
 
 def torch_():
@@ -42,22 +42,27 @@ def halfed(oracle, x):
 def name_the_case(request):
     print("\n[gpu-case] %s" % request.node.nodeid, flush=True)
     for k in ENV:
-        os.environ.pop(k, None)
+        nt.tuning_set(k, None)
     yield
     for k in ENV:
-        os.environ.pop(k, None)
+        nt.tuning_set(k, None)
 
 
 # ---- k cut into pieces ------------------------------------------------------------
 
+@pytest.mark.parametrize("atomic", (False, True))
 @pytest.mark.parametrize("ta,tb", TRANS)
-def test_split_k_against_oracle(gpu, oracle, ta, tb):
-    """Forced piece counts on both tile shapes, every beta (1: nothing to prepare, 0: c is
-    cleared first, other: c is scaled first), a ragged k and a bias riding on the first piece."""
+def test_split_k_against_oracle(gpu, oracle, ta, tb, atomic):
+    """Forced piece counts on both tile shapes, every beta, a ragged k and a bias. Through the workspace (the
+    pieces are added in their order by a second kernel, which also applies beta and the bias) and with the
+    pieces adding to c with atomics (beta 1: nothing to prepare, 0: c is cleared first, other: c is scaled
+    first; the bias rides on the first piece)."""
     torch = torch_()
+    nt.tuning_set("NTSAMD_F32_SPLIT_ATOMIC", 1 if atomic else None)
     for cfg, splits, (M, N, K) in (("0", "2", (128, 256, 1024)), ("0", "4", (100, 72, 1500)), ("1", "8", (64, 192, 4096)),
                                    ("1", "4", (37, 64, 1111)), ("0", "16", (256, 128, 4100))):
-        os.environ["NTSAMD_TILE_CFG"], os.environ["NTSAMD_SPLIT_K"] = cfg, splits
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
+        nt.tuning_set("NTSAMD_SPLIT_K", splits)
         a = oracle.uniform(stored((M, K), ta), 11)
         b = oracle.uniform(stored((K, N), tb), 12)
         c0 = oracle.uniform((M, N), 13)
@@ -87,13 +92,13 @@ def test_split_k_is_chosen_for_weight_gradient_shapes_and_can_be_turned_off(gpu,
     got = {}
     for mode in (None, "1"):
         if mode:
-            os.environ["NTSAMD_SPLIT_K"] = mode
+            nt.tuning_set("NTSAMD_SPLIT_K", mode)
         c = dev(c0, gpu)
         nt.matrix_mul(dev(a, gpu), X_TRANS, dev(b, gpu), X_NOTRANS, c, 1.0, 1.0)
         got[mode] = c.cpu().numpy()
         assert_fp32(got[mode], ref, K, mag, what="weight gradient, split mode %s" % mode)
     # strided batch of long-k products
-    os.environ.pop("NTSAMD_SPLIT_K", None)
+    nt.tuning_set("NTSAMD_SPLIT_K", None)
     B, M, N, K = 3, 64, 64, 2048
     a, b, c0 = oracle.uniform((B, M, K), 4), oracle.uniform((B, K, N), 5), oracle.uniform((B, M, N), 6)
     ref = oracle.matmul_batched(a, X_NOTRANS, b, X_NOTRANS, c0.copy(), 0.5, 0.25)
@@ -101,6 +106,93 @@ def test_split_k_is_chosen_for_weight_gradient_shapes_and_can_be_turned_off(gpu,
     nt.matrix_mul_batched_strided(dev(a, gpu), X_NOTRANS, dev(b, gpu), X_NOTRANS, c, B, M * K, K * N, M * N,
                                   M, K, K, N, M, N, 0.5, 0.25)
     assert_fp32(c.cpu().numpy(), ref, K, what="batched long k")
+
+
+def test_split_k_gives_the_same_bits_on_every_run(gpu, oracle):
+    """Weight-gradient shapes (few tiles, a long k) are cut along k by the library's own choice. The pieces are
+    added in their order, so twenty runs of a float product, of a half one and of the column sums over many rows
+    give bit-identical results, as the reference's cublasSgemm does."""
+    torch = torch_()
+    for half in (False, True):
+        for (M, N, K) in ((512, 512, 4096), (256, 512, 4096), (100, 200, 3000 if not half else 3008)):
+            a = dev(oracle.normal((K, M), 1, 0, 0.5), gpu, half)
+            b = dev(oracle.normal((K, N), 2, 0, 0.5), gpu, half)
+            c0 = dev(oracle.uniform((M, N), 3), gpu, half)
+            first = None
+            for run in range(20):
+                c = c0.clone()
+                nt.matrix_mul(a, X_TRANS, b, X_NOTRANS, c, 1.0, 1.0)
+                if first is None:
+                    first = c
+                assert torch.equal(c, first), "half=%d %dx%dx%d run %d" % (half, M, N, K, run)
+    xs = oracle.normal((8192, 300), 4)
+    x = dev(xs, gpu).reshape(8192, 300, 1)
+    first = None
+    for run in range(20):
+        out = torch.full((300,), float("nan"), device=gpu)
+        nt.reduce_sum_xz(x, out)
+        if first is None:
+            first = out
+            assert_fp32(out.cpu().numpy(), oracle.reduce_sum(xs, 0), 8192, oracle.reduce_sum(np.abs(xs), 0),
+                        what="column sums in pieces")
+        assert torch.equal(out, first), "column sums run %d" % run
+
+
+def test_two_host_threads_on_one_stream_keep_their_pieces_apart(gpu, oracle):
+    """Two host threads issue half weight gradients (512 x 512 x 4096, cut along k) to the NULL stream, as every
+    caller of the nts:: layer does. Each call's product and summing kernels must stay together on the stream: were
+    they to interleave (A product, B product, A sum, B sum), A would sum B's pieces. Every result is checked."""
+    import threading
+    torch = torch_()
+    M, N, K = 512, 512, 4096
+    work = []
+    for t in range(2):
+        a = halfed(oracle, oracle.normal((K, M), 50 + t, 0, 0.5))
+        b = halfed(oracle, oracle.normal((K, N), 60 + t, 0, 0.5))
+        work.append((dev(a, gpu, True), dev(b, gpu, True), oracle.matmul2d(a, X_TRANS, b, X_NOTRANS)))
+    L = nt.load()
+    failures = []
+
+    def issue(t):
+        a, b, ref = work[t]
+        outs = [torch.empty((M, N), device=gpu, dtype=torch.float16) for _ in range(40)]
+        for c in outs:
+            rc = L.ntsamd_matrix_mul(0, None, a.data_ptr(), X_TRANS, nt.X_FLOAT16, b.data_ptr(), X_NOTRANS, nt.X_FLOAT16,
+                                     c.data_ptr(), nt.X_FLOAT16, K, M, K, N, M, N, 1.0, 0.0)
+            if rc != 0:
+                failures.append("thread %d: rc %d" % (t, rc))
+                return
+        torch.cuda.synchronize()
+        for i, c in enumerate(outs):
+            if not torch.equal(c, outs[0]):
+                failures.append("thread %d: product %d differs from the thread's first" % (t, i))
+                break
+        try:
+            assert_fp16(outs[0].float().cpu().numpy(), ref, what="thread %d" % t)
+        except AssertionError as e:
+            failures.append(str(e))
+
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=issue, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
+
+
+def test_workspaces_can_be_released_and_come_back(gpu, oracle):
+    torch = torch_()
+    M, N, K = 256, 256, 4096
+    a, b = dev(oracle.normal((K, M), 1, 0, 0.5), gpu), dev(oracle.normal((K, N), 2, 0, 0.5), gpu)
+    c1, c2 = torch.empty((M, N), device=gpu), torch.empty((M, N), device=gpu)
+    nt.tuning_set("NTSAMD_SPLIT_K", 8)
+    nt.matrix_mul(a, X_TRANS, b, X_NOTRANS, c1)
+    nt.release_workspaces(0)
+    nt.release_workspaces(-1)            # nothing left to free: still fine
+    nt.matrix_mul(a, X_TRANS, b, X_NOTRANS, c2)
+    assert torch.equal(c1, c2)
+    assert_fp32(c1.cpu().numpy(), oracle.matmul2d(a.cpu().numpy(), X_TRANS, b.cpu().numpy(), X_NOTRANS), K)
 
 
 # ---- column sums on the side -----------------------------------------------------------
@@ -117,7 +209,7 @@ def test_matrix_mul_colsum(gpu, oracle, half, ta, tb):
     # 16-byte friendly shapes ride in the product kernel; the ragged ones take the separate pass
     shapes = [(128, 128, 64), (64, 256, 512), (200, 72, 100), (96, 40, 2048), (33, 29, 57), (5, 7, 3), (130, 64, 33)]
     for cfg in ("0", "1"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K) in enumerate(shapes):
             a = oracle.normal(stored((M, K), ta), 100 + i, 0, 0.5)
             b = oracle.normal(stored((K, N), tb), 200 + i, 0, 0.5)
@@ -147,7 +239,7 @@ def test_colsum_with_split_k_and_without_a_product(gpu, oracle):
     a, b = oracle.uniform((K, M), 1), oracle.uniform((K, N), 2)
     c0, s0 = oracle.uniform((M, N), 3), oracle.uniform((N,), 4)
     for splits in ("1", "8"):
-        os.environ["NTSAMD_SPLIT_K"] = splits
+        nt.tuning_set("NTSAMD_SPLIT_K", splits)
         for sbeta in (1.0, 0.0, 0.5):
             c, s = dev(c0, gpu), dev(s0, gpu)
             nt.matrix_mul_colsum(dev(a, gpu), X_TRANS, dev(b, gpu), X_NOTRANS, c, s, 1.0, 1.0, sbeta)
@@ -155,7 +247,7 @@ def test_colsum_with_split_k_and_without_a_product(gpu, oracle):
             assert_fp32(s.cpu().numpy(), sbeta * s0 + oracle.reduce_sum(b, 0), K,
                         np.abs(sbeta * s0) + oracle.reduce_sum(np.abs(b), 0), what="splits %s sbeta %g" % (splits, sbeta))
     # a product with no rows still owes the sums
-    os.environ.pop("NTSAMD_SPLIT_K", None)
+    nt.tuning_set("NTSAMD_SPLIT_K", None)
     torch = torch_()
     s = dev(s0, gpu)
     nt.matrix_mul_colsum(torch.empty((K, 0), device=gpu), X_TRANS, dev(b, gpu), X_NOTRANS,
@@ -172,9 +264,9 @@ def test_half_colsum_with_k_cut(gpu, oracle):
     ref = oracle.matmul2d(a, X_TRANS, b, X_NOTRANS, c0.copy(), 1.0, 1.0)
     for splits in ("1", "8", None):
         if splits is None:
-            os.environ.pop("NTSAMD_SPLIT_K", None)
+            nt.tuning_set("NTSAMD_SPLIT_K", None)
         else:
-            os.environ["NTSAMD_SPLIT_K"] = splits
+            nt.tuning_set("NTSAMD_SPLIT_K", splits)
         for sbeta in (1.0, 0.0):
             c, s = dev(c0, gpu, True), dev(s0, gpu, True)
             nt.matrix_mul_colsum(dev(a, gpu, True), X_TRANS, dev(b, gpu, True), X_NOTRANS, c, s, 1.0, 1.0, sbeta)
@@ -183,7 +275,7 @@ def test_half_colsum_with_k_cut(gpu, oracle):
             sref = sbeta * s0 + oracle.reduce_sum(b, 0)
             smag = np.abs(sbeta * s0) + oracle.reduce_sum(np.abs(b), 0)
             assert np.abs(s.float().cpu().numpy() - sref).max() <= 2.0 ** -10 * smag.max() + 1e-6, what
-    os.environ.pop("NTSAMD_SPLIT_K", None)
+    nt.tuning_set("NTSAMD_SPLIT_K", None)
 
 
 # ---- the reduction ------------------------------------------------------------------------

@@ -5,7 +5,6 @@ library's workspace, which the capturing stream does not have yet: the one alloc
 in the relaxed capture mode) and a conversion are captured once and replayed with new inputs; every
 replay must reproduce the eager results bit for bit (the float product cut along k, whose additions are
 unordered: within the fp32 limit)."""
-import os
 
 import numpy as np
 import pytest
@@ -43,7 +42,7 @@ def test_replays_match_eager(gpu, oracle):
         nt.convert_data_type(h, h16)
         nt.matrix_mul(big_a16, X_NOTRANS, big_b16, X_NOTRANS, cut16, 1.0, 0.0)
 
-    os.environ["NTSAMD_SPLIT_K"] = "4"                  # the product with the long k goes out in four pieces
+    nt.tuning_set("NTSAMD_SPLIT_K", "4")                  # the product with the long k goes out in four pieces
     try:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -73,4 +72,4 @@ def test_replays_match_eager(gpu, oracle):
                 else:
                     assert torch.equal(got, ref), "replay %d: %s" % (rep, name)
     finally:
-        os.environ.pop("NTSAMD_SPLIT_K", None)
+        nt.tuning_set("NTSAMD_SPLIT_K", None)

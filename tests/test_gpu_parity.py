@@ -7,7 +7,6 @@ on sampled rows plus size-independent properties (scaling, accumulation,
 transposition). Limits are in tests/tolerance.py.
 """
 import itertools
-import os
 
 import numpy as np
 import pytest
@@ -50,11 +49,11 @@ def magnitude(oracle, a, ta, b, tb, alpha, beta=0.0, c0=None, bias=None):
 def name_the_case(request):
     # a GPU fault can take the box with it: say which test is running first
     print("\n[gpu-case] %s" % request.node.nodeid, flush=True)
-    os.environ.pop("NTSAMD_TILE_CFG", None)
-    os.environ.pop("NTSAMD_SPLIT_K", None)
+    nt.tuning_set("NTSAMD_TILE_CFG", None)
+    nt.tuning_set("NTSAMD_SPLIT_K", None)
     yield
-    os.environ.pop("NTSAMD_TILE_CFG", None)
-    os.environ.pop("NTSAMD_SPLIT_K", None)
+    nt.tuning_set("NTSAMD_TILE_CFG", None)
+    nt.tuning_set("NTSAMD_SPLIT_K", None)
 
 
 # ---- fixtures held by the reference and by the compiled reference ------------
@@ -164,7 +163,7 @@ def test_fp32_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
     # 128 x 128, 64 x 64, 32 x 128 (at most 32 rows; else the rule's choice), 16 rows per workgroup on the same kernel
     for cfg in ("0", "1", "3", "4"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K) in enumerate(SHAPES):
             a = oracle.uniform(stored((M, K), ta), 1000 + i)
             b = oracle.uniform(stored((K, N), tb), 2000 + i)
@@ -182,7 +181,7 @@ def test_fp16_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
     # 128 x 128, 64 x 64, 256 x 256 (eight waves up to k = 2048, four beyond: the last shape)
     for cfg in ("0", "1", "2"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K) in enumerate(SHAPES + [(264, 520, 2304)]):
             # round the inputs to half first; the oracle then runs in fp32 on those values
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 4000 + i, 0, 0.5)))
@@ -207,10 +206,7 @@ def test_half_products_cut_along_k(gpu, oracle, ta, tb):
     shapes = [(8, 8, 264), (72, 136, 1000), (40, 51, 1024), (200, 24, 4096), (16, 512, 2048), (256, 256, 2304)]
     for cfg, pieces in ((None, None), ("0", "2"), ("0", "16"), ("1", "2"), ("1", "16")):
         for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces)):
-            if val is None:
-                os.environ.pop(key, None)
-            else:
-                os.environ[key] = val
+            nt.tuning_set(key, val)
         for i, (M, N, K) in enumerate(shapes if cfg else shapes[-2:]):
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 8000 + i, 0, 0.5)))
             b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 8100 + i, 0, 0.5)))
@@ -243,8 +239,8 @@ def test_batches_of_half_products_cut_along_k(gpu, oracle):
     of a merged tensor): every piece of every item finds its place in the workspace and in c, and what lies
     between the rows of c stays as it was. Twice in a row on one stream: the second call reuses the workspace."""
     torch = torch_()
-    os.environ["NTSAMD_TILE_CFG"] = "1"
-    os.environ["NTSAMD_SPLIT_K"] = "4"
+    nt.tuning_set("NTSAMD_TILE_CFG", "1")
+    nt.tuning_set("NTSAMD_SPLIT_K", "4")
     M, N, K, count = 40, 72, 1536, 3
     ldc, between = 3 * N, N
     a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((count, M, K), 8400, 0, 0.5)))
@@ -264,8 +260,8 @@ def test_half_products_cut_along_k_on_two_streams(gpu, oracle):
     such products at the same time must not see each other's. The sums are added in a fixed order, so each result
     must equal, bit for bit, what the same product gives on its own."""
     torch = torch_()
-    os.environ["NTSAMD_TILE_CFG"] = "1"
-    os.environ["NTSAMD_SPLIT_K"] = "8"
+    nt.tuning_set("NTSAMD_TILE_CFG", "1")
+    nt.tuning_set("NTSAMD_SPLIT_K", "8")
     M, N, K = 64, 512, 4096
     ops = []
     for i in range(2):
@@ -323,7 +319,7 @@ def test_half_in_float_out_on_the_main_path(gpu, oracle, ta, tb):
     the fp32 limit applies."""
     torch = torch_()
     for cfg in ("0", "1", "2"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K) in enumerate([(8, 8, 8), (64, 72, 40), (136, 264, 96), (257, 120, 64), (300, 520, 128)]):
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 7000 + i, 0, 0.5)))
             b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 7100 + i, 0, 0.5)))
@@ -347,7 +343,7 @@ def test_fp32_rows_of_any_length_and_alignment(gpu, oracle, ta, tb):
     k >= K that is not discarded, would poison the result."""
     torch = torch_()
     for cfg in ("0", "1"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K, shift) in enumerate([(129, 67, 33, 1), (70, 131, 130, 3), (255, 257, 63, 2), (3, 2, 1, 1), (64, 64, 515, 5)]):
             a = oracle.uniform(stored((M, K), ta), 8100 + i)
             b = oracle.uniform(stored((K, N), tb), 8200 + i)
@@ -363,7 +359,7 @@ def test_fp32_rows_of_any_length_and_alignment(gpu, oracle, ta, tb):
                 nt.matrix_mul(av, ta, bv, tb, c, alpha, beta)
                 assert_fp32(c.cpu().numpy(), ref, K, magnitude(oracle, a, ta, b, tb, alpha, beta, c0),
                             what="cfg%s %dx%dx%d shift %d alpha=%g beta=%g" % (cfg, M, N, K, shift, alpha, beta))
-    os.environ.pop("NTSAMD_TILE_CFG", None)
+    nt.tuning_set("NTSAMD_TILE_CFG", None)
     # a batch of products whose items are an odd number of elements apart
     count, M, N, K = 5, 45, 51, 37
     a = oracle.uniform((count,) + stored((M, K), ta), 8400)
@@ -435,7 +431,7 @@ def test_half_rows_of_any_length_and_alignment(gpu, oracle, ta, tb, out_float):
     # the two long ones run many turns of the straight-line loop (a ring of four slabs in registers between memory
     # and LDS), with a ragged last slab after a complete one and with a last slab that is complete
     for (M, N, K) in ((203, 301, 77), (131, 135, 259), (9, 7, 5), (1, 300, 1), (70, 67, 1003), (33, 141, 1056)):
-        os.environ["NTSAMD_TILE_CFG"] = "1" if K == 1056 else "0"
+        nt.tuning_set("NTSAMD_TILE_CFG", "1" if K == 1056 else "0")
         a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((M, K), ta), 31)))
         b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((K, N), tb), 32)))
         bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((N,), 33)))
@@ -597,7 +593,7 @@ def test_fused_bias_and_rectify(gpu, oracle, half):
     (row-indexed bias), with beta, and with a NaN and a negative zero forced into the result."""
     torch = torch_()
     for cfg in ("0", "1", "2") if half else ("0", "1"):
-        os.environ["NTSAMD_TILE_CFG"] = cfg
+        nt.tuning_set("NTSAMD_TILE_CFG", cfg)
         for i, (M, N, K) in enumerate([(64, 64, 32), (136, 264, 96), (257, 120, 64), (33, 35, 37) if not half else (40, 48, 56)]):
             x = oracle.normal((M, K), 9000 + i)
             w = oracle.normal((K, N), 9100 + i, 0, 0.3)
@@ -618,7 +614,7 @@ def test_fused_bias_and_rectify(gpu, oracle, half):
                     assert_fp16(got, ref, what="cfg%s %dx%dx%d beta=%g" % (cfg, M, N, K, beta))
                 else:
                     assert_fp32(got, ref, K, what="cfg%s %dx%dx%d beta=%g" % (cfg, M, N, K, beta))
-    os.environ.pop("NTSAMD_TILE_CFG", None)
+    nt.tuning_set("NTSAMD_TILE_CFG", None)
     if not half:
         # bias by row group (generic path) with the activation
         x, w, b = oracle.normal((60, 20), 9400), oracle.normal((20, 30), 9401), oracle.normal((6,), 9402)
