@@ -293,6 +293,33 @@ int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS
  */
 int ntsamd_release_workspaces(int devID);
 
+/*
+ * ntsamd_matrix_mul for callers that cannot allocate: it calls no hipMalloc, no hipFree and no allocating
+ * library routine, ever. HAS NO COUNTERPART IN THE REFERENCE; it is for code under HIP graph capture,
+ * tight serving loops and harnesses that forbid allocation, where ntsamd_matrix_mul's first product cut along
+ * k on a stream would allocate that stream's workspace. Same arguments, same result, same kernels; the partial
+ * products of a k cut into pieces go to a static array in device memory of NTSAMD_STATIC_SCRATCH_BYTES, which
+ * is part of the library's code object: every GPU the library runs on holds one copy from the moment the code
+ * is loaded there (ntsamd_init(devID) does that, and is the place to do it before a capture begins) until the
+ * process ends.
+ *   splits = 0           the library chooses, among the ways to cut k whose partial products fit the array
+ *                        (one piece, and no scratch at all, for most shapes: see ntsamd_matrix_mul);
+ *   splits = 2, 4, 8, 16 k is cut into that many pieces. NTSAMD_ERR_ARGUMENT, with the sizes in the message,
+ *                        if splits x nc x mc x 4 bytes exceed NTSAMD_STATIC_SCRATCH_BYTES, if a piece would
+ *                        be shorter than 128 (half) or 64 (float) values of k, or if the operands cannot take
+ *                        the 16-byte path (half: 16-byte aligned, rows of whole 16-byte pieces).
+ * All calls on one GPU share that GPU's array, on whatever stream: calls that may overlap on one GPU (different
+ * streams, or graphs replayed side by side) race on it and must be ordered by the caller. The array keeps the
+ * last call's partial products; every call overwrites all it reads, so nothing has to be cleared.
+ */
+#define NTSAMD_STATIC_SCRATCH_BYTES (16 << 20)
+int ntsamd_matrix_mul_static(int devID, void * stream,
+                             const void * a, int transposedA, int dataTypeA,
+                             const void * b, int transposedB, int dataTypeB,
+                             void * c, int dataTypeC,
+                             int na, int ma, int nb, int mb, int nc, int mc,
+                             float alpha, float beta, int splits);
+
 #ifdef __cplusplus
 }
 #endif

@@ -280,6 +280,40 @@ std::mutex g_splitMutex;                            /* guards the map, not the w
 std::map<std::pair<int, hipStream_t>, SplitWork *> g_splitWork;   /* entries are never removed */
 std::atomic<int> g_splitAlive;
 
+/* The entry point that allocates nothing keeps its partial products here instead: part of the code object, so
+   every device the library runs on holds its own copy from the moment the code is loaded there until the process
+   ends. In host code the array's name is only a handle for hipGetSymbolAddress; the address on each device is
+   looked up once, with that device current, and kept in g_scratch. */
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)NTSAMD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+struct StaticScratch {
+    std::atomic<float *> ptr;
+    std::mutex inUse;
+};
+StaticScratch g_scratch[MAX_DEVICES];
+std::mutex g_scratchMutex;
+
+/* the static scratch of devID, which is current; NULL with the message set if the runtime cannot name it */
+float * static_scratch(int devID)
+{
+    float * ptr = g_scratch[devID].ptr.load(std::memory_order_acquire);
+    if (ptr != NULL)
+        return ptr;
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    ptr = g_scratch[devID].ptr.load(std::memory_order_acquire);
+    if (ptr != NULL)
+        return ptr;
+    void * found = NULL;
+    const hipError_t err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || found == NULL) {
+        (void)hipGetLastError();
+        fail(NTSAMD_ERR_DEVICE, "cannot locate the static scratch on device %d: %s", devID, hipGetErrorString(err));
+        return NULL;
+    }
+    g_scratch[devID].ptr.store(static_cast<float *>(found), std::memory_order_release);
+    return static_cast<float *>(found);
+}
+
 /* A workspace held for the launches of one call; released when the call returns. */
 struct WorkHold {
     float * mem;
@@ -331,6 +365,18 @@ struct WorkHold {
         mem = w->mem;
         bytes = SPLIT_WORK_BYTES;
         held = &w->inUse;
+    }
+    /* the static scratch of devID (current); false with the message set if it cannot be found */
+    bool take_static(int devID)
+    {
+        float * ptr = static_scratch(devID);
+        if (ptr == NULL)
+            return false;
+        g_scratch[devID].inUse.lock();
+        mem = ptr;
+        bytes = STATIC_SCRATCH_BYTES;
+        held = &g_scratch[devID].inUse;
+        return true;
     }
 };
 
@@ -398,6 +444,12 @@ struct Grid {
     long long strideA1, strideB1, strideC1;
 };
 
+/* The entry point that allocates nothing: partial products go to the static scratch; splits = 0 lets the estimate
+   choose among what fits there, 2, 4, 8 or 16 asks for that many pieces */
+struct NoAlloc {
+    int splits;
+};
+
 int run(int devID, void * stream, Kind kind, const Shape & s,
         const void * a, const void * b, void * c,
         int lda, int ldb, int ldc,
@@ -405,7 +457,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         const PtrBatch * ptrs,
         float alpha, float beta,
         const void * bias, int biasMode, int biasLen, int biasRowDiv,
-        void * colSum = NULL, float colSumBeta = 0.f, int act = ACT_NONE, const Grid * grid = NULL)
+        void * colSum = NULL, float colSumBeta = 0.f, int act = ACT_NONE, const Grid * grid = NULL,
+        const NoAlloc * noAlloc = NULL)
 {
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
@@ -483,19 +536,41 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
        can add to c with atomics instead (in no fixed order; dense results without activation only, and c gets
        its beta first): only if the knob asks for it, or when there is no workspace to be had. */
     const bool atomicAble = !half && vec && !ptrs && act == ACT_NONE && dense;
-    const bool atomicAsked = atomicAble && tn.f32SplitAtomic.load(std::memory_order_relaxed) > 0;
+    const bool atomicAsked = atomicAble && !noAlloc && tn.f32SplitAtomic.load(std::memory_order_relaxed) > 0;
     const bool maySplit = atomicAsked || ((half ? fetch16 == F16_DIRECT : vec) && !ptrs);
-    const size_t workBytes = atomicAsked ? 0 : SPLIT_WORK_BYTES;
+    const size_t workBytes = atomicAsked ? 0 : (noAlloc ? STATIC_SCRATCH_BYTES : SPLIT_WORK_BYTES);
     /* pieces that meet in a workspace gather no column sums: cutting costs a pass of its own over b then (a
        launch, b read once more) */
     const bool colSumAside = colSum != NULL && vec && count == 1 && !atomicAsked;
     const double cutExtra = colSumAside ? 2.3 + (half ? 2.0 : 4.0) * s.K * s.N / 4.0e6 : 0.0;
     const bool fast32 = kind == KIND_F32 && vec && !ptrs && colSum == NULL;
-    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, workBytes, cutExtra, fast32);
+    int forcedSplits = -1;
+    if (noAlloc && noAlloc->splits != 0) {
+        forcedSplits = noAlloc->splits;
+        if (forcedSplits != 2 && forcedSplits != 4 && forcedSplits != 8 && forcedSplits != 16)
+            return fail(NTSAMD_ERR_ARGUMENT, "k can be cut into 2, 4, 8 or 16 pieces (or 0: the library chooses), not %d",
+                        forcedSplits);
+        if (!maySplit)
+            return fail(NTSAMD_ERR_ARGUMENT, "this product cannot be cut along k (half operands must be 16-byte "
+                        "aligned with rows of whole 16-byte pieces, rows shorter than 2097152 elements)");
+        if (s.K / forcedSplits < (half ? 128 : 64))
+            return fail(NTSAMD_ERR_ARGUMENT, "k = %d is too short for %d pieces (at least %d each)", s.K, forcedSplits,
+                        half ? 128 : 64);
+        if ((long long)s.M * s.N * count * forcedSplits * 4 > (long long)STATIC_SCRATCH_BYTES)
+            return fail(NTSAMD_ERR_ARGUMENT, "%d partial products of %d x %d floats (%lld bytes) exceed the static "
+                        "scratch of %lld bytes", forcedSplits, s.M, s.N, (long long)s.M * s.N * count * forcedSplits * 4,
+                        (long long)STATIC_SCRATCH_BYTES);
+    }
+    Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, workBytes, cutExtra, fast32, forcedSplits);
     WorkHold work;
     bool viaWork = false;
     if (plan.splits > 1 && !atomicAsked) {
-        work.take_stream(devID, hs);
+        if (noAlloc) {
+            if (!work.take_static(devID))
+                return NTSAMD_ERR_DEVICE;
+        }
+        else
+            work.take_stream(devID, hs);
         viaWork = work.mem != NULL;
         if (!viaWork && !atomicAble)
             plan = choose_plan(s.M, s.N, s.K, count, half, false, beta != 1.f, 0, 0.0, fast32);
@@ -529,7 +604,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         else {
             /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS. It runs before the product
                on the same stream, so the two can share the workspace. */
-            if (!half && !s.bKContig)
+            if (!half && !s.bKContig && !noAlloc)
                 work.take_stream(devID, hs);
             rc = s.bKContig ? launch_reduce_sum_xz(half, b, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
                             : launch_reduce_sum_xz(half, b, s.K, s.N, 1, colSum, colSumBeta, hs, work.mem, work.bytes / 4);
@@ -588,6 +663,10 @@ int ntsamd_init(int devID)
     if (scope.status != NTSAMD_OK)
         return scope.status;
     (void)tuning();
+    /* naming the static scratch makes the runtime load the code object on this device: here rather than at the
+       first product, which may be issued where nothing may allocate */
+    if (static_scratch(devID) == NULL)
+        return NTSAMD_ERR_DEVICE;
     return NTSAMD_OK;
 }
 
@@ -633,6 +712,32 @@ int ntsamd_tuning_set(const char * name, int value)
             return NTSAMD_OK;
         }
     return fail(NTSAMD_ERR_ARGUMENT, "no knob named %s", name);
+}
+
+int ntsamd_matrix_mul_static(int devID, void * stream,
+                             const void * a, int transposedA, int dataTypeA,
+                             const void * b, int transposedB, int dataTypeB,
+                             void * c, int dataTypeC,
+                             int na, int ma, int nb, int mb, int nc, int mc,
+                             float alpha, float beta, int splits)
+{
+    Kind kind;
+    Shape s;
+    int st = check_types(dataTypeA, dataTypeB, dataTypeC, kind);
+    if (st == NTSAMD_OK)
+        st = check_shape(transposedA, transposedB, na, ma, nb, mb, nc, mc, s);
+    if (st != NTSAMD_OK)
+        return st;
+    if (splits < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative number of pieces");
+    if (s.M == 0 || s.N == 0)
+        return NTSAMD_OK;
+    st = check_pointers(a, b, c);
+    if (st != NTSAMD_OK)
+        return st;
+    const NoAlloc na0 = {splits};
+    return run(devID, stream, kind, s, a, b, c, ma, mb, mc, 0, 0, 0, 1, NULL, alpha, beta,
+               NULL, NTSAMD_BIAS_NONE, 0, 1, NULL, 0.f, ACT_NONE, NULL, &na0);
 }
 
 int ntsamd_matrix_mul_bias(int devID, void * stream,

@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 15
+    assert len(names) == 16
     assert sorted(nt.EXPORTS) == names
     lib = C.CDLL(nt.LIB_PATH)
     for name in names:
@@ -81,6 +81,11 @@ def test_argument_errors_need_no_device():
     assert call_mm(L, ta=nt.X_TRANS, dims=(2, 3, 3, 2, 2, 2)) == 1
     assert call_mm(L, dims=(2, 3, 3, 2, 2, 3)) == 1
     assert call_mm(L, dims=(-2, 3, 3, 2, 2, 2)) == 1
+    # the entry point that allocates nothing checks its arguments the same way, and its number of pieces
+    args = (0, None, 0x1000, 1, 2, 0x1000, 1, 2, 0x1000, 2)
+    assert L.ntsamd_matrix_mul_static(*args, 2, 3, 3, 2, 2, 2, 1.0, 0.0, -1) == 1
+    assert L.ntsamd_matrix_mul_static(*args, 2, 3, 2, 3, 2, 3, 1.0, 0.0, 0) == 1
+    assert L.ntsamd_matrix_mul_static(*args, 0, 3, 3, 2, 0, 2, 1.0, 0.0, 0) == 0       # no rows: nothing to do
     assert L.ntsamd_release_workspaces(1000) == 3
     assert L.ntsamd_release_workspaces(-1) == 0                                        # none allocated: nothing to do
     # null pointers
