@@ -7,8 +7,14 @@ A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM: one launch of the configuration's product through the C
 ABI (two launches for the attention pair). The default workload is the
 MulAndShift linear layer, fp32 X[32x128x512] x W[512x2048] + b[2048]: the first
-configuration the metric's target is quoted on. `--all` adds one line per
-configuration before the headline line; the LAST line printed is the headline.
+configuration the metric's target is quoted on. The headline line (the LAST line
+printed) also carries, under "configs", the kernel time, TFLOP/s and fraction of
+the matrix peak of every one of the baseline's five configurations, measured in
+the same run. `--all` adds one full line per configuration before the headline.
+
+Whatever --warmup says, every configuration first runs until SETTLE_S seconds of
+GPU time have passed: the clocks of the part need tens of milliseconds of load to
+settle, and a short warm-up would time the ramp.
 
 Each JSON line carries
   value/unit       TFLOP/s = 2 M N K batch / time, over the timed steps
@@ -29,6 +35,8 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6}     # MI355X dense matrix peaks (datasheet)
 HBM_TBS = 8.0
+SETTLE_S = 0.15                                 # GPU time under load before anything is timed
+BASELINE_CONFIGS = (1, 2, 3, 4, 5)
 
 
 def configs():
@@ -360,12 +368,24 @@ def graph_replayed(wl, dev, ev, steps_in_graph=50, replays=20):
     return ev.time(g.replay, stream, replays) / steps_in_graph
 
 
-def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
+def settle(wl, ev, stream):
+    """Runs the workload until SETTLE_S seconds of GPU time have passed; returns the launches it took."""
+    done, spent = 0, 0.0
+    reps = 8
+    while spent < SETTLE_S:
+        spent += ev.time(wl.run, stream, reps) * reps
+        done += reps
+        reps = min(reps * 2, 512)
+    return done
+
+
+def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0):
     import torch
     wl = Workload(idx, dev, oracle)
     cfg = wl.cfg
     ev = HipEvents()
     stream = torch.cuda.current_stream(dev).cuda_stream
+    settled = settle(wl, ev, stream)
     for _ in range(warmup):
         wl.run()
     torch.cuda.synchronize()
@@ -380,16 +400,19 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
     kt_graph = graph_replayed(wl, dev, ev) if kt / wl.launches < 20e-6 else None
     peak = PEAK_TFLOPS[cfg["dtype"]]
     achieved = wl.flops / kt / 1e12
-    # the attention pair moves 16 flops per byte: it is bound by memory, not by the matrix pipe
-    if idx in (3, 7, 9, 11, 12):
-        roof = {"bound": "hbm", "achieved": round(wl.bytes / kt / 1e9, 1), "peak": HBM_TBS * 1e3, "unit": "GB/s",
-                "frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4)}
-    else:
-        roof = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4)}
-    roof.update({"traffic": measured_traffic(idx), "kernel_us": round(kt / wl.launches * 1e6, 2),
+    # Every configuration is held against the dense matrix peak of its data type: that is what the metric and its
+    # targets are quoted in. The attention-shaped batches move only 16 flops per byte, so their HBM fraction is given
+    # beside it.
+    roof = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+            "frac": round(achieved / peak, 4)}
+    traffic = measured_traffic(idx)
+    roof.update({"traffic": traffic,
+                 "traffic_source": None if traffic is None else
+                 "committed rocprofv3 FETCH_SIZE/WRITE_SIZE table (profiles/hbm_traffic_per_step.md), not measured in this run",
+                 "kernel_us": round(kt / wl.launches * 1e6, 2),
                  "kernel_us_best": round(kt_best / wl.launches * 1e6, 2),
-                 "mfma_tflops": round(achieved, 3), "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)})
+                 "hbm_frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4),
+                 "hbm_floor_us": round(wl.bytes / (HBM_TBS * 1e12) * 1e6, 2)})
     if kt_graph is not None:
         # launches this short are issued by the host about as fast as the GPU runs them: the same launches
         # replayed from a HIP graph, for what the kernel itself takes (not used for value, achieved or frac)
@@ -409,13 +432,26 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu):
         "data": "synthetic",
         "config": {"workload": cfg["name"], "M": cfg["M"], "N": cfg["N"], "K": cfg["K"], "batch": cfg["batch"],
                    "launches_per_step": wl.launches, "inputs": "resident in HBM", "flops_per_step": wl.flops,
-                   "algorithmic_bytes_per_step": wl.bytes},
+                   "algorithmic_bytes_per_step": wl.bytes,
+                   "settle": "%d untimed steps (%.2f s of GPU time) before the %d warm-up steps" % (settled, SETTLE_S, warmup)},
         "pct_of_peak": round(100.0 * wl.flops / wall / 1e12 / peak, 2),
         "roofline": roof,
     }
     if with_cpu:
-        out["cpu_baseline"] = cpu_baseline(idx)
+        out["cpu_baseline"] = cpu_baseline(idx, cpu_budget_s)
     return out
+
+
+def brief(line):
+    """What the headline line keeps of another configuration's line."""
+    keep = {"workload": line["config"]["workload"], "dtype": line["dtype"], "steps": line["steps"],
+            "kernel_us": line["roofline"]["kernel_us"], "launches_per_step": line["config"]["launches_per_step"],
+            "value": line["value"], "unit": line["unit"], "pct_of_peak": line["pct_of_peak"],
+            "roofline": {k: line["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "hbm_frac",
+                                                          "traffic", "traffic_source")}}
+    if "cpu_baseline" in line:
+        keep["cpu_baseline"] = line["cpu_baseline"]
+    return keep
 
 
 def main():
@@ -451,12 +487,25 @@ def main():
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "copies": args.steps}))
         return
     oracle = Oracle()
+    with_cpu = not args.no_cpu
+    lines = {}
     if args.all:
         for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13):
+            if idx == args.config:
+                continue
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
-            print(json.dumps(bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle,
-                                       not args.no_cpu)), flush=True)
-    print(json.dumps(bench_one(args.config, args.steps, args.warmup, dev, oracle, not args.no_cpu)), flush=True)
+            lines[idx] = bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle, with_cpu)
+            print(json.dumps(lines[idx]), flush=True)
+    head = bench_one(args.config, args.steps, args.warmup, dev, oracle, with_cpu)
+    lines[args.config] = head
+    # the other configurations of the baseline, each settled and timed like the headline (at least 50 steps, so that
+    # a short headline run still gives them a steady reading; a tenth for the 1 ms product), CPU leg on a 3 s sample
+    for idx in BASELINE_CONFIGS:
+        if idx not in lines:
+            steps = max(50, args.steps) if idx != 5 else max(20, args.steps // 10)
+            lines[idx] = bench_one(idx, steps, args.warmup, dev, oracle, with_cpu, cpu_budget_s=3.0)
+    head["configs"] = [brief(lines[idx]) for idx in BASELINE_CONFIGS]
+    print(json.dumps(head), flush=True)
 
 
 if __name__ == "__main__":

@@ -660,6 +660,26 @@ def sampled_f64(a, ta, b, tb, rows, alpha=1.0):
     return alpha * (A @ B)
 
 
+def whole_f64(a, ta, b, tb):
+    """op(a) op(b) in double precision on the host, the WHOLE result: a mistake in the mapping of workgroups to
+    tiles (the renumbering by XCD, the last group of tile rows, an unwritten tile) cannot hide between samples."""
+    A = (a.T if ta == X_TRANS else a).astype(np.float64)
+    B = (b.T if tb == X_TRANS else b).astype(np.float64)
+    return A @ B
+
+
+def library_magnitude(gpu, a, ta, b, tb, half=False):
+    """(|a| |b|)_ij for the component-wise measure, at sizes where the CPU oracle would take minutes: one more
+    product of the library itself, on the absolute values (every term positive: no cancellation to get wrong)."""
+    torch = torch_()
+    ga, gb = dev_tensor(np.abs(a), gpu, half), dev_tensor(np.abs(b), gpu, half)
+    rows = a.shape[1] if ta == X_TRANS else a.shape[0]
+    cols = b.shape[0] if tb == X_TRANS else b.shape[1]
+    m = torch.empty((rows, cols), device=gpu)
+    nt.matrix_mul(ga, ta, gb, tb, m)
+    return m.cpu().numpy().astype(np.float64)
+
+
 def test_config1_and_2_linear_layer(gpu, oracle):
     """fp32 [4096x512] x [512x2048], plain and with the bias of MulAndShift."""
     torch = torch_()
@@ -669,9 +689,17 @@ def test_config1_and_2_linear_layer(gpu, oracle):
     gx, gw, gb = dev_tensor(x, gpu), dev_tensor(w, gpu), dev_tensor(bias, gpu)
     c = torch.full((4096, 2048), float("nan"), device=gpu)
     nt.matrix_mul(gx, X_NOTRANS, gw, X_NOTRANS, c)
-    rows = np.random.default_rng(0).choice(4096, 96, replace=False)
     got = c.cpu().numpy()
-    assert_fp32(got[rows], sampled_f64(x, X_NOTRANS, w, X_NOTRANS, rows), 512)
+    # every element, against double precision, under both measures
+    want = whole_f64(x, X_NOTRANS, w, X_NOTRANS)
+    mag = library_magnitude(gpu, x, X_NOTRANS, w, X_NOTRANS)
+    assert_fp32(got, want, 512, mag, what="configuration 2 without its bias, whole result")
+    # configuration 1's own operands: both uniform
+    w1 = oracle.uniform((512, 2048), 2)
+    c1 = torch.full((4096, 2048), float("nan"), device=gpu)
+    nt.matrix_mul(gx, X_NOTRANS, dev_tensor(w1, gpu), X_NOTRANS, c1)
+    assert_fp32(c1.cpu().numpy(), whole_f64(x, X_NOTRANS, w1, X_NOTRANS), 512,
+                library_magnitude(gpu, x, X_NOTRANS, w1, X_NOTRANS), what="configuration 1, whole result")
     # the oracle itself on a slab of rows (it needs ~1 s per 400 rows here)
     ref = oracle.matmul2d(x[:256].copy(), X_NOTRANS, w, X_NOTRANS)
     assert_fp32(got[:256], ref, 512, magnitude(oracle, x[:256].copy(), X_NOTRANS, w, X_NOTRANS, 1.0))
@@ -679,6 +707,8 @@ def test_config1_and_2_linear_layer(gpu, oracle):
     nt.matrix_mul(gx, X_NOTRANS, gw, X_NOTRANS, cb, bias=gb)
     # the epilogue adds bias[column] to the same accumulators
     assert normwise((cb - c).cpu().numpy(), np.broadcast_to(bias, (4096, 2048))) < 1e-5
+    assert_fp32(cb.cpu().numpy(), want + bias.astype(np.float64), 512, mag + np.abs(bias),
+                what="configuration 2, whole result")
     ref_b, n = oracle.mulandshift(x[:64].copy().reshape(1, 64, 512), w, bias)
     assert n == 2
     assert_fp32(cb.cpu().numpy()[:64], ref_b[0], 512)
@@ -693,11 +723,18 @@ def test_config3_attention_batches(gpu, oracle):
     s = torch.full((256, 128, 128), float("nan"), device=gpu)
     nt.matrix_mul_batched_strided(gq, X_NOTRANS, gk, X_TRANS, s, 256, 8192, 8192, 16384, 128, 64, 128, 64, 128, 128, 0.125)
     s_ref = oracle.matmul_batched(q, X_NOTRANS, k, X_TRANS, None, 0.125)
-    assert_fp32(s.cpu().numpy(), s_ref, 64)
+    s_mag = oracle.matmul_batched(np.abs(q), X_NOTRANS, np.abs(k), X_TRANS, None, 0.125)
+    assert_fp32(s.cpu().numpy(), s_ref, 64, s_mag, what="configuration 3, scores, all 256 items")
+    assert_fp32(s.cpu().numpy(), 0.125 * np.einsum("bik,bjk->bij", q.astype(np.float64), k.astype(np.float64)), 64, s_mag,
+                what="configuration 3, scores against double precision")
     o = torch.full((256, 128, 64), float("nan"), device=gpu)
     nt.matrix_mul_batched_strided(s, X_NOTRANS, gv, X_NOTRANS, o, 256, 16384, 8192, 8192, 128, 128, 128, 64, 128, 64)
-    o_ref = oracle.matmul_batched(s.cpu().numpy(), X_NOTRANS, v, X_NOTRANS)
-    assert_fp32(o.cpu().numpy(), o_ref, 128)
+    sh = s.cpu().numpy()
+    o_ref = oracle.matmul_batched(sh, X_NOTRANS, v, X_NOTRANS)
+    o_mag = oracle.matmul_batched(np.abs(sh), X_NOTRANS, np.abs(v), X_NOTRANS)
+    assert_fp32(o.cpu().numpy(), o_ref, 128, o_mag, what="configuration 3, context, all 256 items")
+    assert_fp32(o.cpu().numpy(), np.einsum("bik,bkj->bij", sh.astype(np.float64), v.astype(np.float64)), 128, o_mag,
+                what="configuration 3, context against double precision")
 
 
 def test_config4_half_tn(gpu, oracle):
@@ -709,8 +746,8 @@ def test_config4_half_tn(gpu, oracle):
     c = torch.full((8192, 4096), float("nan"), device=gpu, dtype=torch.float16)
     nt.matrix_mul(ga, X_TRANS, gb, X_NOTRANS, c)
     got = c.float().cpu().numpy()
-    rows = np.random.default_rng(1).choice(8192, 64, replace=False)
-    assert_fp16(got[rows], sampled_f64(a, X_TRANS, b, X_NOTRANS, rows))
+    # every element against double precision (assert_fp16 also wants every element finite: c held NaN)
+    assert_fp16(got, whole_f64(a, X_TRANS, b, X_NOTRANS), what="configuration 4, whole result")
     # the fp32 oracle on a block of result rows (columns of the stored a)
     sub = np.ascontiguousarray(a[:, :96])
     assert_fp16(got[:96], oracle.matmul2d(sub, X_TRANS, b, X_NOTRANS))
@@ -719,8 +756,12 @@ def test_config4_half_tn(gpu, oracle):
     nt.matrix_mul(ga, X_TRANS, gb, X_NOTRANS, c2, 2.0)
     normal = c.abs() > 2.0 ** -13      # above the first binade, where a value just below 2^-14 may round up into it
     assert normal.float().mean() > 0.9
+    assert bool(torch.isfinite(c2).all())
     assert int((c2[normal] != (2 * c)[normal]).sum()) == 0
     assert torch.equal(c2[normal], (2 * c)[normal])
+    # below that, doubling the fp32 sum before the one rounding can differ from doubling the rounded half by a
+    # half's smallest step at most
+    assert float((c2.float() - 2 * c.float())[~normal].abs().max()) <= 2.0 ** -24
 
 
 def test_config5_ragged_vocab_projection(gpu, oracle):
@@ -733,16 +774,16 @@ def test_config5_ragged_vocab_projection(gpu, oracle):
     c = dev_tensor(c0, gpu)
     nt.matrix_mul(gh, X_NOTRANS, gw, X_TRANS, c, 1.0, 1.0)
     got = c.cpu().numpy()
-    rows = np.random.default_rng(2).choice(4096, 48, replace=False)
-    want = sampled_f64(h, X_NOTRANS, w, X_TRANS, rows) + c0[rows]
-    assert_fp32(got[rows], want, 512)
+    # every element against double precision, under both measures
+    prod = whole_f64(h, X_NOTRANS, w, X_TRANS)
+    mag = library_magnitude(gpu, h, X_NOTRANS, w, X_TRANS) + np.abs(c0)
+    assert_fp32(got, prod + c0, 512, mag, what="configuration 5, whole result")
     # the oracle on the last rows (the ragged right edge is in every row)
     ref = oracle.matmul2d(h[-24:].copy(), X_NOTRANS, w, X_TRANS, c0[-24:].copy(), 1.0, 1.0)
     assert_fp32(got[-24:], ref, 512)
     # accumulate once more: c + h w^T again = c0 + 2 h w^T
     nt.matrix_mul(gh, X_NOTRANS, gw, X_TRANS, c, 1.0, 1.0)
-    want2 = 2 * sampled_f64(h, X_NOTRANS, w, X_TRANS, rows) + c0[rows]
-    assert_fp32(c.cpu().numpy()[rows], want2, 512)
+    assert_fp32(c.cpu().numpy(), 2 * prod + c0, 512, 2 * mag, what="configuration 5 accumulated twice, whole result")
 
 
 def test_a_batch_with_too_many_tiles_is_refused(gpu):
