@@ -22,6 +22,15 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+/* Cache policy of the stores that write c through the fast epilogues (the last argument of the buffer store
+   builtins: sc0 = 1, nt = 2, sc1 = 16). WRITE_THROUGH (sc0 sc1) sends the lines on to memory as they are written
+   instead of leaving them dirty in the XCD's L2: a kernel that ends with its result dirty in L2 is followed by
+   the write-back of all of it before the next kernel on the stream may start (measured: about 5 us after 67 MB
+   of half results, 1.4 of 10.4 us on the attention-shaped batches), while lines written through leave during the
+   kernel. Only for results whose rows are whole 128-byte lines: written through in pieces of lines (rows of
+   30011 floats) the same stores were 4 % slower than the default. */
+constexpr int STORE_DEFAULT = 0, STORE_WRITE_THROUGH = 17;
+
 enum BiasMode { BIAS_NONE = 0, BIAS_COL = 1, BIAS_ROW = 2 };
 
 /* applied to a result element on its way out: y = x < 0 ? 0 : x is the reference's Rectify
@@ -76,6 +85,9 @@ struct GemmParams {
     float * splitWork;
     int act;                               /* Activation of the epilogue */
     int wideRowsOnly;                      /* fp32, measurements: no 16-row MFMAs for products of at most 16 rows */
+    int f16PingPong;                       /* half, 256 x 256 tile: the two wave groups run one phase apart */
+    int storeHint;                         /* != 0: the fast epilogues write c through (STORE_WRITE_THROUGH) */
+    int persistGrid;                       /* half, 256 x 256 tile: > 0 = that many workgroups walk over all tiles */
 };
 
 /* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and
@@ -102,11 +114,12 @@ struct TileCoord {
     int batch, tm, tn, split;
 };
 
-__device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
+/* the tile with number `raw` in the order workgroups are dispatched in (consecutive numbers go to the XCDs in turn) */
+__device__ __forceinline__ TileCoord tile_of_id(const GemmParams & p, int raw)
 {
     int perBatch = p.tilesM * p.tilesN;
     int perSplit = perBatch * p.batch;
-    int id = xcd_contiguous_id((int)blockIdx.x, perSplit * p.splits);
+    int id = xcd_contiguous_id(raw, perSplit * p.splits);
     TileCoord t;
     t.split = id / perSplit;
     id -= t.split * perSplit;
@@ -120,6 +133,11 @@ __device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
     t.tm = firstM + q % gsz;
     t.tn = q / gsz;
     return t;
+}
+
+__device__ __forceinline__ TileCoord tile_of_workgroup(const GemmParams & p)
+{
+    return tile_of_id(p, (int)blockIdx.x);
 }
 
 /* tile shapes the dispatcher can pick from */

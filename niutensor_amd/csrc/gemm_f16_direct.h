@@ -85,7 +85,8 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
 /* SPLIT: the k range is cut into p.splits pieces, one workgroup each, and every workgroup leaves its partial tile
    as plain fp32 (no alpha, beta, bias or activation) in p.splitWork, which holds p.splits x p.batch dense M x N
    matrices; split_reduce.hip adds the pieces up and does what the epilogue would have done. */
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4,
+          bool PP = false>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
@@ -469,6 +470,103 @@ gemm_f16_direct_kernel(const GemmParams p)
                 rest(rest, IntC<NSTAGE + 1>(), IntC<0>());
         }
     }
+    else if constexpr (PP) {
+        /* Ping-pong: the eight waves form two groups, waves 0-3 and waves 4-7, one wave of each on every SIMD.
+           A slab is two phases for a wave: a MEMORY phase (this wave's loads of the slab three ahead go out, all
+           the fragments of the slab come in from LDS) and a COMPUTE phase (the slab's 2 x NM MFMAs back to back,
+           at raised priority), each closed by a workgroup barrier. The second group runs one phase behind the
+           first (it passes one barrier more before it starts and the first one more at the end), so on every
+           SIMD one wave is in its compute phase while the other is in its memory phase: the matrix pipe sees one
+           unbroken run of MFMAs from alternating waves, and the LDS latency, the waits and the barriers of one
+           wave lie under the MFMAs of the other, instead of both waves of a SIMD meeting the same barrier at
+           the same time. Number the barriers b = 0, 1, 2 ... after the one that ends the prologue. The first
+           group reads slab t between barriers 2t-1 and 2t, the second between 2t and 2t+1. Every wave has waited
+           for its own loads of slab t+1 before it leaves the memory phase of slab t (before barrier 2t for the
+           first group, 2t+1 for the second), so slab t+1 is whole in LDS for everybody after barrier 2t+1, which
+           is where its earliest reader starts. A wave overwrites the stage of slab t-1 (with slab t+3) at the
+           start of its memory phase of slab t, after barrier 2t-1 (2t for the second group); the last reads of
+           slab t-1 finished before barrier 2t-1. */
+        static_assert(NSTAGE == 4 && NW == 8 && !CS, "ping-pong: eight waves, four stages, no column sums");
+        if (nk > 0) {
+            const bool follower = wave >= NW / 2;
+            issue_loads(IntC<1>(), 0);
+            if (nk > 1)
+                issue_loads(IntC<1>(), 1);
+            if (nk > 2)
+                issue_loads(IntC<1>(), 2);
+            if (nk > 3)
+                issue_loads(IntC<1>(), 3);
+            if (nk > 3)
+                wait_vmcnt<3 * NL>();
+            else if (nk > 2)
+                wait_vmcnt<2 * NL>();
+            else if (nk > 1)
+                wait_vmcnt<NL>();
+            else
+                wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (follower)
+                __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+
+            /* AHEAD = how many later slabs exist (capped at 3); ISSUE: slab kt+3 exists and is not in flight yet */
+            auto pp_slab = [&](auto AHEADC, auto ISSUEC, auto TAILC, int kt) {
+                constexpr int ahead = decltype(AHEADC)::value;
+                const char * stage = lds + (kt % NSTAGE) * STAGE;
+                if constexpr (decltype(ISSUEC)::value != 0)
+                    issue_loads(TAILC, kt + 3);
+                read_frags(IntC<0>(), stage);
+                read_frags(IntC<1>(), stage);
+                wait_vmcnt<(ahead >= 3 ? 2 : (ahead == 2 ? 1 : 0)) * NL>();
+                wait_lgkmcnt0();
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+                for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+                    for (int g = 0; g < NM; g++) {
+                        const int i = g / TJ, j = g % TJ;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+                    }
+                __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            };
+
+            const int nkFull = K / BKT;
+            int kt = 0;
+            /* the first slab issues nothing: the prologue has slabs 0 to 3 in flight */
+            if (nk > 3)
+                pp_slab(IntC<3>(), IntC<0>(), IntC<0>(), 0);
+            else if (nk > 2)
+                pp_slab(IntC<2>(), IntC<0>(), IntC<0>(), 0);
+            else if (nk > 1)
+                pp_slab(IntC<1>(), IntC<0>(), IntC<0>(), 0);
+            else
+                pp_slab(IntC<0>(), IntC<0>(), IntC<0>(), 0);
+            kt = 1;
+            for (; kt + 3 < nkFull; kt++)
+                pp_slab(IntC<3>(), IntC<1>(), IntC<0>(), kt);      /* slab kt+3 is complete: no tail handling */
+            for (; kt + 3 < nk; kt++)
+                pp_slab(IntC<3>(), IntC<1>(), IntC<1>(), kt);
+            if (kt + 2 < nk) {
+                pp_slab(IntC<2>(), IntC<0>(), IntC<0>(), kt);
+                kt++;
+            }
+            if (kt + 1 < nk) {
+                pp_slab(IntC<1>(), IntC<0>(), IntC<0>(), kt);
+                kt++;
+            }
+            if (kt < nk)
+                pp_slab(IntC<0>(), IntC<0>(), IntC<0>(), kt);
+            if (!follower)
+                __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
     else if (nk > 0) {
         static_assert(DEEP || NSTAGE == 4, "this loop is written for four stages");
         /* prologue: all four stages in flight, then wait for the first */
@@ -570,8 +668,9 @@ gemm_f16_direct_kernel(const GemmParams p)
         const int colW = n0 + wn0 + rdChunk * 8;
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
 
-        auto turn = [&](auto BETAC) {
+        auto turn = [&](auto BETAC, auto AUXC) {
             constexpr bool useOld = decltype(BETAC)::value != 0;
+            constexpr int aux = decltype(AUXC)::value;
             typedef typename std::conditional<useOld, float, half_t>::type StageT;
             /* row pitch: the two half-waves write rows 4 apart; keep them in different banks */
             constexpr int PITCH = TJ * 32 * (int)sizeof(StageT) + (useOld ? 32 : 16);
@@ -615,21 +714,29 @@ gemm_f16_direct_kernel(const GemmParams p)
                             v[e] = (half_t)activate(lo[e] + beta * (float)o[e], act);
                             v[4 + e] = (half_t)activate(hi[e] + beta * (float)o[4 + e], act);
                         }
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(f32x4, v), cr, (int)off, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(f32x4, v), cr, (int)off, 0, aux);
                     }
                     else {
                         const f32x4 v = *reinterpret_cast<const f32x4 *>(src);
-                        __builtin_amdgcn_raw_buffer_store_b128(v, cr, (int)off, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(v, cr, (int)off, 0, aux);
                     }
                 }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
             }
         };
-        if (beta != 0.f)
-            turn(IntC<1>());
-        else
-            turn(IntC<0>());
+        if (beta != 0.f) {
+            if (p.storeHint)
+                turn(IntC<1>(), IntC<STORE_WRITE_THROUGH>());
+            else
+                turn(IntC<1>(), IntC<STORE_DEFAULT>());
+        }
+        else {
+            if (p.storeHint)
+                turn(IntC<0>(), IntC<STORE_WRITE_THROUGH>());
+            else
+                turn(IntC<0>(), IntC<STORE_DEFAULT>());
+        }
         return;
     }
 
@@ -675,7 +782,8 @@ gemm_f16_direct_kernel(const GemmParams p)
         narrow(IntC<0>());
 }
 
-template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4>
+template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4,
+          bool PP = false>
 static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
 {
     GemmParams p = p0;
@@ -684,7 +792,7 @@ static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
     if (!SPLIT)
         p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT, NSTAGE>),
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT, NSTAGE, PP>),
                        grid, dim3(WGM * WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -697,6 +805,10 @@ static int launch_f16_direct(const GemmParams & p, hipStream_t stream)
         /* The big tile on eight waves (wave tile 128 x 64, two waves per SIMD that cover each other's waits at
            the barrier and for LDS) instead of four (wave tile 128 x 128, half the LDS reads per MFMA): measured
            15-20 % faster at k = 512, 3-8 % at k = 1024, level at k = 4096 and 0-4 % slower at k = 8192. */
+        if constexpr (!CS) {
+            if (p.f16PingPong)
+                return launch_f16_direct_shape<OutT, S::BM, S::BN, 2, 4, 1, AKC, BKC, false, false, 4, true>(p, stream);
+        }
         if (p.K <= 2048)
             return launch_f16_direct_shape<OutT, S::BM, S::BN, 2, 4, 1, AKC, BKC, CS>(p, stream);
     }
@@ -723,6 +835,9 @@ static int launch_f16_staged(const GemmParams & p, const PtrBatch * ptrs, int cf
 }
 
 template <bool AKC, bool BKC>
+static int launch_f16_persistent(const GemmParams & p0, hipStream_t stream);     /* gemm_f16_persist.h */
+
+template <bool AKC, bool BKC>
 static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, int vec, bool outF32, int cfg,
                             hipStream_t stream)
 {
@@ -732,6 +847,9 @@ static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, int vec
     if (vec == F16_SCALAR || ptrs)
         return outF32 ? launch_f16_staged<float, AKC, BKC, false>(p, ptrs, cfg, stream)
                       : launch_f16_staged<half_t, AKC, BKC, false>(p, ptrs, cfg, stream);
+    /* many tiles of 256 x 256 with nothing to read in the epilogue: one workgroup per CU walks over them */
+    if (cfg == CFG_256x256 && p.persistGrid > 0 && !outF32)
+        return launch_f16_persistent<AKC, BKC>(p, stream);
     /* a float result: the same main loop, 4-byte stores from the accumulators */
     if (outF32) {
         if (cfg == CFG_256x256)

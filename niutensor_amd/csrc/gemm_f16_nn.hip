@@ -1,5 +1,5 @@
 /* fp16 kernels for op(a),op(b) = nn (n: X_NOTRANS, t: X_TRANS); one file per pair so they build in parallel */
-#include "gemm_f16_direct.h"
+#include "gemm_f16_persist.h"
 namespace ntsamd {
 int launch_f16_nn(const GemmParams & p, const PtrBatch * ptrs, int vec, bool outF32, int cfg, hipStream_t stream)
 {

@@ -519,40 +519,48 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
             return;
         }
         /* beta is tested once, outside the loops: inside them the test would fence every
-           load of c off in a block of its own, one memory round trip after the other */
+           load of c off in a block of its own, one memory round trip after the other; the cache policy of the
+           stores is a constant of the instruction, so it is chosen out here too */
+        auto store_all = [&](auto BETAC, auto AUXC) {
+            constexpr bool useOld = decltype(BETAC)::value != 0;
+            constexpr int aux = decltype(AUXC)::value;
+            float old[useOld ? TI : 1][useOld ? TJ : 1][ACCN];
+            if constexpr (useOld) {
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+#pragma unroll
+                    for (int j = 0; j < TJ; j++)
+#pragma unroll
+                        for (int r = 0; r < ACCN; r++) {
+                            const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
+                            old[i][j][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
+                        }
+            }
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int r = 0; r < ACCN; r++) {
+                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
+                        float v = alpha * acc[i][j][r] + bcol[j];
+                        if constexpr (useOld)
+                            v += beta * old[i][j][r];
+                        v = activate(v, act);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, aux);
+                    }
+        };
         if (beta != 0.f) {
-            float old[TI][TJ][ACCN];
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-#pragma unroll
-                    for (int r = 0; r < ACCN; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
-                        old[i][j][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, (int)off, 0, 0));
-                    }
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-#pragma unroll
-                    for (int r = 0; r < ACCN; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
-                        const float v = activate(alpha * acc[i][j][r] + bcol[j] + beta * old[i][j][r], act);
-                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
-                    }
+            if (p.storeHint)
+                store_all(IntC<1>(), IntC<STORE_WRITE_THROUGH>());
+            else
+                store_all(IntC<1>(), IntC<STORE_DEFAULT>());
         }
         else {
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-#pragma unroll
-                    for (int r = 0; r < ACCN; r++) {
-                        const unsigned off = cOff[j] + (unsigned)(i * 32 + (R16 ? r : 8 * (r / 4) + (r % 4))) * rowPitch;
-                        const float v = activate(alpha * acc[i][j][r] + bcol[j], act);
-                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), cr, (int)off, 0, 0);
-                    }
+            if (p.storeHint)
+                store_all(IntC<0>(), IntC<STORE_WRITE_THROUGH>());
+            else
+                store_all(IntC<0>(), IntC<STORE_DEFAULT>());
         }
     }
     else {

@@ -51,6 +51,7 @@ int fail(int code, const char * fmt, ...)
 /* devices already checked: written once per device, read-only afterwards */
 constexpr int MAX_DEVICES = 64;
 std::atomic<int> g_deviceState[MAX_DEVICES];   /* 0 unknown, 1 good, -1 not gfx950 */
+std::atomic<int> g_deviceCUs[MAX_DEVICES];     /* compute units, known once the state is */
 
 int check_device(int devID)
 {
@@ -67,6 +68,7 @@ int check_device(int devID)
         if (hipGetDeviceProperties(&prop, devID) != hipSuccess)
             return fail(NTSAMD_ERR_DEVICE, "cannot query device %d", devID);
         st = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+        g_deviceCUs[devID].store(prop.multiProcessorCount, std::memory_order_relaxed);
         g_deviceState[devID].store(st, std::memory_order_release);
         if (st == 1)
             return NTSAMD_OK;
@@ -235,9 +237,12 @@ struct Plan {
      NTSAMD_F16_FETCH=0|2        keep half products off the main path (element-wise / register-staged fetch)
      NTSAMD_ATTN_ROWS=0          keep attention with a handful of query rows on the MFMA kernels
      NTSAMD_F32_R16=0            no 16-row MFMAs for float products of at most 16 rows
-     NTSAMD_F32_SPLIT_ATOMIC=1   float pieces of k add to c with atomics (no workspace, no fixed order) */
+     NTSAMD_F32_SPLIT_ATOMIC=1   float pieces of k add to c with atomics (no workspace, no fixed order)
+     NTSAMD_F16_PINGPONG=0       half, 256 x 256 tile: the main loop in which both waves of a SIMD meet one barrier
+     NTSAMD_F16_PERSIST=0        half, 256 x 256 tile: one workgroup per tile, never one per CU that walks over tiles
+     NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -250,6 +255,8 @@ const Knob g_knobs[] = {
     {"NTSAMD_TILE_CFG", &Tuning::tileCfg},   {"NTSAMD_SPLIT_K", &Tuning::splitK},
     {"NTSAMD_F16_FETCH", &Tuning::f16Fetch}, {"NTSAMD_ATTN_ROWS", &Tuning::attnRows},
     {"NTSAMD_F32_R16", &Tuning::f32R16},     {"NTSAMD_F32_SPLIT_ATOMIC", &Tuning::f32SplitAtomic},
+    {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
+    {"NTSAMD_STORE_HINT", &Tuning::storeHint},
 };
 
 const Tuning & tuning()
@@ -501,6 +508,15 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.groupM = 8;
     p.act = act;
     p.wideRowsOnly = tn.f32R16.load(std::memory_order_relaxed) == 0;
+    p.f16PingPong = tn.f16PingPong.load(std::memory_order_relaxed) != 0;
+    {
+        /* results whose rows are whole 128-byte lines are written through (see STORE_WRITE_THROUGH) */
+        const long long unit = kind == KIND_F16 ? 2 : 4;
+        const bool lines = (reinterpret_cast<uintptr_t>(c) & 127u) == 0 && !ptrs && (ldc * unit) % 128 == 0 &&
+                           (strideC * unit) % 128 == 0 && (!grid || (grid->strideC1 * unit) % 128 == 0);
+        const int knob = tn.storeHint.load(std::memory_order_relaxed);
+        p.storeHint = knob >= 0 ? knob : (lines ? 1 : 0);
+    }
     if (grid) {
         p.batchInner = grid->inner;
         p.strideA1 = grid->strideA1;
@@ -577,6 +593,23 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     }
     const int cfg = plan.cfg;
     int rc = 0;
+    /* More 256 x 256 tiles than CUs, a half result in whole 16-byte pieces and nothing to read on the way out
+       (no old c, no bias): one workgroup per CU walks over the tiles and fetches the next tile's first slabs
+       before the finished tile's results leave */
+#ifdef NTSAMD_PROBE
+    const bool probeBias = true;        /* a profiling build: the bias pointer is where the time stamps go */
+#else
+    const bool probeBias = false;
+#endif
+    if (kind == KIND_F16 && cfg == CFG_256x256 && fetch16 == F16_DIRECT && beta == 0.f && (bias == NULL || probeBias) && colSum == NULL &&
+        s.K >= 256 && tn.f16Persist.load(std::memory_order_relaxed) != 0) {
+        const int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
+        const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;
+        const bool wide = ldc % 8 == 0 && s.N % 8 == 0 && aligned16(c) && strideC % 8 == 0 &&
+                          (!grid || grid->strideC1 % 8 == 0);
+        if (wide && cus > 0 && tiles > cus)
+            p.persistGrid = cus;
+    }
     p.splits = 1;
     if (plan.splits > 1) {
         p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 31) / 32 * 32;
