@@ -35,6 +35,14 @@
  *     the finished tile's NST stores and slabs 2 and 3 after them, so "slab 0 has landed" is
  *     vmcnt <= 3 NL + NST and "slab 1 has landed" is vmcnt <= 2 NL + NST; from slab 2 on the
  *     stores are older than every load still awaited.
+ *   - A k-contiguous operand is fetched TWO slabs at a time: a slab of 32 k is 64 bytes of a row, half a cache
+ *     line, and fetched slab by slab every line crossed the path from L2 twice (measured with the same kernel
+ *     fetching whole lines of the wrong bytes: 8192 x 4096 x 1024 with both operands k-contiguous 68.5 -> 63.4 us,
+ *     8192^3 903 -> 845 us). So the eight lanes that fetch a row's 128 bytes sit in one load instruction: a chunk
+ *     of 1 KB is 8 rows x (64 bytes of the even slab, then 64 bytes of the odd slab), the four stages of such an
+ *     operand are two pair slots, and a pair is requested at the start of an even slab, two slabs before its
+ *     first half is read. An mn-contiguous operand keeps its slab-by-slab fetch three slabs ahead (its rows are
+ *     whole lines already). The two operands have their own regions of LDS for that.
  *   - No loads in the epilogue: the compiler cannot see the LDS-direct loads (inline
  *     assembly) and would wait for ALL of them before using a loaded value. Hence beta == 0
  *     and no bias here; products with either run on the one-tile-per-workgroup kernels.
@@ -48,42 +56,39 @@ template <bool AKC, bool BKC>
 __global__ void __launch_bounds__(512, 1)
 gemm_f16_persistent_kernel(const GemmParams p)
 {
-    constexpr int BM = 256, BN = 256, WGN = 4, NW = 8, BKT = 32, KS = 2, NSTAGE = 4;
+    constexpr int BM = 256, BN = 256, WGN = 4, NW = 8, BKT = 32, KS = 2;
     constexpr int WM = 128, WN = 64, TI = 4, TJ = 2, NM = TI * TJ;
-    /* per-operand LDS geometry, bytes: as in gemm_f16_direct_kernel */
-    constexpr int A_RPC = AKC ? 16 : 512 / BM;
-    constexpr int B_RPC = BKC ? 16 : 512 / BN;
-    constexpr int A_NCH = AKC ? BM / 16 : BKT / A_RPC;
-    constexpr int B_NCH = BKC ? BN / 16 : BKT / B_RPC;
-    constexpr int A_CP = AKC ? 1024 : 1088;
-    constexpr int B_CP = BKC ? 1024 : 1088;
-    constexpr int A_BYTES = A_NCH * A_CP;
-    constexpr int B_BYTES = B_NCH * B_CP;
-    constexpr int STAGE = A_BYTES + B_BYTES;
-    constexpr int NLA = A_NCH / NW, NLB = B_NCH / NW;
-    constexpr int NL = NLA + NLB;
+    /* LDS, one region per operand, four slabs each.
+       k-contiguous: two pair slots of 32 KB; a chunk of 1 KB holds 8 rows x [slab parity][64 bytes], the four 16-byte
+           columns of a row's 64 bytes permuted by (row >> 2) & 3 (sixteen consecutive rows reading one logical
+           column hit sixteen different 16-byte bank groups: rows r, r+4, r+8, r+12 share 64 bytes of a 256-byte line).
+       mn-contiguous: four stages of 16 chunks (k rows c and c+16, 512 bytes each), chunks 1088 bytes apart. */
+    constexpr int KC_SLOT = 32 * 1024, KC_REGION = 2 * KC_SLOT;
+    constexpr int MN_CP = 1088, MN_STAGE = 16 * MN_CP, MN_REGION = 4 * MN_STAGE;
+    constexpr int A_REGION = AKC ? KC_REGION : MN_REGION, B_REGION = BKC ? KC_REGION : MN_REGION;
+    constexpr int A_HALF = AKC ? KC_SLOT : 2 * MN_STAGE, B_HALF = BKC ? KC_SLOT : 2 * MN_STAGE;   /* where slabs 2 and 3 begin */
+    /* load instructions per wave: KA, KB per PAIR of slabs (k-contiguous), MA, MB per slab (mn-contiguous) */
+    constexpr int KA = AKC ? 4 : 0, KB = BKC ? 4 : 0, MA = AKC ? 0 : 2, MB = BKC ? 0 : 2;
+    constexpr int KK = KA + KB, MM = MA + MB;
     /* the epilogue's turn through LDS: 32 rows of the wave's 64 columns as halves, rows 144 bytes apart (sixteen
        lanes that write 16 bytes each to sixteen consecutive rows then cover all 64 banks) */
     constexpr int EPI_PITCH = WN * 2 + 16, EPI_WAVE = 32 * EPI_PITCH;
     constexpr int NST = TI * 4;                     /* store instructions per wave and tile: 8 rows of 128 bytes each */
-    static_assert(NW * EPI_WAVE <= 2 * STAGE, "the epilogue's staging must fit stages 2 and 3");
-    static_assert(NSTAGE * STAGE <= 160 * 1024, "the stages must fit LDS");
-    static_assert(3 * NL + NST < 64, "the wait counter has six bits");
+    static_assert(4 * EPI_WAVE <= A_REGION - A_HALF && 4 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
+    static_assert(A_REGION + B_REGION <= 160 * 1024, "the stages must fit LDS");
+    static_assert(MM + NST + KK + 2 * MM < 64, "the wait counter has six bits");
 
-    __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
+    __shared__ __attribute__((aligned(1024))) char lds[A_REGION + B_REGION];
 
-    /* profiling builds (-DNTSAMD_PROBE) keep time stamps of the 100 MHz clock in registers and write them, 16 per
-       workgroup, to where p.bias points when the kernel ends */
+    /* profiling builds (-DNTSAMD_PROBE) leave time stamps of the 100 MHz clock in LDS (thread 0 only) and write
+       them, 16 per workgroup, to where p.bias points when the kernel ends */
 #ifdef NTSAMD_PROBE
-    unsigned long long st[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#define NTSAMD_STAMP(n) do { st[(n)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-    /* and, of slab 8 of every tile, the shader clock at six points of the slab, waves 0 and 4 */
-    unsigned long long fine[6] = {0, 0, 0, 0, 0, 0};
-#define NTSAMD_FINE(n) do { if (kt == 8) fine[(n)] = __builtin_amdgcn_s_memtime(); } while (0)
+    __shared__ unsigned long long stampLds[16];
+#define NTSAMD_STAMP(n) do { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); if (threadIdx.x == 0) stampLds[(n)] = t_; } while (0)
 #else
 #define NTSAMD_STAMP(n) do { } while (0)
-#define NTSAMD_FINE(n) do { } while (0)
 #endif
+#define NTSAMD_FINE(n) do { } while (0)
 
     const int M = p.M, N = p.N, K = p.K;
     const int tid = threadIdx.x;
@@ -91,55 +96,72 @@ gemm_f16_persistent_kernel(const GemmParams p)
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
     const int l32 = lane & 31, lh = lane >> 5;
     const bool follower = wave >= NW / 2;
-    const int nk = (K + BKT - 1) / BKT, nkFull = K / BKT;     /* the launcher guarantees nk >= 8 */
+    const int nk = (K + BKT - 1) / BKT;                        /* the launcher guarantees nk >= 8 */
     const int total = p.tilesM * p.tilesN * p.batch;
 
     /* ---- the tile whose operands are being fetched ---------------------------------- */
+    /* Where a tile lies is scalar arithmetic with divisions in it (a microsecond of it, measured, when it sat
+       between one tile's last slab and its epilogue): locate() works it out for the NEXT tile while the current
+       tile waits for its first slab, adopt() then only has the per-lane offsets left to do. */
+    struct Loc {
+        int m0, n0;
+        half_t * C;
+        const half_t * A, * B;
+    };
+    auto locate = [&](int id) {
+        const TileCoord tc = tile_of_id(p, id);
+        Loc l;
+        l.A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
+        l.B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
+        l.C = static_cast<half_t *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
+        l.m0 = tc.tm * BM;
+        l.n0 = tc.tn * BN;
+        return l;
+    };
     int m0 = 0, n0 = 0;
     half_t * C = NULL;
     const half_t * aTile = NULL, * bTile = NULL, * aEnd = NULL, * bEnd = NULL;
-    int aOff[NLA], bOff[NLB];
-    int aKc[NLA], bKc[NLB];
-    auto setup = [&](int id) {
-        const TileCoord tc = tile_of_id(p, id);
-        const half_t * A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
-        const half_t * B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
-        C = static_cast<half_t *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
-        m0 = tc.tm * BM;
-        n0 = tc.tn * BN;
+    /* a lane's share of its wave's chunks: byte offset from the first element of the slab (of the pair's even slab),
+       and, k-contiguous, the first k of its 16 bytes inside the pair */
+    constexpr int NQA = AKC ? KA : MA, NQB = BKC ? KB : MB;
+    int aOff[NQA], bOff[NQB];
+    int aKc[NQA], bKc[NQB];
+    auto adopt = [&](const Loc & l) {
+        const half_t * A = l.A, * B = l.B;
+        C = l.C;
+        m0 = l.m0;
+        n0 = l.n0;
 #pragma unroll
-        for (int q = 0; q < NLA; q++) {
-            const int ch = wave * NLA + q;
+        for (int q = 0; q < NQA; q++) {
+            const int ch = wave * NQA + q;
             if (AKC) {
-                int row = ch * 16 + (lane >> 2);
-                int col = (lane & 3) ^ ((row >> 2) & 3);
-                aKc[q] = col * 8;
-                int r = m0 + row < M - 1 ? row : M - 1 - m0;
-                aOff[q] = (r * p.lda + col * 8) * 2;
+                const int row = ch * 8 + ((lane >> 2) & 7);
+                const int col = (lane & 3) ^ ((row >> 2) & 3);
+                aKc[q] = (lane >> 5) * 32 + col * 8;
+                const int r = m0 + row < M - 1 ? row : M - 1 - m0;
+                aOff[q] = (r * p.lda + aKc[q]) * 2;
             }
             else {
-                constexpr int LPRA = 64 / A_RPC;
-                int krow = ch + A_NCH * (lane / LPRA);
-                int c = (lane % LPRA) * 8;
+                const int krow = ch + 16 * (lane >> 5);
+                int c = (lane & 31) * 8;
                 c = m0 + c < M - 8 ? c : M - 8 - m0;
                 aKc[q] = 0;
                 aOff[q] = (krow * p.lda + c) * 2;
             }
         }
 #pragma unroll
-        for (int q = 0; q < NLB; q++) {
-            const int ch = wave * NLB + q;
+        for (int q = 0; q < NQB; q++) {
+            const int ch = wave * NQB + q;
             if (BKC) {
-                int row = ch * 16 + (lane >> 2);
-                int col = (lane & 3) ^ ((row >> 2) & 3);
-                bKc[q] = col * 8;
-                int r = n0 + row < N - 1 ? row : N - 1 - n0;
-                bOff[q] = (r * p.ldb + col * 8) * 2;
+                const int row = ch * 8 + ((lane >> 2) & 7);
+                const int col = (lane & 3) ^ ((row >> 2) & 3);
+                bKc[q] = (lane >> 5) * 32 + col * 8;
+                const int r = n0 + row < N - 1 ? row : N - 1 - n0;
+                bOff[q] = (r * p.ldb + bKc[q]) * 2;
             }
             else {
-                constexpr int LPRB = 64 / B_RPC;
-                int krow = ch + B_NCH * (lane / LPRB);
-                int c = (lane % LPRB) * 8;
+                const int krow = ch + 16 * (lane >> 5);
+                int c = (lane & 31) * 8;
                 c = n0 + c < N - 8 ? c : N - 8 - n0;
                 bKc[q] = 0;
                 bOff[q] = (krow * p.ldb + c) * 2;
@@ -153,31 +175,63 @@ gemm_f16_persistent_kernel(const GemmParams p)
 
     const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);
 
-    auto issue_loads = [&](auto TAIL, int kt) {
-        constexpr bool mayHangOver = decltype(TAIL)::value != 0;
+    /* the pair of slabs (kt, kt + 1), kt even, of the k-contiguous operands; the pieces that begin at or past K
+       are sent out of range (they read as zero) */
+    auto issue_pair = [&](int kt) {
         const int k0 = kt * BKT;
-        const unsigned stage = ldsBase + (unsigned)((kt % NSTAGE) * STAGE);
-        const bool tail = mayHangOver && k0 + BKT > K;
-        const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
-        const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
-        const i32x4 ad = make_desc(ab, (long long)(aEnd - ab) * 2), bd = make_desc(bb, (long long)(bEnd - bb) * 2);
+        const bool tail = k0 + 2 * BKT > K;
+        const unsigned slot = (unsigned)(((kt >> 1) & 1) * KC_SLOT);
+        if constexpr (AKC) {
+            const half_t * ab = aTile + k0;
+            const i32x4 ad = make_desc(ab, (long long)(aEnd - ab) * 2);
 #pragma unroll
-        for (int q = 0; q < NLA; q++) {
-            int off = aOff[q];
-            if (AKC && tail && k0 + aKc[q] >= K)
-                off = NTSAMD_OOB_OFFSET;
-            lds_dma16(ad, stage + (unsigned)((wave * NLA + q) * A_CP), off);
+            for (int q = 0; q < KA; q++) {
+                int off = aOff[q];
+                if (tail && k0 + aKc[q] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                lds_dma16(ad, ldsBase + slot + (unsigned)((wave * KA + q) * 1024), off);
+            }
         }
+        if constexpr (BKC) {
+            const half_t * bb = bTile + k0;
+            const i32x4 bd = make_desc(bb, (long long)(bEnd - bb) * 2);
 #pragma unroll
-        for (int q = 0; q < NLB; q++) {
-            int off = bOff[q];
-            if (BKC && tail && k0 + bKc[q] >= K)
-                off = NTSAMD_OOB_OFFSET;
-            lds_dma16(bd, stage + (unsigned)(A_BYTES + (wave * NLB + q) * B_CP), off);
+            for (int q = 0; q < KB; q++) {
+                int off = bOff[q];
+                if (tail && k0 + bKc[q] >= K)
+                    off = NTSAMD_OOB_OFFSET;
+                lds_dma16(bd, ldsBase + (unsigned)A_REGION + slot + (unsigned)((wave * KB + q) * 1024), off);
+            }
         }
     };
+    /* slab kt of the mn-contiguous operands (rows of k past K lie past the end of the descriptor: they read as zero) */
+    auto issue_slab = [&](int kt) {
+        const int k0 = kt * BKT;
+        const unsigned stage = (unsigned)((kt & 3) * MN_STAGE);
+        if constexpr (!AKC) {
+            const half_t * ab = aTile + (size_t)k0 * p.lda;
+            const i32x4 ad = make_desc(ab, (long long)(aEnd - ab) * 2);
+#pragma unroll
+            for (int q = 0; q < MA; q++)
+                lds_dma16(ad, ldsBase + stage + (unsigned)((wave * MA + q) * MN_CP), aOff[q]);
+        }
+        if constexpr (!BKC) {
+            const half_t * bb = bTile + (size_t)k0 * p.ldb;
+            const i32x4 bd = make_desc(bb, (long long)(bEnd - bb) * 2);
+#pragma unroll
+            for (int q = 0; q < MB; q++)
+                lds_dma16(bd, ldsBase + (unsigned)A_REGION + stage + (unsigned)((wave * MB + q) * MN_CP), bOff[q]);
+        }
+    };
+    /* slabs kt and kt + 1 (kt even) of both operands, in the order the waits below count on: the pair, then the
+       mn-contiguous operands' slab kt, then their slab kt + 1 */
+    auto issue_two = [&](int kt) {
+        issue_pair(kt);
+        issue_slab(kt);
+        issue_slab(kt + 1);
+    };
 
-    /* ---- fragment addresses (byte offsets inside a stage) ---------------------------- */
+    /* ---- fragment addresses (byte offsets inside the operand's region, slab 0) ----------- */
     /* The b fragment is the FIRST operand of the MFMA here: its lane rho (0..31) supplies the result's ROW rho, and
        result register r of a lane with half-wave h holds row 8 (r/4) + 4 h + r%4. Column pcol(rho) of the b block
        goes to fragment lane rho, with groups of four columns dealt out as
@@ -195,37 +249,43 @@ gemm_f16_persistent_kernel(const GemmParams p)
 #pragma unroll
     for (int kk = 0; kk < KS; kk++) {
         const int sw = (l32 >> 2) & 3, swB = (pcol >> 2) & 3;
-        aFrag[kk] = (wm0 + l32) * 64 + ((kk * 2 + lh) ^ sw) * 16;
-        bFrag[kk] = A_BYTES + (wn0 + pcol) * 64 + ((kk * 2 + lh) ^ swB) * 16;
+        const int ra = wm0 + l32, rb = wn0 + pcol;
+        aFrag[kk] = (ra >> 3) * 1024 + (ra & 7) * 64 + ((kk * 2 + lh) ^ sw) * 16;
+        bFrag[kk] = A_REGION + (rb >> 3) * 1024 + (rb & 7) * 64 + ((kk * 2 + lh) ^ swB) * 16;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const int kr = 16 * kk + 8 * lh + 4 * h + trRow;
-            aTr[kk][h] = (kr % A_NCH) * A_CP + (kr / A_NCH) * (BM * 2) + (wm0 + trCol) * 2;
-            bTr[kk][h] = A_BYTES + (kr % B_NCH) * B_CP + (kr / B_NCH) * (BN * 2) + (wn0 + trColB) * 2;
+            aTr[kk][h] = (kr % 16) * MN_CP + (kr / 16) * (BM * 2) + (wm0 + trCol) * 2;
+            bTr[kk][h] = A_REGION + (kr % 16) * MN_CP + (kr / 16) * (BN * 2) + (wn0 + trColB) * 2;
         }
     }
+    /* where slab kt of an operand begins inside its region */
+    auto slab_base = [&](bool kc, int kt) {
+        return kc ? ((kt >> 1) & 1) * KC_SLOT + (kt & 1) * 512 : (kt & 3) * MN_STAGE;
+    };
 
     f16x8 fa[KS][TI], fb[KS][TJ];
-    auto read_frags = [&](const char * stage) {
+    auto read_frags = [&](int kt) {
+        const char * sa = lds + slab_base(AKC, kt), * sb = lds + slab_base(BKC, kt);
 #pragma unroll
         for (int kk = 0; kk < KS; kk++) {
 #pragma unroll
             for (int i = 0; i < TI; i++) {
                 if constexpr (AKC)
-                    fa[kk][i] = *reinterpret_cast<const f16x8 *>(stage + aFrag[kk] + i * 32 * 64);
+                    fa[kk][i] = *reinterpret_cast<const f16x8 *>(sa + aFrag[kk] + i * 4096);
                 else {
-                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][0] + i * 64));
-                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][1] + i * 64));
+                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[kk][0] + i * 64));
+                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[kk][1] + i * 64));
                     fa[kk][i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 }
             }
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
                 if constexpr (BKC)
-                    fb[kk][j] = *reinterpret_cast<const f16x8 *>(stage + bFrag[kk] + j * 32 * 64);
+                    fb[kk][j] = *reinterpret_cast<const f16x8 *>(sb + bFrag[kk] + j * 4096);
                 else {
-                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][0] + j * 64));
-                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][1] + j * 64));
+                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[kk][0] + j * 64));
+                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[kk][1] + j * 64));
                     fb[kk][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 }
             }
@@ -234,43 +294,37 @@ gemm_f16_persistent_kernel(const GemmParams p)
 
     f32x16 acc[TI][TJ];
 
-    /* One slab: memory phase, barrier, compute phase, barrier (see the ping-pong loop of gemm_f16_direct_kernel).
-       AHEAD = how many later slabs exist (capped at 3); ISSUE: slab kt+3 exists and is not in flight yet; EXTRA:
-       stores of the previous tile that may still be in flight behind the loads this slab waits for. */
-    auto pp_slab = [&](auto AHEADC, auto ISSUEC, auto TAILC, auto EXTRAC, int kt) {
-        constexpr int ahead = decltype(AHEADC)::value;
-        const char * stage = lds + (kt % NSTAGE) * STAGE;
-        NTSAMD_FINE(0);
-        if constexpr (decltype(ISSUEC)::value != 0)
-            issue_loads(TAILC, kt + 3);
-        read_frags(stage);
-        NTSAMD_FINE(1);
-        wait_vmcnt<(ahead >= 3 ? 2 : (ahead == 2 ? 1 : 0)) * NL + decltype(EXTRAC)::value>();
-        wait_lgkmcnt0();
-        NTSAMD_FINE(2);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        NTSAMD_FINE(3);
-        __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-        for (int kk = 0; kk < KS; kk++)
-#pragma unroll
-            for (int g = 0; g < NM; g++) {
-                const int i = g / TJ, j = g % TJ;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
-            }
-        __builtin_amdgcn_s_setprio(0);
-        __builtin_amdgcn_sched_barrier(0);
-        NTSAMD_FINE(4);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        NTSAMD_FINE(5);
+    /* s_waitcnt takes its count as a constant: the handful of counts the loop below asks for, picked by a scalar
+       branch (once per slab and wave) */
+    auto wait_vm = [&](int n) {
+        if (n == 0) wait_vmcnt<0>();
+        else if (n == MM) wait_vmcnt<MM>();
+        else if (n == 2 * MM) wait_vmcnt<2 * MM>();
+        else if (n == KK + MM) wait_vmcnt<KK + MM>();
+        else if (n == KK + 2 * MM) wait_vmcnt<KK + 2 * MM>();
+        else if (n == NST + KK + 2 * MM) wait_vmcnt<NST + KK + 2 * MM>();
+        else if (n == MM + KK + 2 * MM) wait_vmcnt<MM + KK + 2 * MM>();
+        else if (n == MM + NST + KK + 2 * MM) wait_vmcnt<MM + NST + KK + 2 * MM>();
+        else wait_vmcnt<0>();
     };
 
-    /* The main loop of one tile whose first four slabs are in flight. EXTRA: stores issued after those loads. */
-    auto main_loop = [&](auto EXTRAC, auto PROBEC) {
-        constexpr int pb = decltype(PROBEC)::value;      /* first time stamp of this tile */
-        (void)pb;
+    /* The main loop of one tile whose first four slabs are in flight, requested as issue_two(0), `extra` other
+       operations (the previous tile's stores), issue_two(2). One slab is a memory phase, a barrier, a compute phase
+       and a barrier (see the ping-pong loop of gemm_f16_direct_kernel). At the start of its memory phase a wave may
+       overwrite the slabs before kt: an even slab (from 2 on) requests the pair (kt + 2, kt + 3) of the
+       k-contiguous operands, every slab (from 1 on) requests slab kt + 3 of the others, where they exist. When the
+       phase ends slab kt + 1 must be whole; what may still be in flight is what was requested after its last piece:
+         slab 0:  the previous tile's stores and slabs 2 and 3                                  extra + KK + 2 MM
+         even kt: the mn-contiguous slab kt + 2 (requested in slab kt - 1), the pair (kt + 2, kt + 3) and the
+                  mn-contiguous slab kt + 3 (both requested in slab kt)                          KK + 2 MM
+         odd kt:  the mn-contiguous slabs kt + 2 and kt + 3 (the pair that holds slab kt + 1 was requested in slab
+                  kt - 1, before them)                                                           2 MM
+         slab nk - 3: nothing comes after slab nk - 1: the pair (nk - 1, nk) if kt is even, and the mn-contiguous
+                  slab nk - 1                                                                    (KK +) MM
+         the last two slabs: nothing.
+       The loop is ONE copy of the slab's code whatever kt is (the compiler spilled accumulators when the first and
+       last slabs had copies of their own: fourteen of them). */
+    auto main_loop = [&](int extra) {
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -278,30 +332,75 @@ gemm_f16_persistent_kernel(const GemmParams p)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     acc[i][j][r] = 0.f;
-        wait_vmcnt<3 * NL + decltype(EXTRAC)::value>();
+        /* slab 0 is whole: after its last piece came its neighbour's mn-contiguous part, the stores, and slabs 2 and 3 */
+        wait_vm(MM + extra + KK + 2 * MM);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         if (follower)
             __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        NTSAMD_STAMP(pb);
-        pp_slab(IntC<3>(), IntC<0>(), IntC<0>(), EXTRAC, 0);
-        pp_slab(IntC<3>(), IntC<1>(), IntC<0>(), IntC<0>(), 1);   /* nk >= 8: slabs 4 and 5 are complete */
-        pp_slab(IntC<3>(), IntC<1>(), IntC<0>(), IntC<0>(), 2);
-        NTSAMD_STAMP(pb + 1);
-        int kt = 3;
-#ifdef NTSAMD_PROBE
-        pp_slab(IntC<3>(), IntC<1>(), IntC<0>(), IntC<0>(), kt);
-        kt++;
-        NTSAMD_STAMP(pb + 2);
-#endif
-        for (; kt + 3 < nkFull; kt++)
-            pp_slab(IntC<3>(), IntC<1>(), IntC<0>(), IntC<0>(), kt);
+        NTSAMD_STAMP(extra ? 7 : 1);
+        /* the second half of a slab: barrier, the slab's MFMAs at raised priority, barrier */
+        auto compute = [&](int kt) {
+            (void)kt;
+            wait_lgkmcnt0();
+            NTSAMD_FINE(2);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            NTSAMD_FINE(3);
+            __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+                for (int g = 0; g < NM; g++) {
+                    const int i = g / TJ, j = g % TJ;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+                }
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            NTSAMD_FINE(4);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            NTSAMD_FINE(5);
+        };
+        /* One slab. ISSUE: 2 = it requests the pair (kt + 2, kt + 3) if kt is even and slab kt + 3 of the
+           mn-contiguous operands, 1 = the pair only, 0 = nothing. What may stay in flight is a constant for odd kt
+           and one for even kt. (Written with the slab's place in the tile as compile-time flags and few copies: a
+           single loop over all slabs with everything tested at run time, and a copy per distinct slab, both made
+           the compiler move or spill accumulators.) */
+        auto slab = [&](auto ISSUEC, auto ODDC, auto EVENC, int kt) {
+            constexpr int ISSUE = decltype(ISSUEC)::value;
+            const bool odd = (kt & 1) != 0;
+            if constexpr (ISSUE >= 1 && KK > 0) {
+                if (!odd)
+                    issue_pair(kt + 2);
+            }
+            if constexpr (ISSUE >= 2 && MM > 0)
+                issue_slab(kt + 3);
+            read_frags(kt);
+            if constexpr (decltype(ODDC)::value == decltype(EVENC)::value)
+                wait_vmcnt<decltype(ODDC)::value>();
+            else {
+                if (odd)
+                    wait_vmcnt<decltype(ODDC)::value>();
+                else
+                    wait_vmcnt<decltype(EVENC)::value>();
+            }
+            compute(kt);
+        };
+        /* slab 0 requests nothing (slabs 2 and 3 are in flight) and counts the previous tile's stores */
+        read_frags(0);
+        if (extra)
+            wait_vmcnt<NST + KK + 2 * MM>();
+        else
+            wait_vmcnt<KK + 2 * MM>();
+        compute(0);
+        int kt = 1;
         for (; kt + 3 < nk; kt++)
-            pp_slab(IntC<3>(), IntC<1>(), IntC<1>(), IntC<0>(), kt);
-        pp_slab(IntC<2>(), IntC<0>(), IntC<0>(), IntC<0>(), kt);
-        pp_slab(IntC<1>(), IntC<0>(), IntC<0>(), IntC<0>(), kt + 1);
-        pp_slab(IntC<0>(), IntC<0>(), IntC<0>(), IntC<0>(), kt + 2);
+            slab(IntC<2>(), IntC<2 * MM>(), IntC<KK + 2 * MM>(), kt);
+        slab(IntC<1>(), IntC<MM>(), IntC<KK + MM>(), kt);          /* slab nk - 3: after slab nk - 1 of the mn-contiguous operands nothing is requested */
+        slab(IntC<0>(), IntC<0>(), IntC<0>(), kt + 1);
+        slab(IntC<0>(), IntC<0>(), IntC<0>(), kt + 2);
         if (!follower)
             __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -325,7 +424,8 @@ gemm_f16_persistent_kernel(const GemmParams p)
         const int rdRow = lane >> 3, rdChunk = lane & 7;
         const int colW = en0 + wn0 + rdChunk * 8;
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
-        char * mine = lds + 2 * STAGE + wave * EPI_WAVE;
+        /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's */
+        char * mine = lds + (wave < 4 ? A_HALF : A_REGION + B_HALF) + (wave & 3) * EPI_WAVE;
         char * wr = mine + l32 * EPI_PITCH + lh * 16;
         const char * rd = mine + rdRow * EPI_PITCH + rdChunk * 16;
 #pragma unroll
@@ -364,23 +464,22 @@ gemm_f16_persistent_kernel(const GemmParams p)
     if (id >= total)
         return;
     NTSAMD_STAMP(0);
-    setup(id);
-    issue_loads(IntC<0>(), 0);
-    issue_loads(IntC<0>(), 1);
-    issue_loads(IntC<0>(), 2);
-    issue_loads(IntC<0>(), 3);
-    main_loop(IntC<0>(), IntC<1>());
-    NTSAMD_STAMP(4);
+    adopt(locate(id));
+    issue_two(0);
+    issue_two(2);
+    int extra = 0;
     for (;;) {
+        id += (int)gridDim.x;
+        const bool more = id < total;
+        const Loc next = locate(more ? id : 0);          /* while the first slab is on its way */
+        main_loop(extra);
+        NTSAMD_STAMP(extra ? 10 : 4);
         /* every wave has passed the last barrier of the main loop: nobody reads the stages any more */
         const int em0 = m0, en0 = n0;
         half_t * eC = C;
-        id += (int)gridDim.x;
-        const bool more = id < total;
         if (more) {
-            setup(id);
-            issue_loads(IntC<0>(), 0);
-            issue_loads(IntC<0>(), 1);
+            adopt(next);
+            issue_two(0);
         }
         __builtin_amdgcn_sched_barrier(0);
         NTSAMD_STAMP(more ? 5 : 11);
@@ -389,32 +488,20 @@ gemm_f16_persistent_kernel(const GemmParams p)
         NTSAMD_STAMP(more ? 6 : 12);
         if (!more)
             break;
-        /* stages 2 and 3 are free once every wave has read its staged rows back */
+        /* where slabs 2 and 3 go is free once every wave has read its staged rows back */
         wait_lgkmcnt0();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue_loads(IntC<0>(), 2);
-        issue_loads(IntC<0>(), 3);
-        main_loop(IntC<NST>(), IntC<7>());
-        NTSAMD_STAMP(10);
+        issue_two(2);
+        extra = NST;
     }
 #ifdef NTSAMD_PROBE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     NTSAMD_STAMP(13);
     if (tid == 0) {
         unsigned long long * out = const_cast<unsigned long long *>(static_cast<const unsigned long long *>(p.bias)) + (size_t)blockIdx.x * 16;
-#pragma unroll
         for (int n = 0; n < 16; n++)
-            out[n] = st[n];
-    }
-    if (lane == 0 && (wave == 0 || wave == 4)) {
-        unsigned long long * out = const_cast<unsigned long long *>(static_cast<const unsigned long long *>(p.bias)) +
-                                   (size_t)gridDim.x * 16 + ((size_t)blockIdx.x * 2 + wave / 4) * 8;
-#pragma unroll
-        for (int n = 0; n < 6; n++)
-            out[n] = fine[n];
-        out[6] = __builtin_amdgcn_s_memtime();
-        out[7] = __builtin_amdgcn_s_memrealtime();
+            out[n] = stampLds[n];
     }
 #endif
 }

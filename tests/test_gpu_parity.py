@@ -764,6 +764,41 @@ def test_config4_half_tn(gpu, oracle):
     assert float((c2.float() - 2 * c.float())[~normal].abs().max()) <= 2.0 ** -24
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_walk_over_more_tiles_than_cus(gpu, oracle, ta, tb):
+    """More 256 x 256 tiles than the part has CUs: one workgroup per CU walks over them, fetches the next tile while
+    the finished one leaves, and requests k-contiguous operands two slabs at a time. Ragged edges in m and n, a k
+    that ends inside a slab and inside a pair of slabs, odd and even numbers of slabs, batches; every element against
+    double precision, and bit for bit against the one-tile-per-workgroup kernels (the sums run in the same order)."""
+    torch = torch_()
+    knobs = ("NTSAMD_TILE_CFG", "NTSAMD_F16_PINGPONG", "NTSAMD_F16_PERSIST")
+    try:
+        for i, (M, N, K, batch) in enumerate(((4100, 4360, 264, 1), (4360, 4100, 1000, 1), (4352, 4352, 328, 1),
+                                              (1100, 1300, 296, 9))):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch,) + stored((M, K), ta), 7100 + i, 0, 0.05)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch,) + stored((K, N), tb), 7200 + i, 0, 0.05)))
+            ga, gb = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True)
+            got = {}
+            for walk in (1, 0):
+                for key, val in zip(knobs, (2, walk, walk)):
+                    nt.tuning_set(key, val)
+                c = torch.full((batch, M, N), float("nan"), device=gpu, dtype=torch.float16)
+                if batch == 1:
+                    nt.matrix_mul(ga[0], ta, gb[0], tb, c[0], 0.75, 0.0)
+                else:
+                    na, ma = a.shape[1:]
+                    nb, mb = b.shape[1:]
+                    nt.matrix_mul_batched_strided(ga, ta, gb, tb, c, batch, na * ma, nb * mb, M * N, na, ma, nb, mb, M, N, 0.75, 0.0)
+                got[walk] = c
+            assert torch.equal(got[1], got[0]), "%dx%dx%d x%d: the walk and the one-tile kernels differ" % (M, N, K, batch)
+            res = got[1].float().cpu().numpy()
+            for item in range(batch):
+                assert_fp16(res[item], 0.75 * whole_f64(a[item], ta, b[item], tb), what="%dx%dx%d item %d" % (M, N, K, item))
+    finally:
+        for key in knobs:
+            nt.tuning_set(key, None)
+
+
 def test_config5_ragged_vocab_projection(gpu, oracle):
     """fp32 H[4096x512] x W[30011x512]^T accumulated into C[4096x30011] with beta = 1."""
     torch = torch_()
