@@ -56,24 +56,28 @@ template <bool AKC, bool BKC>
 __global__ void __launch_bounds__(512, 1)
 gemm_f16_persistent_kernel(const GemmParams p)
 {
-    constexpr int BM = 256, BN = 256, WGN = 4, NW = 8, BKT = 32, KS = 2;
-    constexpr int WM = 128, WN = 64, TI = 4, TJ = 2, NM = TI * TJ;
+    constexpr int BM = 256, BN = 256, WGN = 4, NW = 8, BKT = 32;
+    constexpr int WM = 128, WN = 64, TI = WM / 16, TJ = WN / 16;      /* 16 x 16 blocks of v_mfma_f32_16x16x32_f16: a slab is ONE k step */
     /* LDS, one region per operand, four slabs each.
        k-contiguous: two pair slots of 32 KB; a chunk of 1 KB holds 8 rows x [slab parity][64 bytes], the four 16-byte
            columns of a row's 64 bytes permuted by (row >> 2) & 3 (sixteen consecutive rows reading one logical
            column hit sixteen different 16-byte bank groups: rows r, r+4, r+8, r+12 share 64 bytes of a 256-byte line).
-       mn-contiguous: four stages of 16 chunks (k rows c and c+16, 512 bytes each), chunks 1088 bytes apart. */
+       mn-contiguous: four stages of 16 chunks (k rows c and c+16, 512 bytes each), chunks 1088 bytes apart and
+           chunks 8-15 another 32 bytes on: a transposing read of lanes 0-31 takes 32 bytes from each of k rows s and
+           8 + s (s = 0..3), i.e. from chunks s and 8 + s, which then lie 64 s and 64 s + 32 bytes into a 256-byte
+           line of the 64 banks. */
     constexpr int KC_SLOT = 32 * 1024, KC_REGION = 2 * KC_SLOT;
-    constexpr int MN_CP = 1088, MN_STAGE = 16 * MN_CP, MN_REGION = 4 * MN_STAGE;
+    constexpr int MN_CP = 1088, MN_STAGE = 69 * 256, MN_REGION = 4 * MN_STAGE;
+    static_assert(15 * MN_CP + 32 + 1024 <= MN_STAGE, "sixteen chunks must fit a stage");
     constexpr int A_REGION = AKC ? KC_REGION : MN_REGION, B_REGION = BKC ? KC_REGION : MN_REGION;
     constexpr int A_HALF = AKC ? KC_SLOT : 2 * MN_STAGE, B_HALF = BKC ? KC_SLOT : 2 * MN_STAGE;   /* where slabs 2 and 3 begin */
     /* load instructions per wave: KA, KB per PAIR of slabs (k-contiguous), MA, MB per slab (mn-contiguous) */
     constexpr int KA = AKC ? 4 : 0, KB = BKC ? 4 : 0, MA = AKC ? 0 : 2, MB = BKC ? 0 : 2;
     constexpr int KK = KA + KB, MM = MA + MB;
-    /* the epilogue's turn through LDS: 32 rows of the wave's 64 columns as halves, rows 144 bytes apart (sixteen
-       lanes that write 16 bytes each to sixteen consecutive rows then cover all 64 banks) */
-    constexpr int EPI_PITCH = WN * 2 + 16, EPI_WAVE = 32 * EPI_PITCH;
-    constexpr int NST = TI * 4;                     /* store instructions per wave and tile: 8 rows of 128 bytes each */
+    /* the epilogue's turn through LDS: 16 rows of the wave's 64 columns as halves, rows 144 bytes apart (32 lanes
+       that write 8 bytes each, 16 rows x 2 pieces, then cover all 64 banks) */
+    constexpr int EPI_PITCH = WN * 2 + 16, EPI_WAVE = 16 * EPI_PITCH;
+    constexpr int NST = TI * 2;                     /* store instructions per wave and tile: 8 rows of 128 bytes each */
     static_assert(4 * EPI_WAVE <= A_REGION - A_HALF && 4 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
     static_assert(A_REGION + B_REGION <= 160 * 1024, "the stages must fit LDS");
     static_assert(MM + NST + KK + 2 * MM < 64, "the wait counter has six bits");
@@ -94,7 +98,6 @@ gemm_f16_persistent_kernel(const GemmParams p)
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
-    const int l32 = lane & 31, lh = lane >> 5;
     const bool follower = wave >= NW / 2;
     const int nk = (K + BKT - 1) / BKT;                        /* the launcher guarantees nk >= 8 */
     const int total = p.tilesM * p.tilesN * p.batch;
@@ -213,14 +216,14 @@ gemm_f16_persistent_kernel(const GemmParams p)
             const i32x4 ad = make_desc(ab, (long long)(aEnd - ab) * 2);
 #pragma unroll
             for (int q = 0; q < MA; q++)
-                lds_dma16(ad, ldsBase + stage + (unsigned)((wave * MA + q) * MN_CP), aOff[q]);
+                lds_dma16(ad, ldsBase + stage + (unsigned)((wave * MA + q) * MN_CP + 32 * ((wave * MA + q) >> 3)), aOff[q]);
         }
         if constexpr (!BKC) {
             const half_t * bb = bTile + (size_t)k0 * p.ldb;
             const i32x4 bd = make_desc(bb, (long long)(bEnd - bb) * 2);
 #pragma unroll
             for (int q = 0; q < MB; q++)
-                lds_dma16(bd, ldsBase + (unsigned)A_REGION + stage + (unsigned)((wave * MB + q) * MN_CP), bOff[q]);
+                lds_dma16(bd, ldsBase + (unsigned)A_REGION + stage + (unsigned)((wave * MB + q) * MN_CP + 32 * ((wave * MB + q) >> 3)), bOff[q]);
         }
     };
     /* slabs kt and kt + 1 (kt even) of both operands, in the order the waits below count on: the pair, then the
@@ -232,31 +235,26 @@ gemm_f16_persistent_kernel(const GemmParams p)
     };
 
     /* ---- fragment addresses (byte offsets inside the operand's region, slab 0) ----------- */
-    /* The b fragment is the FIRST operand of the MFMA here: its lane rho (0..31) supplies the result's ROW rho, and
-       result register r of a lane with half-wave h holds row 8 (r/4) + 4 h + r%4. Column pcol(rho) of the b block
-       goes to fragment lane rho, with groups of four columns dealt out as
-           group q = rho / 4 = (q2 q1 q0)  ->  columns 4 (q2 q0 q1) .. + 3   (the two low bits of the group swap)
-       so that registers 8 g .. 8 g + 7 of a lane are columns 16 g + 8 h .. + 7 of the block. */
-    const int q3 = l32 >> 2;
-    const int pcol = 4 * ((q3 & 4) | ((q3 & 1) << 1) | ((q3 >> 1) & 1)) + (l32 & 3);
-    const int trRow = (lane & 15) >> 2;
-    const int trCol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    /* a transposing read hands result lane c the piece of four columns that address lanes with (lane & 3) == c / 4
-       point at: the same exchange of the two low bits of the group number, on the addresses */
-    const int trColB = 16 * ((lane >> 4) & 1) + 8 * (lane & 1) + 4 * ((lane >> 1) & 1);
-    int aFrag[KS], bFrag[KS];
-    int aTr[KS][2], bTr[KS][2];
-#pragma unroll
-    for (int kk = 0; kk < KS; kk++) {
-        const int sw = (l32 >> 2) & 3, swB = (pcol >> 2) & 3;
-        const int ra = wm0 + l32, rb = wn0 + pcol;
-        aFrag[kk] = (ra >> 3) * 1024 + (ra & 7) * 64 + ((kk * 2 + lh) ^ sw) * 16;
-        bFrag[kk] = A_REGION + (rb >> 3) * 1024 + (rb & 7) * 64 + ((kk * 2 + lh) ^ swB) * 16;
+    /* v_mfma_f32_16x16x32_f16: lane l of either operand holds index l % 16 of its block and k = 8 (l / 16) .. + 7; the
+       b fragment is the FIRST operand here, so that result register r of lane l is row l % 16 of the block of c (the
+       a fragment's index) and column 4 (l / 16) + r (the b fragment's index): a lane holds four consecutive columns
+       of one row, 8 bytes of c.
+       k-contiguous: row + 16-byte column of a pair chunk, the column permuted by (row >> 2) & 3.
+       mn-contiguous: two transposing reads, each of which hands a lane four consecutive k (k rows 8 g + 4 h + s,
+       s = 0..3, pointed at by address lanes 4 s + q with their four columns 4 q .. 4 q + 3). */
+    const int rho = lane & 15, g4 = lane >> 4;
+    int aFrag = 0, bFrag = 0, aTr[2] = {0, 0}, bTr[2] = {0, 0};
+    {
+        const int ra = wm0 + rho, rb = wn0 + rho;
+        const int sw = (rho >> 2) & 3;
+        aFrag = (ra >> 3) * 1024 + (ra & 7) * 64 + ((g4 ^ sw) * 16);
+        bFrag = A_REGION + (rb >> 3) * 1024 + (rb & 7) * 64 + ((g4 ^ sw) * 16);
+        const int s4 = rho >> 2, q4 = rho & 3;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            const int kr = 16 * kk + 8 * lh + 4 * h + trRow;
-            aTr[kk][h] = (kr % 16) * MN_CP + (kr / 16) * (BM * 2) + (wm0 + trCol) * 2;
-            bTr[kk][h] = A_REGION + (kr % 16) * MN_CP + (kr / 16) * (BN * 2) + (wn0 + trColB) * 2;
+            const int kr = 8 * g4 + 4 * h + s4, ch = kr & 15;
+            aTr[h] = ch * MN_CP + 32 * (ch >> 3) + (kr >> 4) * (BM * 2) + (wm0 + 4 * q4) * 2;
+            bTr[h] = A_REGION + ch * MN_CP + 32 * (ch >> 3) + (kr >> 4) * (BN * 2) + (wn0 + 4 * q4) * 2;
         }
     }
     /* where slab kt of an operand begins inside its region */
@@ -264,35 +262,32 @@ gemm_f16_persistent_kernel(const GemmParams p)
         return kc ? ((kt >> 1) & 1) * KC_SLOT + (kt & 1) * 512 : (kt & 3) * MN_STAGE;
     };
 
-    f16x8 fa[KS][TI], fb[KS][TJ];
+    f16x8 fa[TI], fb[TJ];
     auto read_frags = [&](int kt) {
         const char * sa = lds + slab_base(AKC, kt), * sb = lds + slab_base(BKC, kt);
 #pragma unroll
-        for (int kk = 0; kk < KS; kk++) {
-#pragma unroll
-            for (int i = 0; i < TI; i++) {
-                if constexpr (AKC)
-                    fa[kk][i] = *reinterpret_cast<const f16x8 *>(sa + aFrag[kk] + i * 4096);
-                else {
-                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[kk][0] + i * 64));
-                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[kk][1] + i * 64));
-                    fa[kk][i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
+        for (int i = 0; i < TI; i++) {
+            if constexpr (AKC)
+                fa[i] = *reinterpret_cast<const f16x8 *>(sa + aFrag + i * 2048);
+            else {
+                f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[0] + i * 32));
+                f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sa + aTr[1] + i * 32));
+                fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
+        }
 #pragma unroll
-            for (int j = 0; j < TJ; j++) {
-                if constexpr (BKC)
-                    fb[kk][j] = *reinterpret_cast<const f16x8 *>(sb + bFrag[kk] + j * 4096);
-                else {
-                    f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[kk][0] + j * 64));
-                    f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[kk][1] + j * 64));
-                    fb[kk][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
+        for (int j = 0; j < TJ; j++) {
+            if constexpr (BKC)
+                fb[j] = *reinterpret_cast<const f16x8 *>(sb + bFrag + j * 2048);
+            else {
+                f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[0] + j * 32));
+                f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(sb + bTr[1] + j * 32));
+                fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
         }
     };
 
-    f32x16 acc[TI][TJ];
+    f32x4 acc[TI][TJ];
 
     /* s_waitcnt takes its count as a constant: the handful of counts the loop below asks for, picked by a scalar
        branch (once per slab and wave) */
@@ -329,9 +324,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
         for (int i = 0; i < TI; i++)
 #pragma unroll
             for (int j = 0; j < TJ; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    acc[i][j][r] = 0.f;
+                acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         /* slab 0 is whole: after its last piece came its neighbour's mn-contiguous part, the stores, and slabs 2 and 3 */
         wait_vm(MM + extra + KK + 2 * MM);
         __builtin_amdgcn_s_barrier();
@@ -350,12 +343,10 @@ gemm_f16_persistent_kernel(const GemmParams p)
             NTSAMD_FINE(3);
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-            for (int kk = 0; kk < KS; kk++)
+            for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int g = 0; g < NM; g++) {
-                    const int i = g / TJ, j = g % TJ;
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
-                }
+                for (int j = 0; j < TJ; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
             NTSAMD_FINE(4);
@@ -406,12 +397,11 @@ gemm_f16_persistent_kernel(const GemmParams p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    /* ---- epilogue of the tile at (em0, en0) of eC: accumulator register r of lane (l32, lh) is row l32 of its
-       block of c and, by the permutation above, column 16 (r/8) + 8 lh + r%8: eight consecutive registers are 16
-       bytes of one row. Block row by block row the wave writes them to its own piece of LDS as rows of 64 halves and
-       reads whole rows back, 8 lanes to a row: every store instruction covers 8 rows of 128 contiguous bytes. The
-       wave's rows of c are one buffer that ends where c ends: rows past M drop off it, columns past N are sent out
-       of range (N is a multiple of 8 here). -------------------------------------------------------------------- */
+    /* ---- epilogue of the tile at (em0, en0) of eC: accumulator register r of lane (rho, g4) is row rho of its block
+       of c and column 4 g4 + r. Block row by block row (16 rows) the wave writes its 8-byte pieces to its own piece
+       of LDS as rows of 64 halves and reads whole rows back, 8 lanes to a row: every store instruction covers 8 rows
+       of 128 contiguous bytes. The wave's rows of c are one buffer that ends where c ends: rows past M drop off it,
+       columns past N are sent out of range (N is a multiple of 8 here). ---------------------------------------- */
     auto epilogue = [&](int em0, int en0, half_t * eC) {
         const float alpha = p.alpha;
         const int act = p.act;
@@ -426,29 +416,27 @@ gemm_f16_persistent_kernel(const GemmParams p)
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
         /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's */
         char * mine = lds + (wave < 4 ? A_HALF : A_REGION + B_HALF) + (wave & 3) * EPI_WAVE;
-        char * wr = mine + l32 * EPI_PITCH + lh * 16;
+        char * wr = mine + rho * EPI_PITCH + g4 * 8;
         const char * rd = mine + rdRow * EPI_PITCH + rdChunk * 16;
 #pragma unroll
         for (int i = 0; i < TI; i++) {
 #pragma unroll
-            for (int j = 0; j < TJ; j++)
+            for (int j = 0; j < TJ; j++) {
+                f16x4 v;
 #pragma unroll
-                for (int g = 0; g < 2; g++) {
-                    f16x8 v;
-#pragma unroll
-                    for (int e = 0; e < 8; e++)
-                        v[e] = (half_t)activate(alpha * acc[i][j][8 * g + e], act);
-                    *reinterpret_cast<f16x8 *>(wr + (j * 32 + 16 * g) * 2) = v;
-                }
+                for (int e = 0; e < 4; e++)
+                    v[e] = (half_t)activate(alpha * acc[i][j][e], act);
+                *reinterpret_cast<f16x4 *>(wr + j * 32) = v;
+            }
             /* the wave's own lanes exchange data through LDS: LDS executes one wave's instructions in order, the
                fences only keep the compiler from reordering */
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
+            for (int q = 0; q < 2; q++) {
                 const f32x4 v = *reinterpret_cast<const f32x4 *>(rd + q * 8 * EPI_PITCH);
-                const int off = (int)(cOffW + (unsigned)(i * 32 + q * 8) * rowPitch);
+                const int off = (int)(cOffW + (unsigned)(i * 16 + q * 8) * rowPitch);
                 if (p.storeHint)
                     __builtin_amdgcn_raw_buffer_store_b128(v, cr, off, 0, STORE_WRITE_THROUGH);
                 else
