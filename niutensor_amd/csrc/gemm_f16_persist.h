@@ -78,7 +78,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
        that write 8 bytes each, 16 rows x 2 pieces, then cover all 64 banks) */
     constexpr int EPI_PITCH = WN * 2 + 16, EPI_WAVE = 16 * EPI_PITCH;
     constexpr int NST = TI * 2;                     /* store instructions per wave and tile: 8 rows of 128 bytes each */
-    static_assert(4 * EPI_WAVE <= A_REGION - A_HALF && 4 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
+    static_assert(8 * EPI_WAVE <= A_REGION - A_HALF && 8 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
     static_assert(A_REGION + B_REGION <= 160 * 1024, "the stages must fit LDS");
     static_assert(MM + NST + KK + 2 * MM < 64, "the wait counter has six bits");
 
@@ -342,11 +342,15 @@ gemm_f16_persistent_kernel(const GemmParams p)
             __builtin_amdgcn_sched_barrier(0);
             NTSAMD_FINE(3);
             __builtin_amdgcn_s_setprio(1);
+            /* block rows forth and back: every second row keeps the b fragment of the MFMA before it (a little less
+               switching at the matrix pipe's inputs: 1-2 % of the run time on random data) */
 #pragma unroll
             for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int j = 0; j < TJ; j++)
+                for (int jj = 0; jj < TJ; jj++) {
+                    const int j = (i & 1) ? TJ - 1 - jj : jj;
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                }
             __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
             NTSAMD_FINE(4);
@@ -402,9 +406,13 @@ gemm_f16_persistent_kernel(const GemmParams p)
        of LDS as rows of 64 halves and reads whole rows back, 8 lanes to a row: every store instruction covers 8 rows
        of 128 contiguous bytes. The wave's rows of c are one buffer that ends where c ends: rows past M drop off it,
        columns past N are sent out of range (N is a multiple of 8 here). ---------------------------------------- */
-    auto epilogue = [&](int em0, int en0, half_t * eC) {
+    auto epilogue_as = [&](auto ACTC, auto THROUGHC, int em0, int en0, half_t * eC) {
+        /* whether there is an activation and how the stores treat the caches are constants of this copy of the code:
+           tested per element, the activation made the epilogue four vector instructions per value, 512 per lane,
+           and with two waves to a SIMD that, not the stores, was what the 3.6 us between two tiles were made of */
+        constexpr int act = decltype(ACTC)::value;
+        constexpr int aux = decltype(THROUGHC)::value ? STORE_WRITE_THROUGH : STORE_DEFAULT;
         const float alpha = p.alpha;
-        const int act = p.act;
         /* a wave whose rows lie past M stores into a buffer of no bytes: every store is dropped, but every store is
            ISSUED, so that all waves have the same number of operations in flight (the waits count them) */
         const int rowsLeft = M - em0 - wm0 > 0 ? M - em0 - wm0 : 0;
@@ -414,12 +422,11 @@ gemm_f16_persistent_kernel(const GemmParams p)
         const int rdRow = lane >> 3, rdChunk = lane & 7;
         const int colW = en0 + wn0 + rdChunk * 8;
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
-        /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's */
-        char * mine = lds + (wave < 4 ? A_HALF : A_REGION + B_HALF) + (wave & 3) * EPI_WAVE;
-        char * wr = mine + rho * EPI_PITCH + g4 * 8;
-        const char * rd = mine + rdRow * EPI_PITCH + rdChunk * 16;
-#pragma unroll
-        for (int i = 0; i < TI; i++) {
+        /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's; two buffers per wave, so
+           that block row i + 1 is on its way into LDS while block row i comes back out */
+        char * mine = lds + (wave < 4 ? A_HALF : A_REGION + B_HALF) + (wave & 3) * (2 * EPI_WAVE);
+        auto put = [&](int i) {
+            char * wr = mine + (i & 1) * EPI_WAVE + rho * EPI_PITCH + g4 * 8;
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
                 f16x4 v;
@@ -428,22 +435,39 @@ gemm_f16_persistent_kernel(const GemmParams p)
                     v[e] = (half_t)activate(alpha * acc[i][j][e], act);
                 *reinterpret_cast<f16x4 *>(wr + j * 32) = v;
             }
+        };
+        put(0);
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
             /* the wave's own lanes exchange data through LDS: LDS executes one wave's instructions in order, the
                fences only keep the compiler from reordering */
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const char * rd = mine + (i & 1) * EPI_WAVE + rdRow * EPI_PITCH + rdChunk * 16;
+            f32x4 v[2];
 #pragma unroll
-            for (int q = 0; q < 2; q++) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(rd + q * 8 * EPI_PITCH);
-                const int off = (int)(cOffW + (unsigned)(i * 16 + q * 8) * rowPitch);
-                if (p.storeHint)
-                    __builtin_amdgcn_raw_buffer_store_b128(v, cr, off, 0, STORE_WRITE_THROUGH);
-                else
-                    __builtin_amdgcn_raw_buffer_store_b128(v, cr, off, 0, STORE_DEFAULT);
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
+            for (int q = 0; q < 2; q++)
+                v[q] = *reinterpret_cast<const f32x4 *>(rd + q * 8 * EPI_PITCH);
+            if (i + 1 < TI)
+                put(i + 1);
+#pragma unroll
+            for (int q = 0; q < 2; q++)
+                __builtin_amdgcn_raw_buffer_store_b128(v[q], cr, (int)(cOffW + (unsigned)(i * 16 + q * 8) * rowPitch), 0, aux);
+        }
+    };
+    auto epilogue = [&](int em0, int en0, half_t * eC) {
+        if (p.act == ACT_RECTIFY) {
+            if (p.storeHint)
+                epilogue_as(IntC<ACT_RECTIFY>(), IntC<1>(), em0, en0, eC);
+            else
+                epilogue_as(IntC<ACT_RECTIFY>(), IntC<0>(), em0, en0, eC);
+        }
+        else {
+            if (p.storeHint)
+                epilogue_as(IntC<ACT_NONE>(), IntC<1>(), em0, en0, eC);
+            else
+                epilogue_as(IntC<ACT_NONE>(), IntC<0>(), em0, en0, eC);
         }
     };
 

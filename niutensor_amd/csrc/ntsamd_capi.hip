@@ -240,9 +240,10 @@ struct Plan {
      NTSAMD_F32_SPLIT_ATOMIC=1   float pieces of k add to c with atomics (no workspace, no fixed order)
      NTSAMD_F16_PINGPONG=0       half, 256 x 256 tile: the main loop in which both waves of a SIMD meet one barrier
      NTSAMD_F16_PERSIST=0        half, 256 x 256 tile: one workgroup per tile, never one per CU that walks over tiles
-     NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment */
+     NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment
+     NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset) */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -256,7 +257,7 @@ const Knob g_knobs[] = {
     {"NTSAMD_F16_FETCH", &Tuning::f16Fetch}, {"NTSAMD_ATTN_ROWS", &Tuning::attnRows},
     {"NTSAMD_F32_R16", &Tuning::f32R16},     {"NTSAMD_F32_SPLIT_ATOMIC", &Tuning::f32SplitAtomic},
     {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
-    {"NTSAMD_STORE_HINT", &Tuning::storeHint},
+    {"NTSAMD_STORE_HINT", &Tuning::storeHint}, {"NTSAMD_GROUP_M", &Tuning::groupM},
 };
 
 const Tuning & tuning()
@@ -505,7 +506,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.biasRowDiv = biasRowDiv > 0 ? biasRowDiv : 1;
     p.biasLen = biasLen > 0 ? biasLen : 1;
     p.batch = count;
-    p.groupM = 8;
+    p.groupM = tn.groupM.load(std::memory_order_relaxed) > 0 ? tn.groupM.load(std::memory_order_relaxed) : 8;     /* the half walk over tiles takes 4 (see where it is chosen) */
     p.act = act;
     p.wideRowsOnly = tn.f32R16.load(std::memory_order_relaxed) == 0;
     p.f16PingPong = tn.f16PingPong.load(std::memory_order_relaxed) != 0;
@@ -609,6 +610,11 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                           (!grid || grid->strideC1 % 8 == 0);
         if (wide && cus > 0 && tiles > cus)
             p.persistGrid = cus;
+            /* four tile rows share a sweep over the tile columns: the 32 tiles an XCD works on at a time are 4 x 8,
+               the same twelve operand panels as 8 x 4, and their stores spread over twice as many columns of c
+               (measured 1-2 % ahead of 8 at 8192 x 4096 x 1024, level elsewhere) */
+            if (tn.groupM.load(std::memory_order_relaxed) <= 0)
+                p.groupM = 4;
     }
     p.splits = 1;
     if (plan.splits > 1) {
