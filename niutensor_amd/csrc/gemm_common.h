@@ -29,7 +29,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
    of half results, 1.4 of 10.4 us on the attention-shaped batches), while lines written through leave during the
    kernel. Only for results whose rows are whole 128-byte lines: written through in pieces of lines (rows of
    30011 floats) the same stores were 4 % slower than the default. */
-constexpr int STORE_DEFAULT = 0, STORE_WRITE_THROUGH = 17;
+constexpr int STORE_DEFAULT = 0, STORE_WRITE_THROUGH = 17, STORE_STREAM = 2;      /* nt = 2: the line is the first to leave the cache again */
 
 enum BiasMode { BIAS_NONE = 0, BIAS_COL = 1, BIAS_ROW = 2 };
 

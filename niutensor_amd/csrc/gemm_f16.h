@@ -142,7 +142,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     const int M = p.M, N = p.N, K = p.K;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);      /* the same in every lane: said explicitly, so that descriptors built from it are scalars */
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
     const int l32 = lane & 31, lh = lane >> 5;
 

@@ -115,7 +115,9 @@ gemm_f32_kernel(const GemmParams p, const PT tab)
     /* R16: a workgroup multiplies the first 16 rows of what it stages, and the workgroups stand 16 rows apart */
     const int m0 = tc.tm * (R16 ? 16 : BM), n0 = tc.tn * BN;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    /* the wave number is the same in every lane: said explicitly, or every buffer access whose descriptor is built
+       from it (the epilogue's 64 stores per lane) is wrapped in a loop that tests the descriptor lane by lane */
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
     const int l32 = R16 ? (lane & 15) : (lane & 31);      /* row / column inside a block */
     const int lh = R16 ? (lane >> 4) : (lane >> 5);        /* k slot */

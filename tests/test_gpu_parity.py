@@ -769,7 +769,7 @@ def test_half_walk_over_more_tiles_than_cus(gpu, oracle, ta, tb):
     """More 256 x 256 tiles than the part has CUs: one workgroup per CU walks over them, fetches the next tile while
     the finished one leaves, and requests k-contiguous operands two slabs at a time. Ragged edges in m and n, a k
     that ends inside a slab and inside a pair of slabs, odd and even numbers of slabs, batches; every element against
-    double precision, and bit for bit against the one-tile-per-workgroup kernels (the sums run in the same order)."""
+    double precision, and to the last half bit against the one-tile-per-workgroup kernels."""
     torch = torch_()
     knobs = ("NTSAMD_TILE_CFG", "NTSAMD_F16_PINGPONG", "NTSAMD_F16_PERSIST")
     try:
@@ -790,7 +790,12 @@ def test_half_walk_over_more_tiles_than_cus(gpu, oracle, ta, tb):
                     nb, mb = b.shape[1:]
                     nt.matrix_mul_batched_strided(ga, ta, gb, tb, c, batch, na * ma, nb * mb, M * N, na, ma, nb, mb, M, N, 0.75, 0.0)
                 got[walk] = c
-            assert torch.equal(got[1], got[0]), "%dx%dx%d x%d: the walk and the one-tile kernels differ" % (M, N, K, batch)
+            # the walk multiplies 16 x 16 x 32 blocks, the one-tile kernels 32 x 32 x 16: the same products summed in
+            # another order inside the matrix pipe, so a sum next to a rounding boundary may come out one half apart
+            w, o = got[1].float(), got[0].float()
+            step = torch.maximum(w.abs(), o.abs()) * 2.0 ** -10 + 2.0 ** -24
+            assert bool(((w - o).abs() <= step).all()), "%dx%dx%d x%d: the walk and the one-tile kernels differ" % (M, N, K, batch)
+            assert float((w != o).float().mean()) < 1e-3
             res = got[1].float().cpu().numpy()
             for item in range(batch):
                 assert_fp16(res[item], 0.75 * whole_f64(a[item], ta, b[item], tb), what="%dx%dx%d item %d" % (M, N, K, item))
