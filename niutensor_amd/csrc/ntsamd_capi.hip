@@ -608,7 +608,10 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;
         const bool wide = ldc % 8 == 0 && s.N % 8 == 0 && aligned16(c) && strideC % 8 == 0 &&
                           (!grid || grid->strideC1 % 8 == 0);
-        if (wide && cus > 0 && tiles > cus)
+        /* from one tile per CU on: with CUs to spare the part is not held back by its power limit, and the older
+           kernels' longer lead of the loads counts for more than the energy this one saves (measured: 4096^3 112 ->
+           103 us, but 2048 x 4096 x 8192 on 128 CUs 147 -> 177 us with both operands k-contiguous) */
+        if (wide && cus > 0 && (tiles >= cus || tn.f16Persist.load(std::memory_order_relaxed) == 2))
             p.persistGrid = cus;
             /* four tile rows share a sweep over the tile columns: the 32 tiles an XCD works on at a time are 4 x 8,
                the same twelve operand panels as 8 x 4, and their stores spread over twice as many columns of c
