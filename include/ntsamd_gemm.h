@@ -15,7 +15,16 @@
  *   - data types use TENSOR_DATA_TYPE values: X_FLOAT = 2, X_FLOAT16 = 3
  *     (XDataType.h:33). Supported triples (a, b, c): (X_FLOAT, X_FLOAT, X_FLOAT),
  *     (X_FLOAT16, X_FLOAT16, X_FLOAT16) and (X_FLOAT16, X_FLOAT16, X_FLOAT);
- *     anything else fails with "Unsupported data type!" (XTensorBLAS.cu:101-103);
+ *     anything else fails with "Unsupported data type!" (XTensorBLAS.cu:101-103).
+ *     Beyond the reference: (X_FLOAT, X_FLOAT16, X_FLOAT16) and (X_FLOAT, X_FLOAT16,
+ *     X_FLOAT) give the result of ConvertDataType(a, X_FLOAT16) followed by the half
+ *     product, bit for bit, without the conversion pass or its temporary where the
+ *     product is short (the probabilities of the half attention,
+ *     source/sample/transformer/submodel/Attention.cpp:228-235): a is rounded to half,
+ *     to nearest even, where the kernel fetches it. Long products round a once, into
+ *     the stream's workspace, and run as all-half products (ntsamd_matrix_mul_static
+ *     and ntsamd_matrix_mul_batched_grid never do: they always round in the fetch).
+ *     Not offered by the pointer-list and column-sum entry points;
  *   - the result is c = alpha * op(a) * op(b) + beta * c. With beta == 0 the
  *     kernels never read c, so the caller does not have to zero it first (the
  *     reference calls SetZeroAll before every beta == 0 product,

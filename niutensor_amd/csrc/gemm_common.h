@@ -88,6 +88,7 @@ struct GemmParams {
     int f16PingPong;                       /* half, 256 x 256 tile: the two wave groups run one phase apart */
     int storeHint;                         /* != 0: the fast epilogues write c through (STORE_WRITE_THROUGH) */
     int persistGrid;                       /* half, 256 x 256 tile: > 0 = that many workgroups walk over all tiles */
+    int aF32;                              /* half product whose a is stored as float: rounded to half on its way to LDS */
 };
 
 /* The dispatcher hands consecutive workgroup ids to the 8 XCDs in turn, and

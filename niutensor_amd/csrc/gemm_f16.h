@@ -35,6 +35,7 @@
 #pragma once
 #include "gemm_common.h"
 #include "gemm_f32.h"   /* make_rsrc, IntC, NTSAMD_OOB_OFFSET */
+#include <type_traits>
 
 namespace ntsamd {
 
@@ -98,7 +99,11 @@ __device__ __forceinline__ float buffer_load_out<half_t>(__amdgpu_buffer_rsrc_t 
     return (float)__builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rsrc, byteOffset, 0, 0));
 }
 
-template <typename OutT, int BM, int BN, int BKT, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool VEC, typename PT>
+/* AT: the element type of a in memory. With float, a is rounded to half (to nearest even, as
+   _CudaConvertDataType does, core/getandset/ConvertDataType.cu:31-38) on its way from the registers into LDS: the
+   product of float probabilities with half values needs no converted copy of the probabilities
+   (source/sample/transformer/submodel/Attention.cpp:228-235). */
+template <typename OutT, int BM, int BN, int BKT, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool VEC, typename PT, typename AT = half_t>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_kernel(const GemmParams p, const PT tab)
 {
@@ -125,16 +130,18 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     __shared__ __attribute__((aligned(16))) half_t Bs[2][BSIZE];
 
     const TileCoord tc = tile_of_workgroup(p);
-    const half_t * __restrict__ A;
+    constexpr bool AF32 = std::is_same<AT, float>::value;
+    constexpr int ASZ = (int)sizeof(AT);
+    const AT * __restrict__ A;
     const half_t * __restrict__ B;
     OutT * __restrict__ C;
     if constexpr (sizeof(PT) > 1) {
-        A = static_cast<const half_t *>(tab.a[tc.batch]);
+        A = static_cast<const AT *>(tab.a[tc.batch]);
         B = static_cast<const half_t *>(tab.b[tc.batch]);
         C = static_cast<OutT *>(tab.c[tc.batch]);
     }
     else {
-        A = static_cast<const half_t *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
+        A = static_cast<const AT *>(p.a) + batch_offset(tc.batch, p.batchInner, p.strideA, p.strideA1);
         B = static_cast<const half_t *>(p.b) + batch_offset(tc.batch, p.batchInner, p.strideB, p.strideB1);
         C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
     }
@@ -160,7 +167,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             aMN[s] = row;
             aLds[s] = row * LDK + aK[s];
             int r = m0 + row < M - 1 ? row : M - 1 - m0;
-            aOff[s] = (r * p.lda + aK[s]) * 2;
+            aOff[s] = (r * p.lda + aK[s]) * ASZ;
         }
         else {
             aK[s] = g / (BM / 8);
@@ -168,7 +175,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             aLds[s] = aK[s] * LDA + aMN[s];
             /* columns past M are fetched from nowhere (zeros); a piece that straddles M runs on into the next
                row of k, into columns of the tile that are never stored */
-            aOff[s] = m0 + aMN[s] < M ? (aK[s] * p.lda + aMN[s]) * 2 : NTSAMD_OOB_OFFSET;
+            aOff[s] = m0 + aMN[s] < M ? (aK[s] * p.lda + aMN[s]) * ASZ : NTSAMD_OOB_OFFSET;
         }
     }
 #pragma unroll
@@ -190,20 +197,22 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         }
     }
 
-    const half_t * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
+    const AT * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
     const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const half_t * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
+    const AT * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
     const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
 
-    f16x8 ra[RING][NA], rb[RING][NB];
+    /* a float a waits in the ring as it came (two registers of four floats per piece) and is rounded when it moves on to LDS */
+    f16x8 ra[AF32 ? 1 : RING][AF32 ? 1 : NA], rb[RING][NB];
+    f32x4 raF[AF32 ? RING : 1][AF32 ? NA : 1][2];
 
     auto load_global = [&](auto RINGC, auto TAIL, int k0) {
         constexpr int rg = decltype(RINGC)::value;
         constexpr bool mayHangOver = decltype(TAIL)::value != 0;
         if constexpr (VEC) {
-            const half_t * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
+            const AT * ab = AKC ? aTile + k0 : aTile + (size_t)k0 * p.lda;
             const half_t * bb = BKC ? bTile + k0 : bTile + (size_t)k0 * p.ldb;
-            const long long aLeft = (long long)(aEnd - ab) * 2, bLeft = (long long)(bEnd - bb) * 2;
+            const long long aLeft = (long long)(aEnd - ab) * ASZ, bLeft = (long long)(bEnd - bb) * 2;
             const int aBytes = aLeft >> 31 ? 0x7fffffff : (int)aLeft, bBytes = bLeft >> 31 ? 0x7fffffff : (int)bLeft;
             __amdgpu_buffer_rsrc_t ar = make_rsrc(ab, aLeft);
             __amdgpu_buffer_rsrc_t br = make_rsrc(bb, bLeft);
@@ -220,16 +229,31 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 int off = aOff[s];
                 if (AKC && tail && k0 + aK[s] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                if constexpr (mayHangOver)
-                    ra[rg][s] = buffer_load_f16x8_any(ar, off, aBytes);
-                else
-                    ra[rg][s] = buffer_load_f16x8(ar, off);
-                if constexpr (mayHangOver && AKC)
-                    if (tail) {
+                if constexpr (AF32) {
+                    /* floats start on dwords, and a 16-byte buffer load is range-checked dword by dword: nothing
+                       hangs over the end of the buffer half-way */
+                    (void)aBytes;
+                    raF[rg][s][0] = buffer_load_f32x4(ar, off);
+                    raF[rg][s][1] = buffer_load_f32x4(ar, off == NTSAMD_OOB_OFFSET ? off : off + 16);
+                    if constexpr (mayHangOver && AKC)
+                        if (tail) {
 #pragma unroll
-                        for (int e = 1; e < 8; e++)
-                            ra[rg][s][e] = k0 + aK[s] + e < K ? ra[rg][s][e] : (half_t)0;
-                    }
+                            for (int e = 1; e < 8; e++)
+                                raF[rg][s][e / 4][e % 4] = k0 + aK[s] + e < K ? raF[rg][s][e / 4][e % 4] : 0.f;
+                        }
+                }
+                else {
+                    if constexpr (mayHangOver)
+                        ra[rg][s] = buffer_load_f16x8_any(ar, off, aBytes);
+                    else
+                        ra[rg][s] = buffer_load_f16x8(ar, off);
+                    if constexpr (mayHangOver && AKC)
+                        if (tail) {
+#pragma unroll
+                            for (int e = 1; e < 8; e++)
+                                ra[rg][s][e] = k0 + aK[s] + e < K ? ra[rg][s][e] : (half_t)0;
+                        }
+                }
             }
 #pragma unroll
             for (int s = 0; s < NB; s++) {
@@ -253,23 +277,32 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
 #pragma unroll
             for (int s = 0; s < NA; s++) {
                 f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+                f32x4 w[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
                 if (AKC) {
                     int r = m0 + aMN[s] < M - 1 ? m0 + aMN[s] : M - 1;
-                    const half_t * rp = A + (size_t)r * p.lda;
+                    const AT * rp = A + (size_t)r * p.lda;
 #pragma unroll
                     for (int e = 0; e < 8; e++)
-                        if (k0 + aK[s] + e < K)
-                            v[e] = rp[k0 + aK[s] + e];
+                        if (k0 + aK[s] + e < K) {
+                            if constexpr (AF32) w[e / 4][e % 4] = rp[k0 + aK[s] + e];
+                            else v[e] = rp[k0 + aK[s] + e];
+                        }
                 }
                 else if (k0 + aK[s] < K) {
-                    const half_t * rp = A + (size_t)(k0 + aK[s]) * p.lda;
+                    const AT * rp = A + (size_t)(k0 + aK[s]) * p.lda;
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
                         int c = m0 + aMN[s] + e < M - 1 ? m0 + aMN[s] + e : M - 1;
-                        v[e] = rp[c];
+                        if constexpr (AF32) w[e / 4][e % 4] = rp[c];
+                        else v[e] = rp[c];
                     }
                 }
-                ra[rg][s] = v;
+                if constexpr (AF32) {
+                    raF[rg][s][0] = w[0];
+                    raF[rg][s][1] = w[1];
+                }
+                else
+                    ra[rg][s] = v;
             }
 #pragma unroll
             for (int s = 0; s < NB; s++) {
@@ -298,8 +331,17 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     auto store_lds = [&](auto RINGC, int buf) {
         constexpr int rg = decltype(RINGC)::value;
 #pragma unroll
-        for (int s = 0; s < NA; s++)
-            *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = ra[rg][s];
+        for (int s = 0; s < NA; s++) {
+            if constexpr (AF32) {
+                f16x8 v;
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    v[e] = (half_t)raF[rg][s][e / 4][e % 4];          /* v_cvt_f16_f32: to nearest even */
+                *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = v;
+            }
+            else
+                *reinterpret_cast<f16x8 *>(&As[buf][aLds[s]]) = ra[rg][s];
+        }
 #pragma unroll
         for (int s = 0; s < NB; s++)
             *reinterpret_cast<f16x8 *>(&Bs[buf][bLds[s]]) = rb[rg][s];
@@ -523,7 +565,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     }
 }
 
-template <typename OutT, int CFG, bool AKC, bool BKC, bool VEC, typename PT>
+template <typename OutT, int CFG, bool AKC, bool BKC, bool VEC, typename PT, typename AT = half_t>
 static int launch_f16_one(const GemmParams & p0, const PT & tab, hipStream_t stream)
 {
     typedef TileShape<CFG> S;
@@ -532,7 +574,7 @@ static int launch_f16_one(const GemmParams & p0, const PT & tab, hipStream_t str
     p.tilesN = (p.N + S::BN - 1) / S::BN;
     p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
-    hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, S::MINW16, AKC, BKC, VEC, PT>),
+    hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, S::MINW16, AKC, BKC, VEC, PT, AT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();
 }

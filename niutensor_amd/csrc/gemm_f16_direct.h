@@ -820,6 +820,16 @@ static int launch_f16_direct(const GemmParams & p, hipStream_t stream)
     return launch_f16_direct_shape<OutT, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>(p, stream);
 }
 
+/* a in float, rounded to half on its way to LDS (no lists of matrices) */
+template <typename OutT, bool AKC, bool BKC, bool VEC>
+static int launch_f16_staged_a32(const GemmParams & p, int cfg, hipStream_t stream)
+{
+    NoPtrs none = {0};
+    if constexpr (VEC) if (cfg != CFG_64x64)
+        return launch_f16_one<OutT, CFG_128x128, AKC, BKC, VEC, NoPtrs, float>(p, none, stream);
+    return launch_f16_one<OutT, CFG_64x64, AKC, BKC, VEC, NoPtrs, float>(p, none, stream);
+}
+
 template <typename OutT, bool AKC, bool BKC, bool VEC>
 static int launch_f16_staged(const GemmParams & p, const PtrBatch * ptrs, int cfg, hipStream_t stream)
 {
@@ -841,6 +851,13 @@ template <bool AKC, bool BKC>
 static int launch_f16_trans(const GemmParams & p, const PtrBatch * ptrs, int vec, bool outF32, int cfg,
                             hipStream_t stream)
 {
+    if (p.aF32) {
+        if (vec == F16_STAGED)
+            return outF32 ? launch_f16_staged_a32<float, AKC, BKC, true>(p, cfg, stream)
+                          : launch_f16_staged_a32<half_t, AKC, BKC, true>(p, cfg, stream);
+        return outF32 ? launch_f16_staged_a32<float, AKC, BKC, false>(p, cfg, stream)
+                      : launch_f16_staged_a32<half_t, AKC, BKC, false>(p, cfg, stream);
+    }
     if (vec == F16_STAGED)
         return outF32 ? launch_f16_staged<float, AKC, BKC, true>(p, ptrs, cfg, stream)
                       : launch_f16_staged<half_t, AKC, BKC, true>(p, ptrs, cfg, stream);

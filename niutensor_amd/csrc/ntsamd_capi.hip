@@ -128,7 +128,11 @@ int check_shape(int transposedA, int transposedB, int na, int ma, int nb, int mb
     return NTSAMD_OK;
 }
 
-enum Kind { KIND_F32, KIND_F16, KIND_F16_F32OUT };
+/* KIND_A32_*: a half product whose a is stored as float and rounded to half on its way into the kernel's LDS */
+enum Kind { KIND_F32, KIND_F16, KIND_F16_F32OUT, KIND_A32_F16, KIND_A32_F16_F32OUT };
+inline bool kind_a32(Kind k) { return k == KIND_A32_F16 || k == KIND_A32_F16_F32OUT; }
+inline bool kind_out_f32(Kind k) { return k == KIND_F16_F32OUT || k == KIND_A32_F16_F32OUT; }
+inline bool kind_c_half(Kind k) { return k == KIND_F16 || k == KIND_A32_F16; }
 
 int check_types(int ta, int tb, int tc, Kind & kind)
 {
@@ -138,6 +142,10 @@ int check_types(int ta, int tb, int tc, Kind & kind)
         kind = KIND_F16;
     else if (ta == NTSAMD_X_FLOAT16 && tb == NTSAMD_X_FLOAT16 && tc == NTSAMD_X_FLOAT)
         kind = KIND_F16_F32OUT;
+    else if (ta == NTSAMD_X_FLOAT && tb == NTSAMD_X_FLOAT16 && tc == NTSAMD_X_FLOAT16)
+        kind = KIND_A32_F16;
+    else if (ta == NTSAMD_X_FLOAT && tb == NTSAMD_X_FLOAT16 && tc == NTSAMD_X_FLOAT)
+        kind = KIND_A32_F16_F32OUT;
     else
         return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
     return NTSAMD_OK;
@@ -241,9 +249,11 @@ struct Plan {
      NTSAMD_F16_PINGPONG=0       half, 256 x 256 tile: the main loop in which both waves of a SIMD meet one barrier
      NTSAMD_F16_PERSIST=0        half, 256 x 256 tile: one workgroup per tile, never one per CU that walks over tiles
      NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment
-     NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset) */
+     NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset)
+     NTSAMD_A32_CONVERT=0|1      float a with half b: never / whenever it fits the workspace, round a to half in a pass
+                                 of its own before the product */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -258,6 +268,7 @@ const Knob g_knobs[] = {
     {"NTSAMD_F32_R16", &Tuning::f32R16},     {"NTSAMD_F32_SPLIT_ATOMIC", &Tuning::f32SplitAtomic},
     {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
     {"NTSAMD_STORE_HINT", &Tuning::storeHint}, {"NTSAMD_GROUP_M", &Tuning::groupM},
+    {"NTSAMD_A32_CONVERT", &Tuning::a32Convert},
 };
 
 const Tuning & tuning()
@@ -485,6 +496,31 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                     s.M, s.N, count);
 
     const Tuning & tn = tuning();
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    WorkHold work;
+    bool aInWork = false;
+    if (kind_a32(kind) && !noAlloc && !ptrs && !grid && tn.a32Convert.load(std::memory_order_relaxed) != 0) {
+        /* A float a is rounded to half on its way into LDS, through registers: that fetch is about half as fast again
+           as the one that moves halves straight to LDS. A long product is better served by rounding a once, into
+           the stream's workspace, and running the all-half product on that copy (same rounding, same bits): when
+           the time the slower fetch would add exceeds one more launch and one pass over a. */
+        const int rowsA = s.aKContig ? s.M : s.K, colsA = s.aKContig ? s.K : s.M;
+        const long long span = (long long)(count - 1) * strideA + (long long)(rowsA - 1) * lda + colsA;
+        const double slower = 0.5 * 2.0 * s.M * s.N * s.K * count / 7.0e14;
+        const double pass = 2.5e-6 + (double)span * 6.0 / 5.0e12;
+        const bool forced = tn.a32Convert.load(std::memory_order_relaxed) > 0;
+        if (strideA >= 0 && span > 0 && (size_t)span * 2 <= SPLIT_WORK_BYTES && (forced || slower > pass)) {
+            work.take_stream(devID, hs);
+            if (work.mem != NULL) {
+                const int rc = launch_convert(0, a, work.mem, span, hs);
+                if (rc != 0)
+                    return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+                a = work.mem;
+                kind = kind == KIND_A32_F16 ? KIND_F16 : KIND_F16_F32OUT;
+                aInWork = true;
+            }
+        }
+    }
     GemmParams p;
     memset(&p, 0, sizeof(p));
     p.a = a;
@@ -508,11 +544,12 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     p.batch = count;
     p.groupM = tn.groupM.load(std::memory_order_relaxed) > 0 ? tn.groupM.load(std::memory_order_relaxed) : 8;     /* the half walk over tiles takes 4 (see where it is chosen) */
     p.act = act;
+    p.aF32 = kind_a32(kind) ? 1 : 0;
     p.wideRowsOnly = tn.f32R16.load(std::memory_order_relaxed) == 0;
     p.f16PingPong = tn.f16PingPong.load(std::memory_order_relaxed) != 0;
     {
         /* results whose rows are whole 128-byte lines are written through (see STORE_WRITE_THROUGH) */
-        const long long unit = kind == KIND_F16 ? 2 : 4;
+        const long long unit = kind_c_half(kind) ? 2 : 4;
         const bool lines = (reinterpret_cast<uintptr_t>(c) & 127u) == 0 && !ptrs && (ldc * unit) % 128 == 0 &&
                            (strideC * unit) % 128 == 0 && (!grid || (grid->strideC1 * unit) % 128 == 0);
         const int knob = tn.storeHint.load(std::memory_order_relaxed);
@@ -536,7 +573,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
     int fetch16 = F16_SCALAR;
     if (kind != KIND_F32) {
-        const bool direct = vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
+        const bool direct = !kind_a32(kind) && vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
                             aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
                             (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
         fetch16 = direct ? F16_DIRECT : (vec ? F16_STAGED : F16_SCALAR);
@@ -545,7 +582,6 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             fetch16 = knob;
         vec = fetch16 == F16_DIRECT;                               /* what the column-sum by-product needs */
     }
-    hipStream_t hs = static_cast<hipStream_t>(stream);
     const bool half = kind != KIND_F32;
     /* Cutting k into pieces pays when the result has few tiles and k is long (weight gradients, the few rows of a
        decoding step). The pieces of a product on the 16-byte path meet in a workspace and leave the ordinary way
@@ -554,7 +590,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
        its beta first): only if the knob asks for it, or when there is no workspace to be had. */
     const bool atomicAble = !half && vec && !ptrs && act == ACT_NONE && dense;
     const bool atomicAsked = atomicAble && !noAlloc && tn.f32SplitAtomic.load(std::memory_order_relaxed) > 0;
-    const bool maySplit = atomicAsked || ((half ? fetch16 == F16_DIRECT : vec) && !ptrs);
+    /* (the half copy of a float a has the workspace to itself) */
+    const bool maySplit = !aInWork && (atomicAsked || ((half ? fetch16 == F16_DIRECT : vec) && !ptrs));
     const size_t workBytes = atomicAsked ? 0 : (noAlloc ? STATIC_SCRATCH_BYTES : SPLIT_WORK_BYTES);
     /* pieces that meet in a workspace gather no column sums: cutting costs a pass of its own over b then (a
        launch, b read once more) */
@@ -579,7 +616,6 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                         (long long)STATIC_SCRATCH_BYTES);
     }
     Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, workBytes, cutExtra, fast32, forcedSplits);
-    WorkHold work;
     bool viaWork = false;
     if (plan.splits > 1 && !atomicAsked) {
         if (noAlloc) {
@@ -662,7 +698,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             rc = s.bKContig ? launch_f32_tt(p, ptrs, vec, cfg, hs) : launch_f32_tn(p, ptrs, vec, cfg, hs);
     }
     else {
-        bool outF32 = kind == KIND_F16_F32OUT;
+        bool outF32 = kind_out_f32(kind);
         if (s.aKContig)
             rc = s.bKContig ? launch_f16_nt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_nn(p, ptrs, fetch16, outF32, cfg, hs);
         else
@@ -846,7 +882,7 @@ int ntsamd_matrix_mul_colsum(int devID, void * stream,
         st = check_shape(transposedA, transposedB, na, ma, nb, mb, nc, mc, s);
     if (st != NTSAMD_OK)
         return st;
-    if (kind == KIND_F16_F32OUT)
+    if (kind == KIND_F16_F32OUT || kind_a32(kind))
         return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");   /* the sums have the type of b and of c */
     if (s.N == 0)
         return NTSAMD_OK;
@@ -1189,6 +1225,8 @@ int ntsamd_matrix_mul_batched(int devID, void * stream,
         return fail(NTSAMD_ERR_ARGUMENT, "negative batch count");
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
+    if (kind_a32(kind))
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");   /* lists of matrices: one type for a and b */
     if (!a || !b || !c)
         return fail(NTSAMD_ERR_ARGUMENT, "Empty input lists!");
     for (int i = 0; i < count; i++)

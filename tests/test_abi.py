@@ -69,7 +69,7 @@ def call_mm(L, ta=nt.X_NOTRANS, tb=nt.X_NOTRANS, types=(2, 2, 2), dims=(2, 3, 3,
 def test_argument_errors_need_no_device():
     L = nt.load()
     # unsupported data types: X_INT, X_DOUBLE, mixed
-    for types in ((0, 0, 0), (4, 4, 4), (2, 3, 2), (2, 2, 3)):
+    for types in ((0, 0, 0), (4, 4, 4), (3, 2, 2), (3, 2, 3), (2, 2, 3)):
         assert call_mm(L, types=types) == 2
         assert L.ntsamd_last_error().decode() == "Unsupported data type!"
     # transpose flags are the enum values 0 / 1, nothing else
@@ -181,7 +181,7 @@ def test_grid_batch_argument_errors_need_no_device():
     assert call(counts=(1 << 16, 1 << 16)) == 1 and "too many" in L.ntsamd_last_error().decode()
     assert call(counts=(0, 2)) == 0                                       # nothing to do
     assert call(a=None) == 1
-    assert call(types=(2, 3, 2)) == 2                                     # float times half
+    assert call(types=(3, 2, 2)) == 2                                     # half times float
     # results: two items in the same place; heads side by side but rows too short for both; heads side by
     # side with the next batch item starting inside the last row
     assert call(sc=(0, 128)) == 1 and "overlap" in L.ntsamd_last_error().decode()

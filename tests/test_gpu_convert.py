@@ -114,3 +114,110 @@ def test_equal_types_do_nothing_and_bad_pairs_are_refused(gpu):
     assert L.ntsamd_convert_data_type(0, None, a.data_ptr(), 2, b.data_ptr(), 3, -1) == 1
     assert L.ntsamd_convert_data_type(0, None, None, 2, b.data_ptr(), 3, 4) == 1
     assert L.ntsamd_convert_data_type(0, None, a.data_ptr(), 2, b.data_ptr(), 3, 0) == 0
+
+
+@pytest.mark.parametrize("ta", (nt.X_NOTRANS, nt.X_TRANS))
+@pytest.mark.parametrize("tb", (nt.X_NOTRANS, nt.X_TRANS))
+def test_float_a_is_rounded_to_half_inside_the_product(gpu, oracle, ta, tb):
+    """A half product whose a is stored as float (the probabilities after the softmax,
+    source/sample/transformer/submodel/Attention.cpp:228-235: ConvertDataType, then BMMul with the half values):
+    the result is that of oracle_convert_data_type followed by the half product, and the same bits as the
+    library's own conversion pass followed by its product on the same kernel."""
+    torch = torch_()
+    from tolerance import assert_fp16
+    for i, (M, N, K) in enumerate(((128, 64, 128), (100, 72, 50), (257, 129, 333), (40, 30011, 96))):
+        sa = (K, M) if ta == nt.X_TRANS else (M, K)
+        sb = (N, K) if tb == nt.X_TRANS else (K, N)
+        a = ((oracle.uniform(sa, 8100 + i) + 0.5) / 3.0).astype(np.float32)       # values that do not fit a half exactly
+        b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(sb, 8200 + i, 0, 0.5)))
+        a_half = oracle.from_f16_bits(oracle.convert(a, X_FLOAT16))    # what the reference multiplies
+        ga, gb = to_dev(a, gpu), to_dev(b, gpu).half()
+        for out_float in (False, True):
+            ref = oracle.matmul2d(a_half, ta, b, tb, None, 0.5, 0.0)
+            c = torch.full((M, N), float("nan"), device=gpu, dtype=torch.float32 if out_float else torch.float16)
+            nt.matrix_mul(ga, ta, gb, tb, c, 0.5, 0.0)
+            assert_fp16(c.float().cpu().numpy(), ref, what="%dx%dx%d float a, %s result" % (M, N, K, "float" if out_float else "half"))
+            # the library's two steps: a conversion pass, then the product through the same register-staged kernel
+            nt.tuning_set("NTSAMD_F16_FETCH", 2)
+            try:
+                ah = torch.empty(sa, device=gpu, dtype=torch.float16)
+                nt.convert_data_type(ga, ah)
+                c2 = torch.full_like(c, float("nan"))
+                nt.matrix_mul(ah, ta, gb, tb, c2, 0.5, 0.0)
+            finally:
+                nt.tuning_set("NTSAMD_F16_FETCH", None)
+            assert torch.equal(c, c2), "%dx%dx%d: fused rounding and conversion pass differ" % (M, N, K)
+
+
+def test_float_probabilities_times_half_values_in_batches(gpu, oracle):
+    """The attention context of the half training path: probabilities (float, after softmax and dropout) times the
+    heads' values (half), as a strided batch; and the same on merged tensors through the grid entry point."""
+    torch = torch_()
+    from tolerance import assert_fp16
+    batch, lq, lk, dh = 6, 40, 50, 64
+    p = np.abs(oracle.normal((batch, lq, lk), 8300, 0, 1.0)).astype(np.float32)
+    p /= p.sum(axis=-1, keepdims=True)
+    v = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch, lk, dh), 8301, 0, 0.5)))
+    p_half = oracle.from_f16_bits(oracle.convert(p, X_FLOAT16))
+    ref = oracle.matmul_batched(p_half, nt.X_NOTRANS, v, nt.X_NOTRANS, None, 1.0)
+    gp, gv = to_dev(p, gpu), to_dev(v, gpu).half()
+    c = torch.full((batch, lq, dh), float("nan"), device=gpu, dtype=torch.float16)
+    nt.matrix_mul_batched_strided(gp, nt.X_NOTRANS, gv, nt.X_NOTRANS, c, batch, lq * lk, lk * dh, lq * dh, lq, lk, lk, dh, lq, dh, 1.0, 0.0)
+    assert_fp16(c.float().cpu().numpy(), ref, what="float probabilities x half values, strided batch")
+
+
+def test_long_products_round_a_in_a_pass_of_their_own_with_the_same_bits(gpu, oracle):
+    """Where the library rounds a float a in a pass of its own before a long product (into its workspace), the
+    result is the one its conversion entry point followed by the all-half product gives, bit for bit; forced on
+    small shapes and on a batch whose matrices stand apart, and left to the library's own choice at
+    2048 x 2048 x 1024."""
+    torch = torch_()
+    from tolerance import assert_fp16
+    T, NT = nt.X_TRANS, nt.X_NOTRANS
+    for i, (M, N, K, ta, forced) in enumerate(((128, 64, 128, NT, 1), (100, 72, 56, T, 1), (257, 136, 328, NT, 1),
+                                               (2048, 2048, 1024, NT, None), (2048, 2048, 1024, T, None))):
+        sa = (K, M) if ta == T else (M, K)
+        a = ((oracle.uniform(sa, 8400 + i) + 0.5) / 3.0).astype(np.float32)
+        b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((K, N), 8500 + i, 0, 0.5)))
+        ga, gb = to_dev(a, gpu), to_dev(b, gpu).half()
+        ah = torch.empty(sa, device=gpu, dtype=torch.float16)
+        nt.convert_data_type(ga, ah)
+        for out_float in (False, True):
+            c = torch.full((M, N), float("nan"), device=gpu, dtype=torch.float32 if out_float else torch.float16)
+            c2 = torch.full_like(c, float("nan"))
+            nt.tuning_set("NTSAMD_A32_CONVERT", forced)
+            try:
+                nt.matrix_mul(ga, ta, gb, NT, c, 0.5, 0.0)
+            finally:
+                nt.tuning_set("NTSAMD_A32_CONVERT", None)
+            nt.matrix_mul(ah, ta, gb, NT, c2, 0.5, 0.0)
+            assert torch.equal(c, c2), "%dx%dx%d: a rounded before the product differs from convert + product" % (M, N, K)
+            if M <= 300:
+                a_half = oracle.from_f16_bits(oracle.convert(a, X_FLOAT16))
+                assert_fp16(c.float().cpu().numpy(), oracle.matmul2d(a_half, ta, b, NT, None, 0.5, 0.0),
+                            what="%dx%dx%d float a rounded first" % (M, N, K))
+    # a strided batch whose probabilities stand 24 floats apart: the pass covers the gaps too, the product skips them
+    batch, lq, lk, dh, gap = 5, 40, 48, 64, 24
+    p = np.abs(oracle.normal((batch, lq * lk + gap), 8600, 0, 1.0)).astype(np.float32)
+    v = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch, lk, dh), 8601, 0, 0.5)))
+    p_half = oracle.from_f16_bits(oracle.convert(np.ascontiguousarray(p[:, :lq * lk]).reshape(batch, lq, lk), X_FLOAT16))
+    ref = oracle.matmul_batched(p_half, NT, v, NT, None, 1.0)
+    gp, gv = to_dev(p, gpu), to_dev(v, gpu).half()
+    c = torch.full((batch, lq, dh), float("nan"), device=gpu, dtype=torch.float16)
+    nt.tuning_set("NTSAMD_A32_CONVERT", 1)
+    try:
+        nt.matrix_mul_batched_strided(gp, NT, gv, NT, c, batch, lq * lk + gap, lk * dh, lq * dh, lq, lk, lk, dh, lq, dh, 1.0, 0.0)
+    finally:
+        nt.tuning_set("NTSAMD_A32_CONVERT", None)
+    assert_fp16(c.float().cpu().numpy(), ref, what="float probabilities rounded first, strided batch with gaps")
+
+
+def test_mixed_types_that_are_not_offered_are_refused(gpu):
+    torch = torch_()
+    a = torch.zeros((8, 8), device=gpu, dtype=torch.float16)
+    b = torch.zeros((8, 8), device=gpu, dtype=torch.float32)
+    c = torch.zeros((8, 8), device=gpu, dtype=torch.float16)
+    with pytest.raises(nt.NtsAmdError):
+        nt.matrix_mul(a, nt.X_NOTRANS, b, nt.X_NOTRANS, c)          # half a, float b
+    with pytest.raises(nt.NtsAmdError):
+        nt.matrix_mul(b, nt.X_NOTRANS, b, nt.X_NOTRANS, c)          # float operands, half result
