@@ -507,6 +507,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="configuration 1-14 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", action="store_true",
+                    help="time --config alone, without the other baseline configurations beside it (for a profiler: their "
+                         "kernels share names with those of configurations 6, 7, 12 and 14)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (scale for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -544,11 +547,12 @@ def main():
     lines[args.config] = head
     # the other configurations of the baseline, each settled and timed like the headline (at least 50 steps, so that
     # a short headline run still gives them a steady reading; a tenth for the 1 ms product), CPU leg on a 3 s sample
-    for idx in BASELINE_CONFIGS:
+    for idx in BASELINE_CONFIGS if not args.only else ():
         if idx not in lines:
             steps = max(50, args.steps) if idx != 5 else max(20, args.steps // 10)
             lines[idx] = bench_one(idx, steps, args.warmup, dev, oracle, with_cpu, cpu_budget_s=3.0)
-    head["configs"] = [brief(lines[idx]) for idx in BASELINE_CONFIGS]
+    if not args.only:
+        head["configs"] = [brief(lines[idx]) for idx in BASELINE_CONFIGS]
     print(json.dumps(head), flush=True)
 
 
