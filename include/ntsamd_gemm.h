@@ -20,7 +20,7 @@
  *     X_FLOAT) give the result of ConvertDataType(a, X_FLOAT16) followed by the half
  *     product, bit for bit, without the conversion pass or its temporary where the
  *     product is short (the probabilities of the half attention,
- *     source/sample/transformer/submodel/Attention.cpp:228-235): a is rounded to half,
+ *     source/sample/transformer/submodel/Attention.cpp:231-237): a is rounded to half,
  *     to nearest even, where the kernel fetches it. Long products round a once, into
  *     the stream's workspace, and run as all-half products (ntsamd_matrix_mul_static
  *     and ntsamd_matrix_mul_batched_grid never do: they always round in the fetch).

@@ -102,7 +102,7 @@ __device__ __forceinline__ float buffer_load_out<half_t>(__amdgpu_buffer_rsrc_t 
 /* AT: the element type of a in memory. With float, a is rounded to half (to nearest even, as
    _CudaConvertDataType does, core/getandset/ConvertDataType.cu:31-38) on its way from the registers into LDS: the
    product of float probabilities with half values needs no converted copy of the probabilities
-   (source/sample/transformer/submodel/Attention.cpp:228-235). */
+   (source/sample/transformer/submodel/Attention.cpp:231-237). */
 template <typename OutT, int BM, int BN, int BKT, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool VEC, typename PT, typename AT = half_t>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_kernel(const GemmParams p, const PT tab)

@@ -120,7 +120,7 @@ def test_equal_types_do_nothing_and_bad_pairs_are_refused(gpu):
 @pytest.mark.parametrize("tb", (nt.X_NOTRANS, nt.X_TRANS))
 def test_float_a_is_rounded_to_half_inside_the_product(gpu, oracle, ta, tb):
     """A half product whose a is stored as float (the probabilities after the softmax,
-    source/sample/transformer/submodel/Attention.cpp:228-235: ConvertDataType, then BMMul with the half values):
+    source/sample/transformer/submodel/Attention.cpp:231-237: ConvertDataType, then BMMul with the half values):
     the result is that of oracle_convert_data_type followed by the half product, and the same bits as the
     library's own conversion pass followed by its product on the same kernel."""
     torch = torch_()
