@@ -397,6 +397,46 @@ def graph_replayed(wl, dev, ev, steps_in_graph=50, replays=20):
     return ev.time(g.replay, stream, replays) / steps_in_graph
 
 
+def k_scan(dev, ev):
+    """Where the time of configuration 3's first product goes: the same 256 x (128 x 128) results with k from 8 to 512,
+    a launch that does next to nothing, and a plain copy of the bytes the k = 64 product moves; each replayed from a
+    HIP graph (microseconds per launch). The intercept of the scan is what a launch of this grid costs before its
+    first MFMA and after its last; the slope is the matrix pipe."""
+    import torch
+    import niutensor_amd as nt
+    T, NT = nt.X_TRANS, nt.X_NOTRANS
+
+    class One:
+        launches = 1
+
+    def replayed(fn):
+        w = One()
+        w.run = fn
+        return round(min(graph_replayed(w, dev, ev) for _ in range(3)) * 1e6, 2)
+
+    out = {"scan": "256 x (128 x k) . (128 x k)^T, float, replayed from a HIP graph, us per launch", "k": {}}
+    for k in (8, 32, 64, 96, 128, 192, 256, 512):
+        q = torch.randn(256, 128, k, device=dev)
+        kk = torch.randn(256, 128, k, device=dev)
+        s = torch.empty(256, 128, 128, device=dev)
+        out["k"][str(k)] = replayed(lambda: nt.matrix_mul_batched_strided(q, NT, kk, T, s, 256, 128 * k, 128 * k, 16384,
+                                                                         128, k, 128, k, 128, 128, 0.125, 0.0))
+    a = torch.zeros(64, device=dev)
+    b = torch.zeros(64, device=dev, dtype=torch.float16)
+    out["launch_of_one_workgroup_us"] = replayed(lambda: nt.convert_data_type(a, b))
+    x = torch.empty(4 * 1024 * 1024, device=dev)
+    y = torch.empty_like(x)
+    out["copy_16MiB_read_16MiB_written_us"] = replayed(lambda: y.copy_(x))
+    ks = [64, 96, 128, 192, 256, 512]
+    ts = [out["k"][str(k)] for k in ks]
+    n = len(ks)
+    mk, mt = sum(ks) / n, sum(ts) / n
+    slope = sum((k - mk) * (t - mt) for k, t in zip(ks, ts)) / sum((k - mk) ** 2 for k in ks)
+    out["fit_k64_to_512"] = {"us_per_k": round(slope, 4), "intercept_us": round(mt - slope * mk, 2),
+                             "matrix_pipe_alone_us_per_k": round(2.0 * 256 * 128 * 128 / (PEAK_TFLOPS["f32"] * 1e12) * 1e6, 4)}
+    return out
+
+
 def settle(wl, ev, stream):
     """Runs the workload until SETTLE_S seconds of GPU time have passed; returns the launches it took."""
     done, spent = 0, 0.0
@@ -510,6 +550,8 @@ def main():
     ap.add_argument("--only", action="store_true",
                     help="time --config alone, without the other baseline configurations beside it (for a profiler: their "
                          "kernels share names with those of configurations 6, 7, 12 and 14)")
+    ap.add_argument("--k-scan", action="store_true",
+                    help="run only the scan over k of configuration 3's first product (what a launch costs beside its MFMAs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (scale for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -532,6 +574,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "copies": args.steps}))
+        return
+    if args.k_scan:
+        print(json.dumps(k_scan(dev, HipEvents())))
         return
     oracle = Oracle()
     with_cpu = not args.no_cpu
