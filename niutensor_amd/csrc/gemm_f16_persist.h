@@ -60,8 +60,10 @@ gemm_f16_persistent_kernel(const GemmParams p)
     constexpr int WM = 128, WN = 64, TI = WM / 16, TJ = WN / 16;      /* 16 x 16 blocks of v_mfma_f32_16x16x32_f16: a slab is ONE k step */
     /* LDS, one region per operand, four slabs each.
        k-contiguous: two pair slots of 32 KB; a chunk of 1 KB holds 8 rows x [slab parity][64 bytes], the four 16-byte
-           columns of a row's 64 bytes permuted by (row >> 2) & 3 (sixteen consecutive rows reading one logical
-           column hit sixteen different 16-byte bank groups: rows r, r+4, r+8, r+12 share 64 bytes of a 256-byte line).
+           columns of a row's 64 bytes permuted by (row >> 1) & 3. A fragment read has lane l at row l % 16, column
+           l / 16; measured with SQ_LDS_BANK_CONFLICT on that address pattern: none with this permutation, one
+           conflict cycle per cycle with (row >> 2) & 3 (the permutation that is free of conflicts where lane l reads
+           row l % 32, column l / 32, as the 32 x 32 x 16 fragments of the other half kernels do).
        mn-contiguous: four stages of 16 chunks (k rows c and c+16, 512 bytes each), chunks 1088 bytes apart and
            chunks 8-15 another 32 bytes on: a transposing read of lanes 0-31 takes 32 bytes from each of k rows s and
            8 + s (s = 0..3), i.e. from chunks s and 8 + s, which then lie 64 s and 64 s + 32 bytes into a 256-byte
@@ -139,7 +141,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
             const int ch = wave * NQA + q;
             if (AKC) {
                 const int row = ch * 8 + ((lane >> 2) & 7);
-                const int col = (lane & 3) ^ ((row >> 2) & 3);
+                const int col = (lane & 3) ^ ((row >> 1) & 3);
                 aKc[q] = (lane >> 5) * 32 + col * 8;
                 const int r = m0 + row < M - 1 ? row : M - 1 - m0;
                 aOff[q] = (r * p.lda + aKc[q]) * 2;
@@ -157,7 +159,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
             const int ch = wave * NQB + q;
             if (BKC) {
                 const int row = ch * 8 + ((lane >> 2) & 7);
-                const int col = (lane & 3) ^ ((row >> 2) & 3);
+                const int col = (lane & 3) ^ ((row >> 1) & 3);
                 bKc[q] = (lane >> 5) * 32 + col * 8;
                 const int r = n0 + row < N - 1 ? row : N - 1 - n0;
                 bOff[q] = (r * p.ldb + bKc[q]) * 2;
@@ -239,14 +241,14 @@ gemm_f16_persistent_kernel(const GemmParams p)
        b fragment is the FIRST operand here, so that result register r of lane l is row l % 16 of the block of c (the
        a fragment's index) and column 4 (l / 16) + r (the b fragment's index): a lane holds four consecutive columns
        of one row, 8 bytes of c.
-       k-contiguous: row + 16-byte column of a pair chunk, the column permuted by (row >> 2) & 3.
+       k-contiguous: row + 16-byte column of a pair chunk, the column permuted by (row >> 1) & 3.
        mn-contiguous: two transposing reads, each of which hands a lane four consecutive k (k rows 8 g + 4 h + s,
        s = 0..3, pointed at by address lanes 4 s + q with their four columns 4 q .. 4 q + 3). */
     const int rho = lane & 15, g4 = lane >> 4;
     int aFrag = 0, bFrag = 0, aTr[2] = {0, 0}, bTr[2] = {0, 0};
     {
         const int ra = wm0 + rho, rb = wn0 + rho;
-        const int sw = (rho >> 2) & 3;
+        const int sw = (rho >> 1) & 3;
         aFrag = (ra >> 3) * 1024 + (ra & 7) * 64 + ((g4 ^ sw) * 16);
         bFrag = A_REGION + (rb >> 3) * 1024 + (rb & 7) * 64 + ((g4 ^ sw) * 16);
         const int s4 = rho >> 2, q4 = rho & 3;
