@@ -52,7 +52,7 @@
 
 namespace ntsamd {
 
-template <bool AKC, bool BKC>
+template <bool AKC, bool BKC, bool HASB>
 __global__ void __launch_bounds__(512, 1)
 gemm_f16_persistent_kernel(const GemmParams p)
 {
@@ -80,9 +80,14 @@ gemm_f16_persistent_kernel(const GemmParams p)
        that write 8 bytes each, 16 rows x 2 pieces, then cover all 64 banks) */
     constexpr int EPI_PITCH = WN * 2 + 16, EPI_WAVE = 16 * EPI_PITCH;
     constexpr int NST = TI * 2;                     /* store instructions per wave and tile: 8 rows of 128 bytes each */
+    /* HASB: a bias by column, of c's type. The 16 values that a lane's columns take (four 8-byte loads) are requested
+       after the previous tile's stores and before slabs 2 and 3, so the waits of the first two slabs count them with
+       the stores; the first tile's are requested before anything else. */
+    constexpr int NB = HASB ? TJ : 0;
+    constexpr int NSB = NST + NB;                   /* what lies between a later tile's slabs 0-1 and 2-3 */
     static_assert(8 * EPI_WAVE <= A_REGION - A_HALF && 8 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
     static_assert(A_REGION + B_REGION <= 160 * 1024, "the stages must fit LDS");
-    static_assert(MM + NST + KK + 2 * MM < 64, "the wait counter has six bits");
+    static_assert(MM + NSB + KK + 2 * MM < 64, "the wait counter has six bits");
 
     __shared__ __attribute__((aligned(1024))) char lds[A_REGION + B_REGION];
 
@@ -103,6 +108,20 @@ gemm_f16_persistent_kernel(const GemmParams p)
     const bool follower = wave >= NW / 2;
     const int nk = (K + BKT - 1) / BKT;                        /* the launcher guarantees nk >= 8 */
     const int total = p.tilesM * p.tilesN * p.batch;
+    f16x4 bv[HASB ? TJ : 1];
+    /* the bias of the tile whose columns begin at bn0: columns 16 j + 4 (lane / 16) .. + 3 of the wave's 64, what
+       result registers 0-3 of block column j hold; past N the buffer ends and the loads bring zeros */
+    auto load_bias = [&](int bn0) {
+        if constexpr (HASB) {
+            const __amdgpu_buffer_rsrc_t br = make_rsrc(const_cast<half_t *>(static_cast<const half_t *>(p.bias)), (long long)N * 2);
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(br, (bn0 + wn0 + 16 * j + 4 * (lane >> 4)) * 2, 0, 0);
+                bv[j] = __builtin_bit_cast(f16x4, v);
+            }
+        }
+    };
 
     /* ---- the tile whose operands are being fetched ---------------------------------- */
     /* Where a tile lies is scalar arithmetic with divisions in it (a microsecond of it, measured, when it sat
@@ -299,9 +318,9 @@ gemm_f16_persistent_kernel(const GemmParams p)
         else if (n == 2 * MM) wait_vmcnt<2 * MM>();
         else if (n == KK + MM) wait_vmcnt<KK + MM>();
         else if (n == KK + 2 * MM) wait_vmcnt<KK + 2 * MM>();
-        else if (n == NST + KK + 2 * MM) wait_vmcnt<NST + KK + 2 * MM>();
+        else if (n == NSB + KK + 2 * MM) wait_vmcnt<NSB + KK + 2 * MM>();
         else if (n == MM + KK + 2 * MM) wait_vmcnt<MM + KK + 2 * MM>();
-        else if (n == MM + NST + KK + 2 * MM) wait_vmcnt<MM + NST + KK + 2 * MM>();
+        else if (n == MM + NSB + KK + 2 * MM) wait_vmcnt<MM + NSB + KK + 2 * MM>();
         else wait_vmcnt<0>();
     };
 
@@ -388,7 +407,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
         /* slab 0 requests nothing (slabs 2 and 3 are in flight) and counts the previous tile's stores */
         read_frags(0);
         if (extra)
-            wait_vmcnt<NST + KK + 2 * MM>();
+            wait_vmcnt<NSB + KK + 2 * MM>();
         else
             wait_vmcnt<KK + 2 * MM>();
         compute(0);
@@ -433,8 +452,12 @@ gemm_f16_persistent_kernel(const GemmParams p)
             for (int j = 0; j < TJ; j++) {
                 f16x4 v;
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    v[e] = (half_t)activate(alpha * acc[i][j][e], act);
+                for (int e = 0; e < 4; e++) {
+                    if constexpr (HASB)
+                        v[e] = (half_t)activate(alpha * acc[i][j][e] + (float)bv[j][e], act);
+                    else
+                        v[e] = (half_t)activate(alpha * acc[i][j][e], act);
+                }
                 *reinterpret_cast<f16x4 *>(wr + j * 32) = v;
             }
         };
@@ -479,6 +502,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
         return;
     NTSAMD_STAMP(0);
     adopt(locate(id));
+    load_bias(n0);
     issue_two(0);
     issue_two(2);
     int extra = 0;
@@ -491,6 +515,13 @@ gemm_f16_persistent_kernel(const GemmParams p)
         /* every wave has passed the last barrier of the main loop: nobody reads the stages any more */
         const int em0 = m0, en0 = n0;
         half_t * eC = C;
+        if constexpr (HASB) {
+            /* the bias is used from here on: whatever wait the compiler puts before its first use lands here, where
+               nothing is in flight, and not behind the next tile's first slabs */
+#pragma unroll
+            for (int j = 0; j < TJ; j++)
+                asm volatile("" : "+v"(bv[j]));
+        }
         if (more) {
             adopt(next);
             issue_two(0);
@@ -502,12 +533,13 @@ gemm_f16_persistent_kernel(const GemmParams p)
         NTSAMD_STAMP(more ? 6 : 12);
         if (!more)
             break;
+        load_bias(n0);
         /* where slabs 2 and 3 go is free once every wave has read its staged rows back */
         wait_lgkmcnt0();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         issue_two(2);
-        extra = NST;
+        extra = NSB;
     }
 #ifdef NTSAMD_PROBE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -529,7 +561,15 @@ static int launch_f16_persistent(const GemmParams & p0, hipStream_t stream)
     p.splits = 1;
     const long long total = (long long)p.tilesM * p.tilesN * p.batch;
     const unsigned groups = (unsigned)(total < p.persistGrid ? total : p.persistGrid);
-    hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC>), dim3(groups), dim3(512), 0, stream, p);
+#ifdef NTSAMD_PROBE
+    const bool hasBias = false;         /* a profiling build: the bias pointer is where the time stamps go */
+#else
+    const bool hasBias = p.bias != NULL;
+#endif
+    if (hasBias)
+        hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true>), dim3(groups), dim3(512), 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false>), dim3(groups), dim3(512), 0, stream, p);
     return (int)hipGetLastError();
 }
 

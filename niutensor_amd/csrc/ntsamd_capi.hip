@@ -630,15 +630,16 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     }
     const int cfg = plan.cfg;
     int rc = 0;
-    /* More 256 x 256 tiles than CUs, a half result in whole 16-byte pieces and nothing to read on the way out
-       (no old c, no bias): one workgroup per CU walks over the tiles and fetches the next tile's first slabs
-       before the finished tile's results leave */
+    /* More 256 x 256 tiles than CUs, a half result in whole 16-byte pieces and no old c to read on the way out (a
+       bias by column rides along): one workgroup per CU walks over the tiles and fetches the next tile's first
+       slabs before the finished tile's results leave */
 #ifdef NTSAMD_PROBE
     const bool probeBias = true;        /* a profiling build: the bias pointer is where the time stamps go */
 #else
     const bool probeBias = false;
 #endif
-    if (kind == KIND_F16 && cfg == CFG_256x256 && fetch16 == F16_DIRECT && beta == 0.f && (bias == NULL || probeBias) && colSum == NULL &&
+    const bool biasFits = bias == NULL || probeBias || (biasMode == NTSAMD_BIAS_COL && aligned16(bias));
+    if (kind == KIND_F16 && cfg == CFG_256x256 && fetch16 == F16_DIRECT && beta == 0.f && biasFits && colSum == NULL &&
         s.K >= 256 && tn.f16Persist.load(std::memory_order_relaxed) != 0) {
         const int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
         const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;

@@ -804,6 +804,40 @@ def test_half_walk_over_more_tiles_than_cus(gpu, oracle, ta, tb):
             nt.tuning_set(key, None)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_walk_with_a_bias_by_column(gpu, oracle, ta, tb):
+    """The linear layer in half on more tiles than CUs (MulAndShift, source/tensor/core/arithmetic/MulAndShift.cpp:
+    product, then the bias added along the last dimension), with and without Rectify behind it: the walking kernel
+    takes the bias along; every element against double precision (the bias added before the one rounding), to the
+    last half bit against the one-tile kernels, ragged edges included (columns past N read no bias)."""
+    torch = torch_()
+    knobs = ("NTSAMD_TILE_CFG", "NTSAMD_F16_PINGPONG", "NTSAMD_F16_PERSIST")
+    try:
+        for i, (M, N, K) in enumerate(((4100, 4360, 264), (4352, 4352, 1000))):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 7300 + i, 0, 0.05)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 7400 + i, 0, 0.05)))
+            bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((N,), 7500 + i, 0, 0.5)))
+            ga, gb, gbias = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True), dev_tensor(bias, gpu, True)
+            exact = 0.75 * whole_f64(a, ta, b, tb) + bias.astype(np.float64)[None, :]
+            for act in (nt.ACT_NONE, nt.ACT_RECTIFY):
+                got = {}
+                for walk in (1, 0):
+                    for key, val in zip(knobs, (2, walk, walk)):
+                        nt.tuning_set(key, val)
+                    c = torch.full((M, N), float("nan"), device=gpu, dtype=torch.float16)
+                    nt.matrix_mul(ga, ta, gb, tb, c, 0.75, 0.0, bias=gbias, act=act)
+                    got[walk] = c
+                w, o = got[1].float(), got[0].float()
+                step = torch.maximum(w.abs(), o.abs()) * 2.0 ** -10 + 2.0 ** -24
+                assert bool(((w - o).abs() <= step).all()), "%dx%dx%d act %d: the walk and the one-tile kernels differ" % (M, N, K, act)
+                assert float((w != o).float().mean()) < 1e-3
+                want = np.maximum(exact, 0.0) if act == nt.ACT_RECTIFY else exact
+                assert_fp16(got[1].float().cpu().numpy(), want, what="%dx%dx%d with bias, act %d" % (M, N, K, act))
+    finally:
+        for key in knobs:
+            nt.tuning_set(key, None)
+
+
 def test_config5_ragged_vocab_projection(gpu, oracle):
     """fp32 H[4096x512] x W[30011x512]^T accumulated into C[4096x30011] with beta = 1."""
     torch = torch_()
