@@ -77,6 +77,39 @@ static int launch_convert_t(const void * s, void * t, long long n, hipStream_t s
     return (int)hipGetLastError();
 }
 
+/* rows x cols halves whose rows stand srcPitch elements apart (any even address) copied to rows dstPitch apart
+   (a multiple of 8, 16-byte aligned), the columns from cols to dstPitch filled with zeros: what lets a half operand
+   with rows of odd length travel the 16-byte path afterwards. A lane moves one 16-byte piece of a destination row. */
+__global__ void __launch_bounds__(256)
+repitch_f16_kernel(const half_t * __restrict__ s, long long srcPitch, half_t * __restrict__ t, int dstPitch, long long rows, int cols)
+{
+    typedef half_t HV __attribute__((ext_vector_type(8)));
+    const int perRow = dstPitch / 8;
+    const long long pieces = rows * perRow;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (long long)gridDim.x * 256) {
+        const long long row = i / perRow;
+        const int c = (int)(i - row * perRow) * 8;
+        const half_t * src = s + row * srcPitch + c;
+        HV v;
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            v[e] = c + e < cols ? src[e] : (half_t)0.f;
+        *reinterpret_cast<HV *>(t + row * dstPitch + c) = v;
+    }
+}
+
+int launch_repitch_f16(const void * s, long long srcPitch, void * t, int dstPitch, long long rows, int cols, hipStream_t stream)
+{
+    long long blocks = (rows * (dstPitch / 8) + 255) / 256;
+    if (blocks > 256 * 8)
+        blocks = 256 * 8;
+    if (blocks < 1)
+        blocks = 1;
+    hipLaunchKernelGGL(repitch_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const half_t *>(s), srcPitch, static_cast<half_t *>(t), dstPitch, rows, cols);
+    return (int)hipGetLastError();
+}
+
 /* kinds: 0 float -> half, 1 half -> float, 2 float -> int, 3 int -> float */
 int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream)
 {

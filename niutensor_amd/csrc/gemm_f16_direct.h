@@ -151,7 +151,7 @@ gemm_f16_direct_kernel(const GemmParams p)
             constexpr int LPR = 64 / A_RPC;                  /* lanes per row */
             int krow = ch + A_NCH * (lane / LPR);
             int c = (lane % LPR) * 8;
-            c = m0 + c < M - 8 ? c : M - 8 - m0;
+            c = m0 + c < p.mOper - 8 ? c : p.mOper - 8 - m0;
             aKc[q] = 0;
             aOff[q] = (krow * p.lda + c) * 2;
         }
@@ -170,7 +170,7 @@ gemm_f16_direct_kernel(const GemmParams p)
             constexpr int LPR = 64 / B_RPC;
             int krow = ch + B_NCH * (lane / LPR);
             int c = (lane % LPR) * 8;
-            c = n0 + c < N - 8 ? c : N - 8 - n0;
+            c = n0 + c < p.nOper - 8 ? c : p.nOper - 8 - n0;
             bKc[q] = 0;
             bOff[q] = (krow * p.ldb + c) * 2;
         }
@@ -178,8 +178,8 @@ gemm_f16_direct_kernel(const GemmParams p)
 
     const half_t * aTile = AKC ? A + (size_t)m0 * p.lda + kBeg : A + m0 + (size_t)kBeg * p.lda;
     const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb + kBeg : B + n0 + (size_t)kBeg * p.ldb;
-    const half_t * aEnd = A + (size_t)((AKC ? M : p.K) - 1) * p.lda + (AKC ? p.K : M);
-    const half_t * bEnd = B + (size_t)((BKC ? N : p.K) - 1) * p.ldb + (BKC ? p.K : N);
+    const half_t * aEnd = A + (size_t)((AKC ? M : p.K) - 1) * p.lda + p.mOper;
+    const half_t * bEnd = B + (size_t)((BKC ? N : p.K) - 1) * p.ldb + p.nOper;
 
     const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);
 

@@ -168,7 +168,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
             else {
                 const int krow = ch + 16 * (lane >> 5);
                 int c = (lane & 31) * 8;
-                c = m0 + c < M - 8 ? c : M - 8 - m0;
+                c = m0 + c < p.mOper - 8 ? c : p.mOper - 8 - m0;
                 aKc[q] = 0;
                 aOff[q] = (krow * p.lda + c) * 2;
             }
@@ -186,15 +186,15 @@ gemm_f16_persistent_kernel(const GemmParams p)
             else {
                 const int krow = ch + 16 * (lane >> 5);
                 int c = (lane & 31) * 8;
-                c = n0 + c < N - 8 ? c : N - 8 - n0;
+                c = n0 + c < p.nOper - 8 ? c : p.nOper - 8 - n0;
                 bKc[q] = 0;
                 bOff[q] = (krow * p.ldb + c) * 2;
             }
         }
         aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
         bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-        aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
-        bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
+        aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + p.mOper;
+        bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + p.nOper;
     };
 
     const unsigned ldsBase = (unsigned)(size_t)((__attribute__((address_space(3))) char *)lds);

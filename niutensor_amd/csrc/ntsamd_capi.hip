@@ -31,6 +31,7 @@ int launch_scale(bool half, void * v, long long n, float beta, hipStream_t strea
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream,
                          float * work, size_t workFloats);
 int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream);
+int launch_repitch_f16(const void * s, long long srcPitch, void * t, int dstPitch, long long rows, int cols, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -251,9 +252,11 @@ struct Plan {
      NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment
      NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset)
      NTSAMD_A32_CONVERT=0|1      float a with half b: never / whenever it fits the workspace, round a to half in a pass
-                                 of its own before the product */
+                                 of its own before the product
+     NTSAMD_F16_REPITCH=0|1      half operands with rows that are no whole 16-byte pieces: never / whenever they fit the
+                                 workspace, copied there with padded rows so that the product takes the 16-byte path */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert, f16Repitch;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -268,7 +271,7 @@ const Knob g_knobs[] = {
     {"NTSAMD_F32_R16", &Tuning::f32R16},     {"NTSAMD_F32_SPLIT_ATOMIC", &Tuning::f32SplitAtomic},
     {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
     {"NTSAMD_STORE_HINT", &Tuning::storeHint}, {"NTSAMD_GROUP_M", &Tuning::groupM},
-    {"NTSAMD_A32_CONVERT", &Tuning::a32Convert},
+    {"NTSAMD_A32_CONVERT", &Tuning::a32Convert}, {"NTSAMD_F16_REPITCH", &Tuning::f16Repitch},
 };
 
 const Tuning & tuning()
@@ -498,7 +501,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const Tuning & tn = tuning();
     hipStream_t hs = static_cast<hipStream_t>(stream);
     WorkHold work;
-    bool aInWork = false;
+    bool aInWork = false, repitched = false;
     if (kind_a32(kind) && !noAlloc && !ptrs && !grid && tn.a32Convert.load(std::memory_order_relaxed) != 0) {
         /* A float a is rounded to half on its way into LDS, through registers: that fetch is about half as fast again
            as the one that moves halves straight to LDS. A long product is better served by rounding a once, into
@@ -571,9 +574,57 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
        16-byte pieces travel straight to LDS (the main path); all other half operands, and lists of half
        matrices, are fetched 16 bytes at a time through registers, from any even address. */
     bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
+    p.mOper = colsA;
+    p.nOper = colsB;
+    if ((kind == KIND_F16 || kind == KIND_F16_F32OUT) && vec && !ptrs && !grid && !noAlloc && !aInWork &&
+        tn.f16Repitch.load(std::memory_order_relaxed) != 0) {
+        /* A half operand whose rows are no whole 16-byte pieces (a 30011-word vocabulary) keeps the product off the
+           kernels that move operands straight to LDS; fetched through registers it runs at about two thirds of
+           their speed. Where the operand is small beside the product, a copy with padded rows (zeros in the
+           padding) in the stream's workspace costs less than that: one launch and one pass over the operand. */
+        const bool okA = lda % 8 == 0 && colsA % 8 == 0 && aligned16(a) && strideA % 8 == 0;
+        const bool okB = ldb % 8 == 0 && colsB % 8 == 0 && aligned16(b) && strideB % 8 == 0;
+        const int rowsA = s.aKContig ? s.M : s.K, rowsB = s.bKContig ? s.N : s.K;
+        const int padA = (colsA + 7) / 8 * 8, padB = (colsB + 7) / 8 * 8;
+        /* batches: items that follow each other without a gap (or one shared item) are copied as one run of rows */
+        const bool runA = count == 1 || strideA == 0 || strideA == (long long)rowsA * lda;
+        const bool runB = count == 1 || strideB == 0 || strideB == (long long)rowsB * ldb;
+        const long long itemsA = count == 1 || strideA == 0 ? 1 : count, itemsB = count == 1 || strideB == 0 ? 1 : count;
+        const long long elemsA = okA ? 0 : itemsA * rowsA * padA, elemsB = okB ? 0 : itemsB * rowsB * padB;
+        const double slower = 0.4 * 2.0 * s.M * s.N * s.K * count / 7.0e14;
+        const double pass = (okA ? 0.0 : 2.5e-6 + (double)elemsA * 4.0 / 3.0e12) + (okB ? 0.0 : 2.5e-6 + (double)elemsB * 4.0 / 3.0e12);
+        const bool forced = tn.f16Repitch.load(std::memory_order_relaxed) > 0;
+        if ((!okA || !okB) && (okA || runA) && (okB || runB) && (size_t)(elemsA + elemsB) * 2 <= SPLIT_WORK_BYTES &&
+            (forced || slower > pass)) {
+            work.take_stream(devID, hs);
+            if (work.mem != NULL) {
+                _Float16 * at = reinterpret_cast<_Float16 *>(work.mem);
+                int rc = 0;
+                if (!okA) {
+                    rc = launch_repitch_f16(a, lda, at, padA, itemsA * rowsA, colsA, hs);
+                    p.a = a = at;
+                    p.lda = lda = padA;
+                    p.strideA = strideA = strideA == 0 ? 0 : (long long)rowsA * padA;
+                    p.mOper = padA;
+                }
+                if (!okB && rc == 0) {
+                    _Float16 * bt = at + elemsA;
+                    rc = launch_repitch_f16(b, ldb, bt, padB, itemsB * rowsB, colsB, hs);
+                    p.b = b = bt;
+                    p.ldb = ldb = padB;
+                    p.strideB = strideB = strideB == 0 ? 0 : (long long)rowsB * padB;
+                    p.nOper = padB;
+                }
+                if (rc != 0)
+                    return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+                aInWork = true;                 /* the workspace is taken: k is not cut into pieces */
+                repitched = true;
+            }
+        }
+    }
     int fetch16 = F16_SCALAR;
     if (kind != KIND_F32) {
-        const bool direct = !kind_a32(kind) && vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && colsA % 8 == 0 && colsB % 8 == 0 &&
+        const bool direct = !kind_a32(kind) && vec && !ptrs && lda % 8 == 0 && ldb % 8 == 0 && (repitched || (colsA % 8 == 0 && colsB % 8 == 0)) &&
                             aligned16(a) && aligned16(b) && strideA % 8 == 0 && strideB % 8 == 0 &&
                             (!grid || (grid->strideA1 % 8 == 0 && grid->strideB1 % 8 == 0));
         fetch16 = direct ? F16_DIRECT : (vec ? F16_STAGED : F16_SCALAR);

@@ -452,6 +452,52 @@ def test_half_rows_of_any_length_and_alignment(gpu, oracle, ta, tb, out_float):
             assert_fp16(got[:, -1:], ref[:, -1:], what="last column")
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("out_float", [False, True])
+def test_half_rows_of_any_length_copied_to_padded_rows(gpu, oracle, ta, tb, out_float):
+    """The same operands when the library copies them into its workspace with rows padded to whole 16-byte pieces
+    (zeros in the padding) and runs the product on the kernels that move operands straight to LDS: forced here on
+    small shapes (the library does it by itself where the operand is small beside the product), every tile shape,
+    one operand odd and the other not, both odd, a k that is no multiple of 8, a batch with a shared b."""
+    torch = torch_()
+    odt = torch.float32 if out_float else torch.float16
+    try:
+        nt.tuning_set("NTSAMD_F16_REPITCH", 1)
+        for (M, N, K), cfg in (((203, 301, 77), "0"), ((131, 135, 259), "1"), ((9, 7, 5), "1"), ((1, 300, 1), "0"),
+                               ((70, 67, 1003), "0"), ((264, 301, 96), "2"), ((300, 520, 1056), "2"), ((256, 141, 64), "1")):
+            nt.tuning_set("NTSAMD_TILE_CFG", cfg)
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((M, K), ta), 41)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((K, N), tb), 42)))
+            bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((N,), 43)))
+            ref = oracle.matmul2d(a, ta, b, tb) + bias[None, :]
+            for off in (0, 1):
+                abuf = torch.zeros(a.size + off, device=gpu, dtype=torch.float16)
+                bbuf = torch.zeros(b.size + off, device=gpu, dtype=torch.float16)
+                abuf[off:] = dev_tensor(a.ravel(), gpu, True)
+                bbuf[off:] = dev_tensor(b.ravel(), gpu, True)
+                c = torch.full((M, N), float("nan"), device=gpu, dtype=odt)
+                nt.matrix_mul(abuf[off:].view(a.shape), ta, bbuf[off:].view(b.shape), tb, c,
+                              bias=dev_tensor(bias, gpu, True).to(odt))
+                got = c.float().cpu().numpy()
+                assert_fp16(got, ref, what="%dx%dx%d offset %d" % (M, N, K, off))
+                assert_fp16(got[-1:, :], ref[-1:, :], what="last row")
+                assert_fp16(got[:, -1:], ref[:, -1:], what="last column")
+        # a batch of five a's with rows of 77 against one shared b with rows of 301
+        nt.tuning_set("NTSAMD_TILE_CFG", "1")
+        batch, M, N, K = 5, 67, 301, 77
+        a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform((batch,) + stored((M, K), ta), 44)))
+        b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.uniform(stored((K, N), tb), 45)))
+        ga, gb = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True)
+        c = torch.full((batch, M, N), float("nan"), device=gpu, dtype=odt)
+        na, ma = a.shape[1:]
+        nb, mb = b.shape
+        nt.matrix_mul_batched_strided(ga, ta, gb, tb, c, batch, na * ma, 0, M * N, na, ma, nb, mb, M, N, 0.5, 0.0)
+        for item in range(batch):
+            assert_fp16(c[item].float().cpu().numpy(), oracle.matmul2d(a[item], ta, b, tb, None, 0.5, 0.0), what="item %d" % item)
+    finally:
+        nt.tuning_set("NTSAMD_F16_REPITCH", None)
+
+
 def test_lists_of_half_matrices_with_odd_rows(gpu, oracle):
     """Pointer lists of half matrices take the same 16-byte loads (no alignment to rely on)."""
     torch = torch_()
