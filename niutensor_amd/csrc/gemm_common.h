@@ -88,6 +88,7 @@ struct GemmParams {
     int f16PingPong;                       /* half, 256 x 256 tile: the two wave groups run one phase apart */
     int storeHint;                         /* != 0: the fast epilogues write c through (STORE_WRITE_THROUGH) */
     int persistGrid;                       /* half, 256 x 256 tile: > 0 = that many workgroups walk over all tiles */
+    int persistRows;                       /* rows of the tiles they walk over: 128 (a k-contiguous) or 256 */
     int aF32;                              /* half product whose a is stored as float: rounded to half on its way to LDS */
     /* half, 16-byte path: the number of columns a stored row of a / b really has (the operand's row length, rounded
        up to 8 where the operand is a re-pitched copy whose padding holds zeros) */

@@ -52,12 +52,15 @@
 
 namespace ntsamd {
 
-template <bool AKC, bool BKC, bool HASB>
+template <bool AKC, bool BKC, bool HASB, int BM = 256>
 __global__ void __launch_bounds__(512, 1)
 gemm_f16_persistent_kernel(const GemmParams p)
 {
-    constexpr int BM = 256, BN = 256, WGN = 4, NW = 8, BKT = 32;
-    constexpr int WM = 128, WN = 64, TI = WM / 16, TJ = WN / 16;      /* 16 x 16 blocks of v_mfma_f32_16x16x32_f16: a slab is ONE k step */
+    /* BM = 128 (k-contiguous a only): a tile of 128 x 256 for results with fewer 256 x 256 tiles than the part has
+       CUs; the waves stand 2 x 4 as before, each with 64 x 64 of the tile */
+    static_assert(BM == 256 || (BM == 128 && AKC), "the 128-row tile takes a k-contiguous a");
+    constexpr int BN = 256, WGN = 4, NW = 8, BKT = 32;
+    constexpr int WM = BM / 2, WN = 64, TI = WM / 16, TJ = WN / 16;      /* 16 x 16 blocks of v_mfma_f32_16x16x32_f16: a slab is ONE k step */
     /* LDS, one region per operand, four slabs each.
        k-contiguous: two pair slots of 32 KB; a chunk of 1 KB holds 8 rows x [slab parity][64 bytes], the four 16-byte
            columns of a row's 64 bytes permuted by (row >> 1) & 3. A fragment read has lane l at row l % 16, column
@@ -69,12 +72,13 @@ gemm_f16_persistent_kernel(const GemmParams p)
            8 + s (s = 0..3), i.e. from chunks s and 8 + s, which then lie 64 s and 64 s + 32 bytes into a 256-byte
            line of the 64 banks. */
     constexpr int KC_SLOT = 32 * 1024, KC_REGION = 2 * KC_SLOT;
+    constexpr int A_SLOT = BM * 128;                /* a pair of slabs of a k-contiguous a: BM rows of 128 bytes */
     constexpr int MN_CP = 1088, MN_STAGE = 69 * 256, MN_REGION = 4 * MN_STAGE;
     static_assert(15 * MN_CP + 32 + 1024 <= MN_STAGE, "sixteen chunks must fit a stage");
-    constexpr int A_REGION = AKC ? KC_REGION : MN_REGION, B_REGION = BKC ? KC_REGION : MN_REGION;
-    constexpr int A_HALF = AKC ? KC_SLOT : 2 * MN_STAGE, B_HALF = BKC ? KC_SLOT : 2 * MN_STAGE;   /* where slabs 2 and 3 begin */
+    constexpr int A_REGION = AKC ? 2 * A_SLOT : MN_REGION, B_REGION = BKC ? KC_REGION : MN_REGION;
+    constexpr int A_HALF = AKC ? A_SLOT : 2 * MN_STAGE, B_HALF = BKC ? KC_SLOT : 2 * MN_STAGE;   /* where slabs 2 and 3 begin */
     /* load instructions per wave: KA, KB per PAIR of slabs (k-contiguous), MA, MB per slab (mn-contiguous) */
-    constexpr int KA = AKC ? 4 : 0, KB = BKC ? 4 : 0, MA = AKC ? 0 : 2, MB = BKC ? 0 : 2;
+    constexpr int KA = AKC ? BM / 64 : 0, KB = BKC ? 4 : 0, MA = AKC ? 0 : 2, MB = BKC ? 0 : 2;
     constexpr int KK = KA + KB, MM = MA + MB;
     /* the epilogue's turn through LDS: 16 rows of the wave's 64 columns as halves, rows 144 bytes apart (32 lanes
        that write 8 bytes each, 16 rows x 2 pieces, then cover all 64 banks) */
@@ -85,7 +89,9 @@ gemm_f16_persistent_kernel(const GemmParams p)
        the stores; the first tile's are requested before anything else. */
     constexpr int NB = HASB ? TJ : 0;
     constexpr int NSB = NST + NB;                   /* what lies between a later tile's slabs 0-1 and 2-3 */
-    static_assert(8 * EPI_WAVE <= A_REGION - A_HALF && 8 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
+    /* the staging of the epilogue: waves 0 .. EPI_IN_A - 1 in the second half of a's region, the others in b's */
+    constexpr int EPI_IN_A = BM == 256 ? 4 : 2;
+    static_assert(EPI_IN_A * 2 * EPI_WAVE <= A_REGION - A_HALF && (NW - EPI_IN_A) * 2 * EPI_WAVE <= B_REGION - B_HALF, "the epilogue's staging must fit the second halves");
     static_assert(A_REGION + B_REGION <= 160 * 1024, "the stages must fit LDS");
     static_assert(MM + NSB + KK + 2 * MM < 64, "the wait counter has six bits");
 
@@ -204,7 +210,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
     auto issue_pair = [&](int kt) {
         const int k0 = kt * BKT;
         const bool tail = k0 + 2 * BKT > K;
-        const unsigned slot = (unsigned)(((kt >> 1) & 1) * KC_SLOT);
+        const unsigned slot = (unsigned)(((kt >> 1) & 1) * KC_SLOT), slotA = (unsigned)(((kt >> 1) & 1) * A_SLOT);
         if constexpr (AKC) {
             const half_t * ab = aTile + k0;
             const i32x4 ad = make_desc(ab, (long long)(aEnd - ab) * 2);
@@ -213,7 +219,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
                 int off = aOff[q];
                 if (tail && k0 + aKc[q] >= K)
                     off = NTSAMD_OOB_OFFSET;
-                lds_dma16(ad, ldsBase + slot + (unsigned)((wave * KA + q) * 1024), off);
+                lds_dma16(ad, ldsBase + slotA + (unsigned)((wave * KA + q) * 1024), off);
             }
         }
         if constexpr (BKC) {
@@ -279,13 +285,13 @@ gemm_f16_persistent_kernel(const GemmParams p)
         }
     }
     /* where slab kt of an operand begins inside its region */
-    auto slab_base = [&](bool kc, int kt) {
-        return kc ? ((kt >> 1) & 1) * KC_SLOT + (kt & 1) * 512 : (kt & 3) * MN_STAGE;
+    auto slab_base = [&](bool kc, int slotBytes, int kt) {
+        return kc ? ((kt >> 1) & 1) * slotBytes + (kt & 1) * 512 : (kt & 3) * MN_STAGE;
     };
 
     f16x8 fa[TI], fb[TJ];
     auto read_frags = [&](int kt) {
-        const char * sa = lds + slab_base(AKC, kt), * sb = lds + slab_base(BKC, kt);
+        const char * sa = lds + slab_base(AKC, A_SLOT, kt), * sb = lds + slab_base(BKC, KC_SLOT, kt);
 #pragma unroll
         for (int i = 0; i < TI; i++) {
             if constexpr (AKC)
@@ -445,7 +451,7 @@ gemm_f16_persistent_kernel(const GemmParams p)
         const unsigned cOffW = colW + 8 <= N ? (unsigned)(rdRow * p.ldc + colW) * 2u : (unsigned)NTSAMD_OOB_OFFSET;
         /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's; two buffers per wave, so
            that block row i + 1 is on its way into LDS while block row i comes back out */
-        char * mine = lds + (wave < 4 ? A_HALF : A_REGION + B_HALF) + (wave & 3) * (2 * EPI_WAVE);
+        char * mine = lds + (wave < EPI_IN_A ? A_HALF + wave * (2 * EPI_WAVE) : A_REGION + B_HALF + (wave - EPI_IN_A) * (2 * EPI_WAVE));
         auto put = [&](int i) {
             char * wr = mine + (i & 1) * EPI_WAVE + rho * EPI_PITCH + g4 * 8;
 #pragma unroll
@@ -556,7 +562,9 @@ template <bool AKC, bool BKC>
 static int launch_f16_persistent(const GemmParams & p0, hipStream_t stream)
 {
     GemmParams p = p0;
-    p.tilesM = (p.M + 255) / 256;
+    /* p.persistRows: 128 = tiles of 128 x 256 (a k-contiguous), otherwise 256 x 256 */
+    const int bm = AKC && p.persistRows == 128 ? 128 : 256;
+    p.tilesM = (p.M + bm - 1) / bm;
     p.tilesN = (p.N + 255) / 256;
     p.splits = 1;
     const long long total = (long long)p.tilesM * p.tilesN * p.batch;
@@ -566,6 +574,15 @@ static int launch_f16_persistent(const GemmParams & p0, hipStream_t stream)
 #else
     const bool hasBias = p.bias != NULL;
 #endif
+    if constexpr (AKC) {
+        if (bm == 128) {
+            if (hasBias)
+                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true, 128>), dim3(groups), dim3(512), 0, stream, p);
+            else
+                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false, 128>), dim3(groups), dim3(512), 0, stream, p);
+            return (int)hipGetLastError();
+        }
+    }
     if (hasBias)
         hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true>), dim3(groups), dim3(512), 0, stream, p);
     else

@@ -248,7 +248,8 @@ struct Plan {
      NTSAMD_F32_R16=0            no 16-row MFMAs for float products of at most 16 rows
      NTSAMD_F32_SPLIT_ATOMIC=1   float pieces of k add to c with atomics (no workspace, no fixed order)
      NTSAMD_F16_PINGPONG=0       half, 256 x 256 tile: the main loop in which both waves of a SIMD meet one barrier
-     NTSAMD_F16_PERSIST=0        half, 256 x 256 tile: one workgroup per tile, never one per CU that walks over tiles
+     NTSAMD_F16_PERSIST=0|2|3|4  half: never one workgroup per CU that walks over tiles / always over 256 x 256 tiles / never
+                                 over 128 x 256 tiles / always over 128 x 256 tiles (where the kernel can take the product)
      NTSAMD_STORE_HINT=0|1       results never / always written through, whatever their alignment
      NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset)
      NTSAMD_A32_CONVERT=0|1      float a with half b: never / whenever it fits the workspace, round a to half in a pass
@@ -690,22 +691,38 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const bool probeBias = false;
 #endif
     const bool biasFits = bias == NULL || probeBias || (biasMode == NTSAMD_BIAS_COL && aligned16(bias));
-    if (kind == KIND_F16 && cfg == CFG_256x256 && fetch16 == F16_DIRECT && beta == 0.f && biasFits && colSum == NULL &&
+    int launchCfg = cfg;
+    if (kind == KIND_F16 && fetch16 == F16_DIRECT && beta == 0.f && biasFits && colSum == NULL && plan.splits == 1 &&
         s.K >= 256 && tn.f16Persist.load(std::memory_order_relaxed) != 0) {
         const int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
         const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;
+        const long long tiles128 = (long long)((s.M + 127) / 128) * ((s.N + 255) / 256) * count;
         const bool wide = ldc % 8 == 0 && s.N % 8 == 0 && aligned16(c) && strideC % 8 == 0 &&
                           (!grid || grid->strideC1 % 8 == 0);
+        const int knob = tn.f16Persist.load(std::memory_order_relaxed);
         /* from one tile per CU on: with CUs to spare the part is not held back by its power limit, and the older
            kernels' longer lead of the loads counts for more than the energy this one saves (measured: 4096^3 112 ->
            103 us, but 2048 x 4096 x 8192 on 128 CUs 147 -> 177 us with both operands k-contiguous) */
-        if (wide && cus > 0 && (tiles >= cus || tn.f16Persist.load(std::memory_order_relaxed) == 2))
+        if (cfg == CFG_256x256 && wide && cus > 0 && (tiles >= cus || knob == 2)) {
             p.persistGrid = cus;
-            /* four tile rows share a sweep over the tile columns: the 32 tiles an XCD works on at a time are 4 x 8,
-               the same twelve operand panels as 8 x 4, and their stores spread over twice as many columns of c
-               (measured 1-2 % ahead of 8 at 8192 x 4096 x 1024, level elsewhere) */
-            if (tn.groupM.load(std::memory_order_relaxed) <= 0)
-                p.groupM = 4;
+            p.persistRows = 256;
+        }
+        /* fewer 256 x 256 tiles than CUs, but tiles of 128 x 256 give most CUs exactly one (more than one each for
+           some would be a second round at a quarter of the part): the same kernel on tiles of half the height (a
+           k-contiguous), whatever tile shape the estimate chose for the one-tile kernels. Measured at 256 such
+           tiles: k = 4096 75 -> 66 us (b k x n) and 82 -> 67 us (b n x k), k = 2048 40 -> 36 and 43 -> 36, k = 1024
+           21.7 -> 21.2 and 22.8 -> 21.2, k = 512 level or behind. */
+        else if (s.aKContig && wide && cus > 0 &&
+                 ((tiles < cus && tiles128 * 4 >= (long long)cus * 3 && tiles128 <= cus && s.K >= 1024 && knob != 3) || knob == 4)) {
+            p.persistGrid = cus;
+            p.persistRows = 128;
+            launchCfg = CFG_256x256;
+        }
+        /* four tile rows share a sweep over the tile columns: the 32 tiles an XCD works on at a time are 4 x 8,
+           the same twelve operand panels as 8 x 4, and their stores spread over twice as many columns of c
+           (measured 1-2 % ahead of 8 at 8192 x 4096 x 1024, level elsewhere) */
+        if (p.persistGrid > 0 && tn.groupM.load(std::memory_order_relaxed) <= 0)
+            p.groupM = p.persistRows == 128 ? 8 : 4;
     }
     p.splits = 1;
     if (plan.splits > 1) {
@@ -752,9 +769,9 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     else {
         bool outF32 = kind_out_f32(kind);
         if (s.aKContig)
-            rc = s.bKContig ? launch_f16_nt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_nn(p, ptrs, fetch16, outF32, cfg, hs);
+            rc = s.bKContig ? launch_f16_nt(p, ptrs, fetch16, outF32, launchCfg, hs) : launch_f16_nn(p, ptrs, fetch16, outF32, launchCfg, hs);
         else
-            rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, cfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, cfg, hs);
+            rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, launchCfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, launchCfg, hs);
     }
     if (rc == 0 && p.splits > 1 && viaWork)
         rc = launch_split_reduce(p, kind != KIND_F16, hs);

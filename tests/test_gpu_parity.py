@@ -884,6 +884,44 @@ def test_half_walk_with_a_bias_by_column(gpu, oracle, ta, tb):
             nt.tuning_set(key, None)
 
 
+@pytest.mark.parametrize("tb", (X_NOTRANS, X_TRANS))
+def test_half_walk_over_tiles_of_128_rows(gpu, oracle, tb):
+    """Results with fewer 256 x 256 tiles than CUs but enough tiles of 128 x 256: the walking kernel on the lower tile
+    (a stored row by row). Ragged edges, a k that ends inside a pair of slabs, with and without a bias, a batch;
+    every element against double precision, and to the last half bit against the one-tile kernels."""
+    torch = torch_()
+    ta = X_NOTRANS
+    try:
+        for i, (M, N, K, batch, with_bias) in enumerate(((4096, 2048, 520, 1, False), (3900, 2100, 264, 1, True),
+                                                         (4000, 1800, 1000, 1, True), (1000, 1100, 328, 9, False))):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch,) + stored((M, K), ta), 7600 + i, 0, 0.05)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((batch,) + stored((K, N), tb), 7700 + i, 0, 0.05)))
+            bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((N,), 7800 + i, 0, 0.5)))
+            ga, gb = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True)
+            gbias = dev_tensor(bias, gpu, True) if with_bias else None
+            got = {}
+            for walk in (4, 0):
+                nt.tuning_set("NTSAMD_F16_PERSIST", walk)
+                c = torch.full((batch, M, N), float("nan"), device=gpu, dtype=torch.float16)
+                if batch == 1:
+                    nt.matrix_mul(ga[0], ta, gb[0], tb, c[0], 0.75, 0.0, bias=gbias)
+                else:
+                    na, ma = a.shape[1:]
+                    nb, mb = b.shape[1:]
+                    nt.matrix_mul_batched_strided(ga, ta, gb, tb, c, batch, na * ma, nb * mb, M * N, na, ma, nb, mb, M, N, 0.75, 0.0)
+                got[walk] = c
+            w, o = got[4].float(), got[0].float()
+            step = torch.maximum(w.abs(), o.abs()) * 2.0 ** -10 + 2.0 ** -24
+            assert bool(((w - o).abs() <= step).all()), "%dx%dx%d x%d: the walk and the one-tile kernels differ" % (M, N, K, batch)
+            assert float((w != o).float().mean()) < 1e-3
+            res = w.cpu().numpy()
+            for item in range(batch):
+                want = 0.75 * whole_f64(a[item], ta, b[item], tb) + (bias.astype(np.float64)[None, :] if with_bias else 0.0)
+                assert_fp16(res[item], want, what="%dx%dx%d item %d" % (M, N, K, item))
+    finally:
+        nt.tuning_set("NTSAMD_F16_PERSIST", None)
+
+
 def test_config5_ragged_vocab_projection(gpu, oracle):
     """fp32 H[4096x512] x W[30011x512]^T accumulated into C[4096x30011] with beta = 1."""
     torch = torch_()
