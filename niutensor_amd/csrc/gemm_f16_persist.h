@@ -1,39 +1,30 @@
 /*
- * fp16 GEMM for gfx950, 256 x 256 tile, persistent form: one workgroup per CU walks over
- * several tiles of c, and the first four slabs of the NEXT tile are on their way to LDS
- * before the finished tile's results leave. Same arithmetic, same LDS layouts and the same
- * ping-pong main loop as gemm_f16_direct_kernel<..., PP = true> (see gemm_f16_direct.h for
- * both); the results are the same bits.
+ * fp16 GEMM for gfx950, 256 x 256 tile (128 x 256 where the result is small), persistent form: one workgroup per
+ * CU walks over several tiles of c, and the first four slabs of the NEXT tile are on their way to LDS before the
+ * finished tile's results leave. The LDS layout of mn-contiguous operands and the ping-pong main loop (two wave
+ * groups one phase apart, one barrier pair per slab) are those of gemm_f16_direct_kernel<..., PP = true> (see
+ * gemm_f16_direct.h); the MFMA is v_mfma_f32_16x16x32_f16 here, which adds the 32 products of a k step in another
+ * order than the 32 x 32 x 16 form of the other kernels: the two agree to the last half bit or one step apart.
  *
- * Why: a 256 x 256 tile ends with 128 KB of stores per CU. When every CU runs one tile per
- * workgroup, all CUs of a round finish together, 33 MB leave at once (about 7 us at the rate
- * the part sustains for stores alone), nothing is multiplied meanwhile, and the next round of
- * workgroups starts cold: launch, four slabs to fetch before the first MFMA. Here the store
- * burst of a tile overlaps the main loop of the next one, and that loop starts with its
- * operands already in LDS. Only the last tile's stores stay exposed.
+ * Why: a 256 x 256 tile ends with 128 KB of stores per CU. When every CU runs one tile per workgroup, all CUs of a
+ * round finish together, 33 MB leave at once (about 6 us at the rate the fabric takes stores), nothing is
+ * multiplied meanwhile, and the next round of workgroups starts cold: launch, four slabs to fetch before the first
+ * MFMA. Here the next tile's main loop starts with its operands already in LDS.
  *
  * What that takes:
- *   - The epilogue must be short and must write whole 128-byte lines. Turning the accumulators
- *     through LDS two bytes at a time (a lane of v_mfma_f32_32x32x16_f16's result holds one
- *     COLUMN of its block) took 3.9 us per tile in this kernel, measured with time stamps: more
- *     than the stores themselves. Here the MFMA computes the TRANSPOSED block instead (the b
- *     fragment goes in as the first operand, the a fragment as the second: the fragment layouts
- *     of the two operands are the same), so a lane holds one ROW of c, and the columns of the b
- *     tile are dealt to the lanes of its fragment in a permuted order (groups of four columns,
- *     see `pcol`) chosen so that eight consecutive accumulator registers of a lane are eight
- *     consecutive columns: 16 bytes. Storing those straight to memory was measured too: 32
- *     rows x 32 bytes per instruction, four times the cache lines touched, 4.8 us per tile and
- *     the next tile's loads held up behind them. So the 16-byte pieces still cross LDS, 32
- *     rows of the wave's 64 columns at a time (4 writes and 4 reads of 16 bytes per lane where
- *     there were 32 writes of 2 bytes), and leave as whole lines, 8 rows per instruction. The
- *     order of the sum over k is unchanged: the results are the same bits.
- *   - The staging area lies in stages 2 and 3, so the next tile's slabs 0 and 1 are requested
- *     before the epilogue and slabs 2 and 3 after it, behind a barrier (a wave's loads land
- *     anywhere in a stage, also where another wave is still staging).
- *   - Vector-memory operations complete in issue order, loads and stores alike, and one
- *     counter (vmcnt) counts them all. A follow-on tile's slabs 0 and 1 are requested BEFORE
- *     the finished tile's NST stores and slabs 2 and 3 after them, so "slab 0 has landed" is
- *     vmcnt <= 3 NL + NST and "slab 1 has landed" is vmcnt <= 2 NL + NST; from slab 2 on the
+ *   - The epilogue must be short and must write whole 128-byte lines. The b fragment goes into the MFMA as the
+ *     FIRST operand, so result register r of lane l is row l % 16 of its 16 x 16 block and column 4 (l / 16) + r:
+ *     a lane holds four consecutive columns of one row, 8 bytes of c. Block row by block row the wave writes those
+ *     8-byte pieces to its own piece of LDS and reads whole rows back, 8 lanes to a row of the wave's 64 columns:
+ *     a store instruction covers 8 rows of 128 contiguous bytes. Activation and cache policy of the stores are
+ *     compile-time constants of the epilogue's code (tested per value they cost four vector instructions each,
+ *     3.6 us per tile); the turn through LDS is double-buffered.
+ *   - The staging area lies where slabs 2 and 3 go, so the next tile's slabs 0 and 1 are requested before the
+ *     epilogue and slabs 2 and 3 after it, behind a barrier (a wave's loads land anywhere in a stage, also where
+ *     another wave is still staging).
+ *   - Vector-memory operations complete in issue order, loads and stores alike, and one counter (vmcnt) counts
+ *     them all. A follow-on tile's slabs 0 and 1 are requested BEFORE the finished tile's NST stores and slabs 2
+ *     and 3 after them; the waits of the first two slabs count the stores in (see main_loop), from slab 2 on the
  *     stores are older than every load still awaited.
  *   - A k-contiguous operand is fetched TWO slabs at a time: a slab of 32 k is 64 bytes of a row, half a cache
  *     line, and fetched slab by slab every line crossed the path from L2 twice (measured with the same kernel
@@ -43,9 +34,11 @@
  *     operand are two pair slots, and a pair is requested at the start of an even slab, two slabs before its
  *     first half is read. An mn-contiguous operand keeps its slab-by-slab fetch three slabs ahead (its rows are
  *     whole lines already). The two operands have their own regions of LDS for that.
- *   - No loads in the epilogue: the compiler cannot see the LDS-direct loads (inline
- *     assembly) and would wait for ALL of them before using a loaded value. Hence beta == 0
- *     and no bias here; products with either run on the one-tile-per-workgroup kernels.
+ *   - The only loads besides the operands' are the bias (HASB): four 8-byte loads per lane and tile, requested
+ *     between the finished tile's stores and the next tile's slabs 2 and 3 and counted with the stores; their
+ *     first use is pinned behind the main loop, where nothing is in flight, because the compiler cannot see the
+ *     LDS-direct loads (inline assembly) and would otherwise wait for ALL of them wherever it first touched the
+ *     bias. Old c (beta != 0) is not read here: such products run on the one-tile-per-workgroup kernels.
  */
 #pragma once
 #include "gemm_f16_direct.h"
