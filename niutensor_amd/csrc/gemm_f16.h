@@ -146,7 +146,10 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         C = static_cast<OutT *>(p.c) + batch_offset(tc.batch, p.batchInner, p.strideC, p.strideC1);
     }
 
-    const int M = p.M, N = p.N, K = p.K;
+    /* K: the k range of this workgroup, all of p.K or one of p.splits pieces that begins at kBeg (p.kPerSplit is a
+       multiple of the slab depth, so only the last piece has a ragged end, and that is where the operands end too) */
+    const int kBeg = p.splits > 1 ? tc.split * p.kPerSplit : 0;
+    const int M = p.M, N = p.N, K = p.splits > 1 && kBeg + p.kPerSplit < p.K ? p.kPerSplit : p.K - kBeg;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);      /* the same in every lane: said explicitly, so that descriptors built from it are scalars */
@@ -197,10 +200,10 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
         }
     }
 
-    const AT * aTile = AKC ? A + (size_t)m0 * p.lda : A + m0;
-    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb : B + n0;
-    const AT * aEnd = A + (size_t)((AKC ? M : K) - 1) * p.lda + (AKC ? K : M);
-    const half_t * bEnd = B + (size_t)((BKC ? N : K) - 1) * p.ldb + (BKC ? K : N);
+    const AT * aTile = AKC ? A + (size_t)m0 * p.lda + kBeg : A + m0 + (size_t)kBeg * p.lda;
+    const half_t * bTile = BKC ? B + (size_t)n0 * p.ldb + kBeg : B + n0 + (size_t)kBeg * p.ldb;
+    const AT * aEnd = A + (size_t)((AKC ? M : p.K) - 1) * p.lda + (AKC ? p.K : M);
+    const half_t * bEnd = B + (size_t)((BKC ? N : p.K) - 1) * p.ldb + (BKC ? p.K : N);
 
     /* a float a waits in the ring as it came (two registers of four floats per piece) and is rounded when it moves on to LDS */
     f16x8 ra[AF32 ? 1 : RING][AF32 ? 1 : NA], rb[RING][NB];
@@ -500,6 +503,27 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
 
     /* ---- epilogue: accumulator register r of lane l is element
        (8*(r/4) + 4*(l/32) + r%4, l%32) of its 32x32 block ------------------------ */
+    if (p.splits > 1) {
+        /* one of several workgroups that share this tile: the partial tile goes to the workspace as it is (splits x
+           batch dense M x N fp32 matrices), and split_reduce.hip adds the pieces in their order and applies alpha,
+           beta, bias and activation */
+        float * w = p.splitWork + ((size_t)tc.split * p.batch + tc.batch) * M * N;
+#pragma unroll
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col < N) {
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                        if (row < M)
+                            w[(size_t)row * N + col] = acc[i][j][r];
+                    }
+            }
+        }
+        return;
+    }
     const float alpha = p.alpha, beta = p.beta;
     const OutT * __restrict__ bias = static_cast<const OutT *>(p.bias);
     const int biasMode = p.biasMode;
@@ -572,8 +596,10 @@ static int launch_f16_one(const GemmParams & p0, const PT & tab, hipStream_t str
     GemmParams p = p0;
     p.tilesM = (p.M + S::BM - 1) / S::BM;
     p.tilesN = (p.N + S::BN - 1) / S::BN;
-    p.splits = 1;
-    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch));
+    /* pieces of k meet in a workspace (the 16-byte fetch, no lists of matrices) or there are none */
+    if (!(VEC && sizeof(PT) == 1 && p.splits > 1 && p.splitWork != NULL))
+        p.splits = 1;
+    dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
     hipLaunchKernelGGL((gemm_f16_kernel<OutT, S::BM, S::BN, 32, S::WGM, S::WGN, S::MINW16, AKC, BKC, VEC, PT, AT>),
                        grid, dim3(S::WGM * S::WGN * 64), 0, stream, p, tab);
     return (int)hipGetLastError();

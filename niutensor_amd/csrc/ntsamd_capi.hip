@@ -643,7 +643,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     const bool atomicAble = !half && vec && !ptrs && act == ACT_NONE && dense;
     const bool atomicAsked = atomicAble && !noAlloc && tn.f32SplitAtomic.load(std::memory_order_relaxed) > 0;
     /* (the half copy of a float a has the workspace to itself) */
-    const bool maySplit = !aInWork && (atomicAsked || ((half ? fetch16 == F16_DIRECT : vec) && !ptrs));
+    const bool maySplit = !aInWork && (atomicAsked || ((half ? fetch16 == F16_DIRECT || fetch16 == F16_STAGED : vec) && !ptrs));
     const size_t workBytes = atomicAsked ? 0 : (noAlloc ? STATIC_SCRATCH_BYTES : SPLIT_WORK_BYTES);
     /* pieces that meet in a workspace gather no column sums: cutting costs a pass of its own over b then (a
        launch, b read once more) */
@@ -774,7 +774,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             rc = s.bKContig ? launch_f16_tt(p, ptrs, fetch16, outF32, launchCfg, hs) : launch_f16_tn(p, ptrs, fetch16, outF32, launchCfg, hs);
     }
     if (rc == 0 && p.splits > 1 && viaWork)
-        rc = launch_split_reduce(p, kind != KIND_F16, hs);
+        rc = launch_split_reduce(p, kind == KIND_F32 || kind_out_f32(kind), hs);
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

@@ -234,6 +234,49 @@ def test_half_products_cut_along_k(gpu, oracle, ta, tb):
                         assert_fp16(c.float().cpu().numpy(), ref, what=what)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_products_fetched_through_registers_cut_along_k(gpu, oracle, ta, tb):
+    """The same cut for the kernel that fetches its operands through registers (rows of any length: the gradient
+    of a layer with a 30011-word vocabulary has few tiles and k = 30011): forced on both tile shapes with 2 and 16
+    pieces, odd row lengths, a ragged last piece, bases that are only 2-byte aligned."""
+    torch = torch_()
+    shapes = [(9, 7, 263), (72, 135, 1001), (40, 51, 1024), (130, 66, 4099)]
+    try:
+        nt.tuning_set("NTSAMD_F16_FETCH", 2)
+        for cfg, pieces in (("0", "2"), ("0", "16"), ("1", "2"), ("1", "16"), (None, None)):
+            for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces)):
+                nt.tuning_set(key, val)
+            for i, (M, N, K) in enumerate(shapes if cfg else shapes[-1:]):
+                a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 8600 + i, 0, 0.5)))
+                b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 8700 + i, 0, 0.5)))
+                bias = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((N,), 8800 + i)))
+                abuf = torch.zeros(a.size + 1, device=gpu, dtype=torch.float16)
+                bbuf = torch.zeros(b.size + 1, device=gpu, dtype=torch.float16)
+                abuf[1:] = dev_tensor(a.ravel(), gpu, True)
+                bbuf[1:] = dev_tensor(b.ravel(), gpu, True)
+                for out_float in (False, True):
+                    c0 = oracle.uniform((M, N), 8900 + i)
+                    if not out_float:
+                        c0 = oracle.from_f16_bits(oracle.to_f16_bits(c0))
+                    for alpha, beta, with_bias, act in ((1.0, 0.0, False, nt.ACT_NONE), (0.5, 1.0, True, nt.ACT_RECTIFY)):
+                        ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
+                        if with_bias:
+                            ref = ref + bias[None, :]
+                        if act == nt.ACT_RECTIFY:
+                            ref = np.maximum(ref, 0)
+                        c = dev_tensor(c0, gpu, not out_float) if beta != 0 else \
+                            torch.full((M, N), float("nan"), device=gpu, dtype=torch.float32 if out_float else torch.float16)
+                        nt.matrix_mul(abuf[1:].view(a.shape), ta, bbuf[1:].view(b.shape), tb, c, alpha, beta,
+                                      bias=dev_tensor(bias, gpu, not out_float) if with_bias else None, act=act)
+                        what = "cfg%s pieces=%s %dx%dx%d alpha=%g beta=%g float=%s" % (cfg, pieces, M, N, K, alpha, beta, out_float)
+                        if out_float:
+                            assert_fp32(c.cpu().numpy(), ref, K, what=what)
+                        else:
+                            assert_fp16(c.float().cpu().numpy(), ref, what=what)
+    finally:
+        nt.tuning_set("NTSAMD_F16_FETCH", None)
+
+
 def test_batches_of_half_products_cut_along_k(gpu, oracle):
     """Three products with their own strides between them and rows of c longer than the result is wide (the heads
     of a merged tensor): every piece of every item finds its place in the workspace and in c, and what lies
