@@ -112,7 +112,12 @@ XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * 
 void _AmdAttentionContext(const XTensor * probs, const XTensor * v, XTensor * out, int nhead)
 {
     CheckNTErrors((probs && v && out), "Empty input tensors!");
-    CheckNTErrors((probs->dataType == v->dataType && probs->dataType == out->dataType), "Unmatched data types!");
+    /* float probabilities may meet half values (the half training path keeps the softmax and its dropout in float,
+       source/sample/transformer/submodel/Attention.cpp:215-232, and converts before the product): the kernel rounds
+       them to half where it fetches them, the ConvertDataType pass and its temporary are not needed */
+    CheckNTErrors((v->dataType == out->dataType &&
+                   (probs->dataType == v->dataType || (probs->dataType == X_FLOAT && v->dataType == X_FLOAT16))),
+                  "Unmatched data types!");
     CheckNTErrors((v->dataType == X_FLOAT || v->dataType == X_FLOAT16), "TODO!");
     CheckNTErrors((v->order >= 2 && out->order == v->order && probs->order == v->order + 1),
                   "Input tensors must have the same order >= 2!");

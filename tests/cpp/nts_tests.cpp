@@ -726,6 +726,19 @@ static bool TestAttention()
                     fprintf(stderr, "attention context case %d masked %d err=%g\n", ci, masked, ce);
                     ok = false;
                 }
+                /* the half model's form of the same step: the float probabilities straight against half values
+                   (no ConvertDataType of the probabilities), a half context */
+                XTensor vHalf = ConvertDataType(*gv, X_FLOAT16);
+                XTensor ctxHalf = AmdAttentionContext(probs, vHalf, nh);
+                ok = ok && ctxHalf.dataType == X_FLOAT16 && ctxHalf.order == 3 && ctxHalf.dimSize[2] == H;
+                XTensor ctxBack = ConvertDataType(ctxHalf, X_FLOAT);
+                std::vector<float> hgot(B * lq * H);
+                ctxBack.GetData(hgot.data());
+                float he = MaxRelErr(hgot, ref);
+                if (!(he < 1e-2F)) {
+                    fprintf(stderr, "attention context with half values case %d masked %d err=%g\n", ci, masked, he);
+                    ok = false;
+                }
             }
             float e = MaxRelErr(got, ref);
             if (!(e < 1e-5F * sqrtf((float)(H / nh + lk)))) {
