@@ -38,17 +38,24 @@
  *     between the finished tile's stores and the next tile's slabs 2 and 3 and counted with the stores; their
  *     first use is pinned behind the main loop, where nothing is in flight, because the compiler cannot see the
  *     LDS-direct loads (inline assembly) and would otherwise wait for ALL of them wherever it first touched the
- *     bias. Old c (beta != 0) is not read here: such products run on the one-tile-per-workgroup kernels.
+ *     bias.
+ *   - Old c (HASC, beta != 0) is read in the epilogue, a block row ahead, as the lane's own 8-byte pieces, and added
+ *     in fp32 before the one rounding. Those loads are the compiler's, and it waits for them by counting what IT
+ *     has issued: so in this form nothing of the next tile is requested before the epilogue is over (the
+ *     accounting of the first slab is then that of a workgroup's first tile).
  */
 #pragma once
 #include "gemm_f16_direct.h"
 
 namespace ntsamd {
 
-template <bool AKC, bool BKC, bool HASB, int BM = 256>
+template <bool AKC, bool BKC, bool HASB, int BM = 256, bool HASC = false>
 __global__ void __launch_bounds__(512, 1)
 gemm_f16_persistent_kernel(const GemmParams p)
 {
+    /* HASC: beta != 0, the old c is read on the way out. Its loads come from the compiler (it places their waits), so
+       nothing of the next tile may be in flight behind the compiler's back while they are: the next tile's first
+       slabs are requested after the epilogue, not before it (about 2 us per tile that the other form hides). */
     /* BM = 128 (k-contiguous a only): a tile of 128 x 256 for results with fewer 256 x 256 tiles than the part has
        CUs; the waves stand 2 x 4 as before, each with 64 x 64 of the tile */
     static_assert(BM == 256 || (BM == 128 && AKC), "the 128-row tile takes a k-contiguous a");
@@ -445,6 +452,22 @@ gemm_f16_persistent_kernel(const GemmParams p)
         /* the staging lies where slabs 2 and 3 go: four waves in a's region, four in b's; two buffers per wave, so
            that block row i + 1 is on its way into LDS while block row i comes back out */
         char * mine = lds + (wave < EPI_IN_A ? A_HALF + wave * (2 * EPI_WAVE) : A_REGION + B_HALF + (wave - EPI_IN_A) * (2 * EPI_WAVE));
+        /* HASC: the old values of a lane's own pieces (row rho of block row i, columns 16 j + 4 g4 .. + 3: 8 bytes),
+           fetched one block row ahead and added in fp32 before the one rounding */
+        const float beta = p.beta;
+        f16x4 cold[HASC ? 2 : 1][HASC ? TJ : 1];
+        auto load_c = [&](int i) {
+            if constexpr (HASC) {
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                    const int col = en0 + wn0 + 16 * j + 4 * g4;
+                    const unsigned off = col < N ? (unsigned)(i * 16 + rho) * rowPitch + (unsigned)col * 2u : (unsigned)NTSAMD_OOB_OFFSET;
+                    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(cr, (int)off, 0, 0);
+                    cold[i & 1][j] = __builtin_bit_cast(f16x4, v);
+                }
+            }
+        };
         auto put = [&](int i) {
             char * wr = mine + (i & 1) * EPI_WAVE + rho * EPI_PITCH + g4 * 8;
 #pragma unroll
@@ -452,15 +475,20 @@ gemm_f16_persistent_kernel(const GemmParams p)
                 f16x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
+                    float x = alpha * acc[i][j][e];
                     if constexpr (HASB)
-                        v[e] = (half_t)activate(alpha * acc[i][j][e] + (float)bv[j][e], act);
-                    else
-                        v[e] = (half_t)activate(alpha * acc[i][j][e], act);
+                        x += (float)bv[j][e];
+                    if constexpr (HASC)
+                        x += beta * (float)cold[i & 1][j][e];
+                    v[e] = (half_t)activate(x, act);
                 }
                 *reinterpret_cast<f16x4 *>(wr + j * 32) = v;
             }
         };
+        load_c(0);
         put(0);
+        if (TI > 1)
+            load_c(1);
 #pragma unroll
         for (int i = 0; i < TI; i++) {
             /* the wave's own lanes exchange data through LDS: LDS executes one wave's instructions in order, the
@@ -475,6 +503,8 @@ gemm_f16_persistent_kernel(const GemmParams p)
                 v[q] = *reinterpret_cast<const f32x4 *>(rd + q * 8 * EPI_PITCH);
             if (i + 1 < TI)
                 put(i + 1);
+            if (i + 2 < TI)
+                load_c(i + 2);
 #pragma unroll
             for (int q = 0; q < 2; q++)
                 __builtin_amdgcn_raw_buffer_store_b128(v[q], cr, (int)(cOffW + (unsigned)(i * 16 + q * 8) * rowPitch), 0, aux);
@@ -521,9 +551,11 @@ gemm_f16_persistent_kernel(const GemmParams p)
             for (int j = 0; j < TJ; j++)
                 asm volatile("" : "+v"(bv[j]));
         }
-        if (more) {
-            adopt(next);
-            issue_two(0);
+        if constexpr (!HASC) {
+            if (more) {
+                adopt(next);
+                issue_two(0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         NTSAMD_STAMP(more ? 5 : 11);
@@ -532,13 +564,23 @@ gemm_f16_persistent_kernel(const GemmParams p)
         NTSAMD_STAMP(more ? 6 : 12);
         if (!more)
             break;
+        if constexpr (HASC)
+            adopt(next);
         load_bias(n0);
         /* where slabs 2 and 3 go is free once every wave has read its staged rows back */
         wait_lgkmcnt0();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue_two(2);
-        extra = NSB;
+        if constexpr (HASC) {
+            /* the stores and the loads of old c lie before all four slabs, as before a workgroup's first tile */
+            issue_two(0);
+            issue_two(2);
+            extra = 0;
+        }
+        else {
+            issue_two(2);
+            extra = NSB;
+        }
     }
 #ifdef NTSAMD_PROBE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -567,19 +609,25 @@ static int launch_f16_persistent(const GemmParams & p0, hipStream_t stream)
 #else
     const bool hasBias = p.bias != NULL;
 #endif
+    const bool hasC = p.beta != 0.f;
+    auto go = [&](auto BMC) {
+        constexpr int bmc = decltype(BMC)::value;
+        if (hasC)       /* (never with a bias as well: that combination has no registers left, the dispatcher keeps it away) */
+            hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false, bmc, true>), dim3(groups), dim3(512), 0, stream, p);
+        else {
+            if (hasBias)
+                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true, bmc, false>), dim3(groups), dim3(512), 0, stream, p);
+            else
+                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false, bmc, false>), dim3(groups), dim3(512), 0, stream, p);
+        }
+    };
     if constexpr (AKC) {
         if (bm == 128) {
-            if (hasBias)
-                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true, 128>), dim3(groups), dim3(512), 0, stream, p);
-            else
-                hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false, 128>), dim3(groups), dim3(512), 0, stream, p);
+            go(IntC<128>());
             return (int)hipGetLastError();
         }
     }
-    if (hasBias)
-        hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, true>), dim3(groups), dim3(512), 0, stream, p);
-    else
-        hipLaunchKernelGGL((gemm_f16_persistent_kernel<AKC, BKC, false>), dim3(groups), dim3(512), 0, stream, p);
+    go(IntC<256>());
     return (int)hipGetLastError();
 }
 

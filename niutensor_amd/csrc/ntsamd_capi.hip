@@ -254,10 +254,11 @@ struct Plan {
      NTSAMD_GROUP_M=n            tile rows that share a sweep over the tile columns (8 if unset)
      NTSAMD_A32_CONVERT=0|1      float a with half b: never / whenever it fits the workspace, round a to half in a pass
                                  of its own before the product
+     NTSAMD_F16_PERSIST_BETA=0   half products that read the old c keep to the one-tile kernels
      NTSAMD_F16_REPITCH=0|1      half operands with rows that are no whole 16-byte pieces: never / whenever they fit the
                                  workspace, copied there with padded rows so that the product takes the 16-byte path */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert, f16Repitch;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert, f16Repitch, f16PersistBeta;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -273,6 +274,7 @@ const Knob g_knobs[] = {
     {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
     {"NTSAMD_STORE_HINT", &Tuning::storeHint}, {"NTSAMD_GROUP_M", &Tuning::groupM},
     {"NTSAMD_A32_CONVERT", &Tuning::a32Convert}, {"NTSAMD_F16_REPITCH", &Tuning::f16Repitch},
+    {"NTSAMD_F16_PERSIST_BETA", &Tuning::f16PersistBeta},
 };
 
 const Tuning & tuning()
@@ -692,7 +694,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
 #endif
     const bool biasFits = bias == NULL || probeBias || (biasMode == NTSAMD_BIAS_COL && aligned16(bias));
     int launchCfg = cfg;
-    if (kind == KIND_F16 && fetch16 == F16_DIRECT && beta == 0.f && biasFits && colSum == NULL && plan.splits == 1 &&
+    if (kind == KIND_F16 && fetch16 == F16_DIRECT && (beta == 0.f || (bias == NULL && tn.f16PersistBeta.load(std::memory_order_relaxed) != 0)) && biasFits && colSum == NULL && plan.splits == 1 &&
         s.K >= 256 && tn.f16Persist.load(std::memory_order_relaxed) != 0) {
         const int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
         const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;

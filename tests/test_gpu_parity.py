@@ -965,6 +965,39 @@ def test_half_walk_over_tiles_of_128_rows(gpu, oracle, tb):
         nt.tuning_set("NTSAMD_F16_PERSIST", None)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_half_walk_that_adds_to_the_old_result(gpu, oracle, ta, tb):
+    """beta != 0 on more tiles than CUs (the gradient products of source/network/XBackwardMath.cpp all add to what the
+    gradient tensor holds): the walking kernel reads the old c on its way out and adds it in fp32 before the one
+    rounding. Tiles of 256 rows in every layout and of 128 rows where a is stored row by row; every element against
+    double precision, and to the last half bit against the one-tile kernels."""
+    torch = torch_()
+    try:
+        cases = [(4100, 4360, 264, 2, 1.0), (4352, 4352, 1000, 2, 0.5)]
+        if ta == X_NOTRANS:
+            cases.append((3900, 2100, 1032, 4, 1.0))
+        for i, (M, N, K, walk, beta) in enumerate(cases):
+            a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 9300 + i, 0, 0.05)))
+            b = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((K, N), tb), 9400 + i, 0, 0.05)))
+            c0 = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal((M, N), 9500 + i, 0, 0.5)))
+            ga, gb = dev_tensor(a, gpu, True), dev_tensor(b, gpu, True)
+            got = {}
+            for knob in (walk, 0):
+                nt.tuning_set("NTSAMD_F16_PERSIST", knob)
+                nt.tuning_set("NTSAMD_TILE_CFG", 2 if knob else None)
+                c = dev_tensor(c0, gpu, True)
+                nt.matrix_mul(ga, ta, gb, tb, c, 0.75, beta)
+                got[knob] = c
+            w, o = got[walk].float(), got[0].float()
+            step = torch.maximum(w.abs(), o.abs()) * 2.0 ** -10 + 2.0 ** -24
+            assert bool(((w - o).abs() <= step).all()), "%dx%dx%d: the walk and the one-tile kernels differ" % (M, N, K)
+            assert float((w != o).float().mean()) < 1e-3
+            assert_fp16(w.cpu().numpy(), 0.75 * whole_f64(a, ta, b, tb) + beta * c0.astype(np.float64), what="%dx%dx%d beta %g" % (M, N, K, beta))
+    finally:
+        nt.tuning_set("NTSAMD_F16_PERSIST", None)
+        nt.tuning_set("NTSAMD_TILE_CFG", None)
+
+
 def test_config5_ragged_vocab_projection(gpu, oracle):
     """fp32 H[4096x512] x W[30011x512]^T accumulated into C[4096x30011] with beta = 1."""
     torch = torch_()
