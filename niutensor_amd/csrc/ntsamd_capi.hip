@@ -702,10 +702,11 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         const bool wide = ldc % 8 == 0 && s.N % 8 == 0 && aligned16(c) && strideC % 8 == 0 &&
                           (!grid || grid->strideC1 % 8 == 0);
         const int knob = tn.f16Persist.load(std::memory_order_relaxed);
-        /* from one tile per CU on: with CUs to spare the part is not held back by its power limit, and the older
-           kernels' longer lead of the loads counts for more than the energy this one saves (measured: 4096^3 112 ->
-           103 us, but 2048 x 4096 x 8192 on 128 CUs 147 -> 177 us with both operands k-contiguous) */
-        if (cfg == CFG_256x256 && wide && cus > 0 && (tiles >= cus || knob == 2)) {
+        /* from three tiles for four CUs on: with more CUs to spare the part is not held back by its power limit, and
+           the older kernels' longer lead of the loads counts for more than the energy this one saves (measured, all
+           four layouts: 192 tiles 28.1 -> 26.4 us at k = 1024 and 52.2 -> 46.7 us at k = 2048, 144 tiles 42.4 -> 43.5 us,
+           128 tiles 140.8 -> 153.7 us at k = 8192) */
+        if (cfg == CFG_256x256 && wide && cus > 0 && (tiles * 4 >= (long long)cus * 3 || knob == 2)) {
             p.persistGrid = cus;
             p.persistRows = 256;
         }
