@@ -9,17 +9,19 @@
  * v_mfma_f32_32x32x16_f16 takes, per lane, eight consecutive k of one row (A) or
  * one column (B): lane l holds row/column l%32 and k = 8*(l/32) .. +7 of the step.
  * Operand staging in LDS, chosen per operand by how it lies in memory:
- *   K-contiguous (a with X_NOTRANS, b with X_TRANS): rows of mn, S[mn][k], pitch
- *       BKT+8 halves. 16-byte global loads and LDS writes along k; a fragment is
- *       one 16-byte LDS read, and the 80-byte pitch spreads the eight lanes of a
- *       128-byte LDS phase over eight bank groups.
+ *   K-contiguous (a with X_NOTRANS, b with X_TRANS): rows of mn, S[mn][k], 64 bytes
+ *       each without padding, the four 16-byte pieces of a row permuted by
+ *       (row >> 2) & 3. 16-byte global loads and LDS writes along k; a fragment is
+ *       one 16-byte LDS read. Neither the writes (sixteen lanes: four rows) nor the
+ *       reads (sixteen lanes: one piece of sixteen rows) meet in a bank.
  *   MN-contiguous (a with X_TRANS, b with X_NOTRANS): rows of k, S[k][mn], pitch
- *       BMN+16 halves. 16-byte global loads and LDS writes along mn; a fragment is
+ *       BMN+32 halves. 16-byte global loads and LDS writes along mn; a fragment is
  *       two ds_read_b64_tr_b16: within 16 lanes the instruction hands lane c the
  *       c-th half of each of the four rows that lanes 0-3, 4-7, 8-11, 12-15 point
  *       at, which is exactly "four consecutive k of column c" when those lane
- *       groups point at four consecutive k rows. The pitch of 32 bytes mod 128
- *       keeps the four rows of one read in different bank groups.
+ *       groups point at four consecutive k rows. Thirty-two lanes take 64 bytes of
+ *       each of four k rows in one cycle of the 64 banks: the pitch of 64 bytes
+ *       mod 256 keeps those apart.
  *
  * Pipeline per slab of BKT values of k, as in the fp32 kernel: all fragments of
  * the current slab sit in registers; a later slab goes global -> registers ->
@@ -111,9 +113,16 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TI = WM / 32, TJ = WN / 32;
     constexpr int KS = BKT / 16;          /* MFMA k steps per slab */
-    constexpr int LDK = BKT + 8;          /* pitch of a K-contiguous operand, halves */
-    constexpr int LDA = BM + 16;          /* pitch of an MN-contiguous a, halves */
-    constexpr int LDB = BN + 16;
+    /* LDS, 64 banks (256 bytes a cycle). K-contiguous operand: rows of 64 bytes, no padding, four to a 256-byte line,
+       the four 16-byte pieces of row r stored at piece ^ ((r >> 2) & 3): the sixteen lanes that write four rows
+       cover a whole line, and so do the sixteen that read one piece of sixteen rows (the 80-byte pitch this replaces
+       made the fourth row of a write wrap into the first: SQ_LDS_BANK_CONFLICT at a third of the LDS cycles).
+       MN-contiguous operand: a transposing read takes 64 bytes from each of four k rows at a time, so the rows
+       stand 64 bytes (mod 256) apart: BM + 32 halves (with + 16 two neighbouring rows shared 32 bytes of banks). */
+    static_assert(BKT == 32, "the permutation of a K-contiguous row is laid out for rows of four 16-byte pieces");
+    constexpr int LDK = BKT;
+    constexpr int LDA = BM + 32;
+    constexpr int LDB = BN + 32;
     constexpr int NA = BM * BKT / 8 / NT;
     constexpr int NB = BN * BKT / 8 / NT;
     constexpr int ASIZE = AKC ? BM * LDK : BKT * LDA;
@@ -168,7 +177,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             int row = g / (BKT / 8);
             aK[s] = (g % (BKT / 8)) * 8;
             aMN[s] = row;
-            aLds[s] = row * LDK + aK[s];
+            aLds[s] = row * LDK + (((aK[s] >> 3) ^ ((row >> 2) & 3)) << 3);
             int r = m0 + row < M - 1 ? row : M - 1 - m0;
             aOff[s] = (r * p.lda + aK[s]) * ASZ;
         }
@@ -188,7 +197,7 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
             int row = g / (BKT / 8);
             bK[s] = (g % (BKT / 8)) * 8;
             bMN[s] = row;
-            bLds[s] = row * LDK + bK[s];
+            bLds[s] = row * LDK + (((bK[s] >> 3) ^ ((row >> 2) & 3)) << 3);
             int r = n0 + row < N - 1 ? row : N - 1 - n0;
             bOff[s] = (r * p.ldb + bK[s]) * 2;
         }
@@ -360,12 +369,12 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
     auto read_frags = [&](auto SET, int buf) {
         constexpr int set = decltype(SET)::value;
         if constexpr (AKC) {
-            const half_t * as = &As[buf][(wm0 + l32) * LDK + 8 * lh];
+            const half_t * as = &As[buf][(wm0 + l32) * LDK];
 #pragma unroll
             for (int kk = 0; kk < KS; kk++)
 #pragma unroll
                 for (int i = 0; i < TI; i++)
-                    fa[set][kk][i] = *reinterpret_cast<const f16x8 *>(as + i * 32 * LDK + kk * 16);
+                    fa[set][kk][i] = *reinterpret_cast<const f16x8 *>(as + i * 32 * LDK + (((2 * kk + lh) ^ ((l32 >> 2) & 3)) << 3));
         }
         else {
             const half_t * as = &As[buf][(8 * lh + trRow) * LDA + wm0 + trCol];
@@ -379,12 +388,12 @@ gemm_f16_kernel(const GemmParams p, const PT tab)
                 }
         }
         if constexpr (BKC) {
-            const half_t * bs = &Bs[buf][(wn0 + l32) * LDK + 8 * lh];
+            const half_t * bs = &Bs[buf][(wn0 + l32) * LDK];
 #pragma unroll
             for (int kk = 0; kk < KS; kk++)
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
-                    fb[set][kk][j] = *reinterpret_cast<const f16x8 *>(bs + j * 32 * LDK + kk * 16);
+                    fb[set][kk][j] = *reinterpret_cast<const f16x8 *>(bs + j * 32 * LDK + (((2 * kk + lh) ^ ((l32 >> 2) & 3)) << 3));
         }
         else {
             const half_t * bs = &Bs[buf][(8 * lh + trRow) * LDB + wn0 + trCol];
