@@ -37,6 +37,7 @@ PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6}     # MI355X dense matrix peaks (dat
 HBM_TBS = 8.0
 SETTLE_S = 0.15                                 # GPU time under load before anything is timed
 BASELINE_CONFIGS = (1, 2, 3, 4, 5)
+LAYOUT_OF_4 = "TN"                              # how configuration 4's operands are stored (--layout changes it)
 
 
 def configs():
@@ -115,10 +116,19 @@ class Workload:
             self.bytes = 2 * 4.0 * 256 * (128 * 64 + 128 * 64 + 128 * 128)
             self.launches = 2
         elif idx == 4:
+            # LAYOUT_OF_4 (--layout, for profiles of the other three layouts of the same product): the first letter
+            # says how a is stored (T: k x m as in the baseline's configuration, N: m x k), the second how b is
+            ta, tb = (T if LAYOUT_OF_4[0] == "T" else NT), (T if LAYOUT_OF_4[1] == "T" else NT)
+            if LAYOUT_OF_4 != "TN":
+                self.cfg = dict(self.cfg, name=self.cfg["name"] + " -- the same product with its operands stored " + LAYOUT_OF_4)
             self.a = g(oracle.normal((1024, 8192), 1, 0, 0.02)).half()
             self.b = g(oracle.normal((1024, 4096), 2, 0, 0.02)).half()
+            if ta == NT:
+                self.a = self.a.t().contiguous()
+            if tb == T:
+                self.b = self.b.t().contiguous()
             self.c = torch.empty((8192, 4096), device=dev, dtype=torch.float16)
-            self.run = lambda: nt.matrix_mul(self.a, T, self.b, NT, self.c, 1.0, 0.0)
+            self.run = lambda: nt.matrix_mul(self.a, ta, self.b, tb, self.c, 1.0, 0.0)
             self.flops = 2.0 * 8192 * 4096 * 1024
             self.bytes = 2.0 * (1024 * 8192 + 1024 * 4096 + 8192 * 4096)
             self.launches = 1
@@ -550,11 +560,15 @@ def main():
     ap.add_argument("--only", action="store_true",
                     help="time --config alone, without the other baseline configurations beside it (for a profiler: their "
                          "kernels share names with those of configurations 6, 7, 12 and 14)")
+    ap.add_argument("--layout", choices=("TN", "TT", "NN", "NT"), default="TN",
+                    help="configuration 4 with its operands stored another way (TN is the baseline's: a as k x m, b as k x n)")
     ap.add_argument("--k-scan", action="store_true",
                     help="run only the scan over k of configuration 3's first product (what a launch costs beside its MFMAs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (scale for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
+    global LAYOUT_OF_4
+    LAYOUT_OF_4 = args.layout
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path has no multi-GPU part (each product is independent); "
                          "run with --gpus 1")
