@@ -19,9 +19,20 @@ settle, and a short warm-up would time the ramp.
 Each JSON line carries
   value/unit       TFLOP/s = 2 M N K batch / time, over the timed steps
   roofline         the same kernel timed with HIP events on its own stream,
-                   against the MI355X dense matrix peak of the data type
-  cpu_baseline     the CPU restatement of the reference's naive path (1 thread,
-                   as the reference runs it) on a bounded sample of the same product
+                   against the MI355X dense matrix peak of the data type;
+                   kernel_us is with ONE set of buffers used again every step
+                   (configurations 1-4 then sit in the 256 MB Infinity Cache),
+                   kernel_us_rotated with enough sets in turn to exceed it
+  check            the buffers the timed steps wrote, compared after the timed
+                   region with a float64 evaluation of sampled rows (and every
+                   element tested for being finite); a miss ends the run with
+                   a non-zero exit code
+  kernels          what the library planned for each launch of a step (kernel
+                   family, tile shape, fetch route, pieces of k)
+  nts_layer_us     the same operator through the nts:: C++ layer (a child
+                   process: tests/cpp/build/nts_tests --bench)
+  cpu_baseline     the reference's CPU path (1 thread, as the reference runs it)
+                   on a bounded sample of the same product
 """
 import argparse
 import ctypes as C
@@ -37,6 +48,9 @@ PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6}     # MI355X dense matrix peaks (dat
 HBM_TBS = 8.0
 SETTLE_S = 0.15                                 # GPU time under load before anything is timed
 BASELINE_CONFIGS = (1, 2, 3, 4, 5)
+ATTENTION_FORMS = (8, 11, 12)                   # configuration 3 as the transformer runs it: one kernel, or the two halves of training
+CACHE_BYTES = 256 << 20                         # Infinity Cache of the part
+ROTATE_BYTES = 320 << 20                        # what the sets of buffers cycled by kernel_us_rotated add up to, at least
 LAYOUT_OF_4 = "TN"                              # how configuration 4's operands are stored (--layout changes it)
 
 
@@ -85,6 +99,7 @@ class Workload:
         import torch
         import niutensor_amd as nt
         self.idx = idx
+        self.dev = dev
         self.cfg = configs()[idx]
         T, NT = nt.X_TRANS, nt.X_NOTRANS
         g = lambda x: torch.from_numpy(x).to(dev)
@@ -227,6 +242,116 @@ class Workload:
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
+    def check(self):
+        """The buffers the timed steps wrote against a float64 evaluation (torch, on the device: neither this
+        library nor the oracle) of sampled rows, at least 64 of them, and every element of every result tested for
+        being finite. Steps that accumulate (beta = 1) are checked on one more step from a fresh start of the same
+        buffers. Returns max_err (norm-wise: max |got - ref| / max |ref|), the limit (1e-5 sqrt(K) in float, 1e-2 in
+        half) and whether both tests passed."""
+        import math
+        import torch
+        idx, dev = self.idx, self.dev
+        gen = torch.Generator(device="cpu")
+        gen.manual_seed(20251 + idx)
+        pick = lambda n, k: torch.randperm(n, generator=gen)[:k].sort().values.to(dev)
+        d = lambda t: t.double()
+        half = self.cfg["dtype"] == "f16"
+        limit = 1e-2 if half else 1e-5 * math.sqrt(self.cfg["K"])
+        pairs, whole, rows = [], [], 0
+
+        def heads(t, n=8):          # [b, l, n * dh] -> [n, b, l, dh]
+            b, l, hd = t.shape
+            return t.reshape(b, l, n, hd // n).permute(2, 0, 1, 3)
+
+        def merged(t):              # [n, b, l, dh] -> [b, l, n * dh]
+            n, b, l, dh = t.shape
+            return t.permute(1, 2, 0, 3).reshape(b, l, n * dh)
+
+        if idx in (1, 2, 10):
+            r = pick(4096, 64)
+            ref = d(self.x[r]) @ d(self.w)
+            if idx != 1:
+                ref = ref + d(self.b)
+            if idx == 10:
+                ref = ref.clamp(min=0)
+            pairs, whole, rows = [(self.c[r], ref)], [self.c], 64
+        elif idx == 3:
+            r = pick(256, 8)
+            sc = d(self.q[r]) @ d(self.k[r]).transpose(1, 2) * 0.125
+            pairs, whole, rows = [(self.s[r], sc), (self.o[r], sc @ d(self.v[r]))], [self.s, self.o], 8 * 128
+            limit = 1e-5 * math.sqrt(128)
+        elif idx == 4:
+            r = pick(8192, 64)
+            a_rows = self.a[:, r].t() if LAYOUT_OF_4[0] == "T" else self.a[r]
+            b_full = self.b.t() if LAYOUT_OF_4[1] == "T" else self.b
+            pairs, whole, rows = [(self.c[r], d(a_rows) @ d(b_full))], [self.c], 64
+        elif idx == 5:
+            r = pick(4096, 64)
+            self.c.uniform_(-1, 1)
+            c0 = d(self.c[r])
+            self.run()
+            pairs, whole, rows = [(self.c[r], c0 + d(self.h[r]) @ d(self.w).t())], [self.c], 64
+        elif idx == 6:
+            r, rk = pick(4096, 64), pick(512, 64)
+            for t in (self.dx, self.dw, self.db):
+                t.zero_()
+            self.run()
+            pairs = [(self.dx[r], d(self.dy[r]) @ d(self.w).t()), (self.dw[rk], d(self.x[:, rk]).t() @ d(self.dy)),
+                     (self.db, d(self.dy).sum(0))]
+            whole, rows, limit = [self.dx, self.dw, self.db], 128, 1e-5 * math.sqrt(4096)
+        elif idx == 7:
+            r = pick(256, 8)
+            self.dq.zero_()
+            self.dk.zero_()
+            self.run()
+            pairs = [(self.dq[r], d(self.ds[r]) @ d(self.k[r]) * 0.125),
+                     (self.dk[r], d(self.ds[r]).transpose(1, 2) @ d(self.q[r]) * 0.125)]
+            whole, rows, limit = [self.dq, self.dk], 8 * 128, 1e-5 * math.sqrt(128)
+        elif idx in (8, 9):
+            r = pick(32, 2)
+            q, k, v = (heads(d(t[r])) for t in (self.q, self.k, self.v))
+            ref = merged(torch.softmax(q @ k.transpose(2, 3) * 0.125, -1) @ v)
+            pairs, whole, rows = [(self.o[r], ref)], [self.o], 2 * 128
+            limit = 1e-2 if half else 1e-5 * math.sqrt(64 + 128)
+        elif idx == 11:
+            r = pick(32, 2)
+            q, k = heads(d(self.q[r])), heads(d(self.k[r]))
+            pairs, whole, rows = [(self.p[:, r], torch.softmax(q @ k.transpose(2, 3) * 0.125, -1))], [self.p], 8 * 2 * 128
+            limit = 1e-5 * math.sqrt(64 + 128)
+        elif idx == 12:
+            r = pick(32, 2)
+            pairs, whole, rows = [(self.o[r], merged(d(self.p[:, r]) @ heads(d(self.v[r]))))], [self.o], 2 * 128
+        elif idx == 13:
+            rk = pick(512, 64)
+            self.dw.zero_()
+            self.run()
+            pairs, whole, rows = [(self.dw[rk], d(self.x[:, rk]).t() @ d(self.dy))], [self.dw], 64
+        elif idx == 14:
+            r = pick(256, 8)
+            pairs, whole, rows = [(self.o[r], d(self.p[r].half()) @ d(self.v[r]))], [self.o], 8 * 128
+        err = max(float((d(got) - ref).abs().max() / ref.abs().max()) for got, ref in pairs)
+        finite = all(bool(torch.isfinite(t).all()) for t in whole)
+        ok = finite and err <= limit
+        return {"max_err": float("%.3e" % err), "limit": float("%.3e" % limit), "sampled_rows": rows,
+                "all_finite": finite, "ok": ok,
+                "against": "float64 evaluation of the sampled rows (torch on the device), norm-wise: max|got - ref| / max|ref|"}
+
+    def tensor_sets(self):
+        """For kernel_us_rotated: enough copies of this configuration's device buffers that, used in turn, the sets
+        add up to ROTATE_BYTES, more than the part's Infinity Cache holds (one set if one alone exceeds the cache).
+        Returns the list of sets (name -> tensor) and the bytes of one set."""
+        import torch
+        own = {n: t for n, t in vars(self).items() if isinstance(t, torch.Tensor) and t.is_cuda}
+        one = sum(t.numel() * t.element_size() for t in own.values())
+        if one > CACHE_BYTES:
+            return [own], one
+        n = -(-ROTATE_BYTES // one)
+        return [own] + [{k: t.clone() for k, t in own.items()} for _ in range(n - 1)], one
+
+    def use(self, tensors):
+        for name, t in tensors.items():
+            setattr(self, name, t)
+
 
 class HipEvents:
     """hipEvent timing on the stream the kernels are launched on."""
@@ -266,6 +391,12 @@ def cpu_baseline(idx, budget_s=12.0):
     if use_ref:
         o.uniform, o.normal = gen.uniform, gen.normal
     kind = "reference" if use_ref else "port"
+    if use_ref:
+        why = "the reference's own CPU sources, compiled by oracle/Makefile into oracle/_ref (test infrastructure)"
+    elif idx in (1, 2, 3, 5, 8, 10, 11, 12):
+        why = "oracle/_ref/libnts_ref.so is not in this tree: the C restatement of the reference's CPU path runs instead"
+    else:
+        why = "the reference has no CPU arithmetic for this step (half operands, or a gradient step): the C restatement on fp32 values"
     flags = "-O3" if use_ref else "-O3 -march=native"
     cfg = configs()[idx]
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
@@ -368,7 +499,7 @@ def cpu_baseline(idx, budget_s=12.0):
             dt = time.perf_counter() - t0
         fl = 2.0 * rows * N * K
         sample = "%d of %d result rows, all %d columns, K=%d" % (rows, M, N, K)
-    return {"value": round(fl / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": kind,
+    return {"value": round(fl / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": kind, "kind_why": why,
             "sample": sample + " (%.1f s; %.2f GFLOP/s, %s)" % (dt, fl / dt / 1e9, flags)}
 
 
@@ -447,6 +578,63 @@ def k_scan(dev, ev):
     return out
 
 
+def rotated(wl, dev, ev, stream, reps):
+    """Seconds per step with the configuration's buffers changed from step to step: enough sets, used in turn, that
+    no operand or result is still in the 256 MB Infinity Cache when its turn comes again. Steps of less than 20 us
+    are replayed from a HIP graph that holds one step per set, so that changing the buffers costs the host nothing.
+    Returns (seconds per step, number of sets, bytes of one set)."""
+    import torch
+    sets, one = wl.tensor_sets()
+    own = sets[0]
+    if len(sets) == 1:
+        return None, 1, one
+
+    def cycle():
+        for t in sets:
+            wl.use(t)
+            wl.run()
+    try:
+        for _ in range(3):
+            cycle()
+        torch.cuda.synchronize()
+        rounds = max(2, reps // len(sets))
+        per = min(ev.time(cycle, stream, rounds) for _ in range(3)) / len(sets)
+        if per / wl.launches < 20e-6:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                cycle()
+            for _ in range(5):
+                g.replay()
+            torch.cuda.synchronize()
+            st = torch.cuda.current_stream(dev).cuda_stream
+            per = min(ev.time(g.replay, st, 20) for _ in range(3)) / len(sets)
+            del g
+    finally:
+        wl.use(own)
+    return per, len(sets), one
+
+
+def nts_layer_times():
+    """The operators of configurations 2 to 5 through the nts:: C++ layer: tests/cpp/build/nts_tests --bench as a child
+    process (run before this process touches the GPU). Returns {config: line} or a reason why not."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "cpp", "build", "nts_tests")
+    if not os.path.exists(exe):
+        return "tests/cpp/build/nts_tests has not been built"
+    try:
+        p = subprocess.run([exe, "--bench"], capture_output=True, text=True, timeout=180)
+    except subprocess.TimeoutExpired:
+        return "nts_tests --bench did not finish in 180 s"
+    if p.returncode != 0:
+        return "nts_tests --bench ended with code %d: %s" % (p.returncode, (p.stdout + p.stderr)[-300:])
+    out = {}
+    for line in p.stdout.splitlines():
+        if line.startswith("{"):
+            rec = json.loads(line)
+            out[rec["config"]] = rec
+    return out
+
+
 def settle(wl, ev, stream):
     """Runs the workload until SETTLE_S seconds of GPU time have passed; returns the launches it took."""
     done, spent = 0, 0.0
@@ -458,8 +646,9 @@ def settle(wl, ev, stream):
     return done
 
 
-def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0):
+def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0, rotate=True):
     import torch
+    import niutensor_amd as nt
     wl = Workload(idx, dev, oracle)
     cfg = wl.cfg
     ev = HipEvents()
@@ -473,10 +662,17 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0):
     kt = ev.time(wl.run, stream, steps)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
+    # what those steps left in the result buffers, against float64 on sampled rows
+    checked = wl.check()
+    torch.cuda.synchronize()
+    nt.record_plans(True)
+    wl.run()
+    kernels = nt.record_plans(False)
     # shortest of five more groups of launches, reported beside the average (clock and power state move it by a few %)
     reps = max(10, min(200, steps))
     kt_best = min(ev.time(wl.run, stream, reps) for _ in range(5))
     kt_graph = graph_replayed(wl, dev, ev) if kt / wl.launches < 20e-6 else None
+    kt_rot, rot_sets, set_bytes = rotated(wl, dev, ev, stream, reps) if rotate else (None, 0, 0)
     other = None
     if hasattr(wl, "other"):
         # the same result by the steps this configuration replaces, timed the same way (and replayed from a graph,
@@ -509,6 +705,18 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0):
         # launches this short are issued by the host about as fast as the GPU runs them: the same launches
         # replayed from a HIP graph, for what the kernel itself takes (not used for value, achieved or frac)
         roof["kernel_us_graph_replay"] = round(kt_graph / wl.launches * 1e6, 2)
+    if rotate:
+        if kt_rot is None:
+            roof["kernel_us_rotated"] = roof["kernel_us"]
+            resident = "one set of buffers is %.0f MB, more than the %d MB Infinity Cache holds: every step reads HBM" % (
+                set_bytes / 1e6, CACHE_BYTES >> 20)
+        else:
+            roof["kernel_us_rotated"] = round(kt_rot / wl.launches * 1e6, 2)
+            resident = ("one set of buffers (%.0f MB) used again every step: resident in the %d MB Infinity Cache; "
+                        "kernel_us_rotated cycles %d sets (%.0f MB)" % (set_bytes / 1e6, CACHE_BYTES >> 20, rot_sets,
+                                                                       rot_sets * set_bytes / 1e6))
+    else:
+        resident = "one set of buffers used again every step (in the Infinity Cache where it fits its 256 MB)"
     out = {
         "metric": "TFLOP/s & % of dense matrix peak for MatrixMul/Batched (fp32, fp16), 1 GPU",
         "value": round(wl.flops / wall / 1e12, 3),
@@ -523,11 +731,14 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0):
         "dtype": cfg["dtype"],
         "data": "synthetic",
         "config": {"workload": cfg["name"], "M": cfg["M"], "N": cfg["N"], "K": cfg["K"], "batch": cfg["batch"],
-                   "launches_per_step": wl.launches, "inputs": "resident in HBM", "flops_per_step": wl.flops,
+                   "launches_per_step": wl.launches, "inputs": "device buffers, filled before the timed region; " + resident,
+                   "flops_per_step": wl.flops,
                    "algorithmic_bytes_per_step": wl.bytes,
                    "settle": "%d untimed steps (%.2f s of GPU time) before the %d warm-up steps" % (settled, SETTLE_S, warmup)},
         "pct_of_peak": round(100.0 * wl.flops / wall / 1e12 / peak, 2),
         "roofline": roof,
+        "check": checked,
+        "kernels": kernels,
     }
     if other is not None:
         out["replaces"] = other
@@ -542,9 +753,15 @@ def brief(line):
             "kernel_us": line["roofline"]["kernel_us"], "launches_per_step": line["config"]["launches_per_step"],
             "value": line["value"], "unit": line["unit"], "pct_of_peak": line["pct_of_peak"],
             "roofline": {k: line["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "hbm_frac",
-                                                          "traffic", "traffic_source")}}
-    if "cpu_baseline" in line:
-        keep["cpu_baseline"] = line["cpu_baseline"]
+                                                          "traffic", "traffic_source")},
+            "max_err": line["check"]["max_err"], "limit": line["check"]["limit"], "check_ok": line["check"]["ok"],
+            "kernels": line["kernels"], "inputs": line["config"]["inputs"]}
+    for k in ("kernel_us_best", "kernel_us_graph_replay", "kernel_us_rotated"):
+        if k in line["roofline"]:
+            keep[k] = line["roofline"][k]
+    for k in ("cpu_baseline", "nts_layer_us", "nts_layer"):
+        if k in line:
+            keep[k] = line[k]
     return keep
 
 
@@ -557,6 +774,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="configuration 1-14 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-rotate", action="store_true",
+                    help="skip kernel_us_rotated (the same steps over enough sets of buffers to exceed the Infinity Cache)")
+    ap.add_argument("--no-nts", action="store_true", help="skip the child process that times the nts:: C++ layer")
     ap.add_argument("--only", action="store_true",
                     help="time --config alone, without the other baseline configurations beside it (for a profiler: their "
                          "kernels share names with those of configurations 6, 7, 12 and 14)")
@@ -572,6 +792,10 @@ def main():
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path has no multi-GPU part (each product is independent); "
                          "run with --gpus 1")
+
+    # the nts:: layer first, in a process of its own, before this one touches the GPU
+    special = args.copy_calibration or args.k_scan
+    nts_layer = None if (args.no_nts or args.only or special) else nts_layer_times()
 
     import torch
     import niutensor_amd as nt
@@ -594,25 +818,41 @@ def main():
         return
     oracle = Oracle()
     with_cpu = not args.no_cpu
+    rotate = not args.no_rotate and not args.only
     lines = {}
     if args.all:
         for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14):
             if idx == args.config:
                 continue
             steps = args.steps if idx != 5 else max(5, args.steps // 10)
-            lines[idx] = bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle, with_cpu)
+            lines[idx] = bench_one(idx, steps, args.warmup if idx != 5 else max(3, args.warmup // 10), dev, oracle, with_cpu,
+                                   rotate=rotate)
             print(json.dumps(lines[idx]), flush=True)
-    head = bench_one(args.config, args.steps, args.warmup, dev, oracle, with_cpu)
+    head = bench_one(args.config, args.steps, args.warmup, dev, oracle, with_cpu, rotate=rotate)
     lines[args.config] = head
     # the other configurations of the baseline, each settled and timed like the headline (at least 50 steps, so that
-    # a short headline run still gives them a steady reading; a tenth for the 1 ms product), CPU leg on a 3 s sample
-    for idx in BASELINE_CONFIGS if not args.only else ():
+    # a short headline run still gives them a steady reading; a tenth for the 1 ms product), CPU leg on a 3 s sample;
+    # then configuration 3 in the forms the transformer really runs it in (one kernel; the two halves of training)
+    for idx in BASELINE_CONFIGS + ATTENTION_FORMS if not args.only else ():
         if idx not in lines:
             steps = max(50, args.steps) if idx != 5 else max(20, args.steps // 10)
-            lines[idx] = bench_one(idx, steps, args.warmup, dev, oracle, with_cpu, cpu_budget_s=3.0)
+            lines[idx] = bench_one(idx, steps, args.warmup, dev, oracle, with_cpu, cpu_budget_s=3.0, rotate=rotate)
+    # the same operators through the nts:: layer (microseconds per launch, a new result tensor per call)
+    if isinstance(nts_layer, dict):
+        for idx, rec in nts_layer.items():
+            if idx in lines:
+                lines[idx]["nts_layer_us"] = rec["us_per_call"]
+                lines[idx]["nts_layer"] = rec
+    elif nts_layer is not None:
+        head["nts_layer_note"] = nts_layer
     if not args.only:
         head["configs"] = [brief(lines[idx]) for idx in BASELINE_CONFIGS]
+        head["attention_forms"] = [brief(lines[idx]) for idx in ATTENTION_FORMS]
     print(json.dumps(head), flush=True)
+    bad = [idx for idx, line in sorted(lines.items()) if not line["check"]["ok"]]
+    if bad:
+        sys.stderr.write("bench.py: the timed buffers of configuration(s) %s do not agree with float64 (see \"check\")\n" % bad)
+        sys.exit(1)
 
 
 if __name__ == "__main__":

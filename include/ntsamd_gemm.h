@@ -43,7 +43,11 @@
  * products with few tiles and a long k, which are cut along k (partial
  * products in fp32, added up in a fixed order by a second kernel, so results
  * are the same bits on every run): allocated at the first such product on that
- * stream, kept until ntsamd_release_workspaces or the end of the process.
+ * stream, kept until ntsamd_release_workspaces or the end of the process. At
+ * most 64 workspaces are alive at a time; a stream that cannot have one (that
+ * limit, or no memory) gets its products in one piece, float and half alike:
+ * slower for those shapes, the same arithmetic as the single piece of any
+ * other product.
  *
  * Threads and streams: every entry point may be called from any host thread.
  * Calls that use a workspace hold its lock from before their first launch
@@ -52,7 +56,10 @@
  * cannot read each other's partial products. Launches on different streams
  * have different workspaces. Kernels recorded into a graph keep the workspace
  * of the stream they were captured on, so graphs captured on one stream and
- * that stream's own launches must not run concurrently. NTSAMD_SPLIT_K=1 in
+ * that stream's own launches must not run concurrently; such a graph holds
+ * the workspace's ADDRESS, so it must be destroyed (or captured again) once
+ * ntsamd_release_workspaces has freed that workspace, and must not be replayed
+ * afterwards. NTSAMD_SPLIT_K=1 in
  * the environment (read once, at the library's first call) keeps every product
  * in one piece and the library from allocating.
  */
@@ -297,7 +304,11 @@ int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS
 /*
  * Frees the workspaces the library allocated on `devID` (every device if devID < 0): one of 32 MiB per stream on
  * which a product was ever cut along k. Waits for the device's work first; the next product that wants a
- * workspace allocates it again. Has no counterpart among the reference's cuBLAS calls (cuBLAS keeps its own
+ * workspace allocates it again, most likely at another address. HIP graphs that recorded products which used a
+ * workspace (products cut along k, a float a rounded once before a long half product, half operands copied with
+ * padded rows) hold the old address: destroy or re-capture them around a release, never replay them after it
+ * (they would read and write freed memory). Do not call this while any stream of the process is being captured:
+ * hipFree is not allowed then. Has no counterpart among the reference's cuBLAS calls (cuBLAS keeps its own
  * workspace inside the handle, released by cublasDestroy, which the reference never calls: XDevice.cpp:100-108).
  */
 int ntsamd_release_workspaces(int devID);
@@ -309,14 +320,19 @@ int ntsamd_release_workspaces(int devID);
  * k on a stream would allocate that stream's workspace. Same arguments, same result, same kernels; the partial
  * products of a k cut into pieces go to a static array in device memory of NTSAMD_STATIC_SCRATCH_BYTES, which
  * is part of the library's code object: every GPU the library runs on holds one copy from the moment the code
- * is loaded there (ntsamd_init(devID) does that, and is the place to do it before a capture begins) until the
- * process ends.
+ * is loaded there until the process ends. ntsamd_init(devID) looks the array's address up and is the place to
+ * do that before a capture begins; the product kernels themselves are separate code objects that the runtime
+ * loads at their first launch, so a product of each kind that will be captured should have run once, eagerly,
+ * before the capture (one warm-up call per data type and transpose pair).
  *   splits = 0           the library chooses, among the ways to cut k whose partial products fit the array
  *                        (one piece, and no scratch at all, for most shapes: see ntsamd_matrix_mul);
- *   splits = 2, 4, 8, 16 k is cut into that many pieces. NTSAMD_ERR_ARGUMENT, with the sizes in the message,
+ *   splits = 2, 4, 8, 16 k is cut into that many pieces (fewer where rounding a piece up to whole slabs of 32
+ *                        makes the last ones empty). NTSAMD_ERR_ARGUMENT, with the sizes in the message,
  *                        if splits x nc x mc x 4 bytes exceed NTSAMD_STATIC_SCRATCH_BYTES, if a piece would
- *                        be shorter than 128 (half) or 64 (float) values of k, or if the operands cannot take
- *                        the 16-byte path (half: 16-byte aligned, rows of whole 16-byte pieces).
+ *                        be shorter than 128 (half) or 64 (float) values of k, if a row of an operand or of
+ *                        c has 2097152 elements or more, or if a measurement knob (NTSAMD_TILE_CFG) holds
+ *                        the product to a tile shape that has no kernel for pieces. Half operands of any
+ *                        even address and row length, and a float a with a half b, can be cut.
  * All calls on one GPU share that GPU's array, on whatever stream: calls that may overlap on one GPU (different
  * streams, or graphs replayed side by side) race on it and must be ordered by the caller. The array keeps the
  * last call's partial products; every call overwrites all it reads, so nothing has to be cleared.

@@ -83,15 +83,31 @@ def load():
     # measurement knobs: exported, but no part of the interface include/ntsamd_gemm.h documents
     L.ntsamd_tuning_set.argtypes = [C.c_char_p, ci]
     L.ntsamd_tuning_set.restype = ci
+    L.ntsamd_last_plan.restype = C.c_char_p
+    L.ntsamd_plan_only.argtypes = [ci]
+    L.ntsamd_plan_only.restype = None
     for name in EXPORTS[2:]:
         getattr(L, name).restype = ci
     _lib = L
     return L
 
 
+_plan_log = None
+
+
+def record_plans(on):
+    """Start (True) or stop (False) keeping what every call through this module was planned as; stopping returns
+    the list. For the benchmark, which prints the kernels of a configuration beside its timings."""
+    global _plan_log
+    log, _plan_log = _plan_log, ([] if on else None)
+    return log
+
+
 def _check(rc):
     if rc != 0:
         raise NtsAmdError("ntsamd error %d: %s" % (rc, load().ntsamd_last_error().decode()))
+    if _plan_log is not None:
+        _plan_log.append(load().ntsamd_last_plan().decode())
 
 
 def _dtype_code(t):
@@ -159,6 +175,18 @@ def tuning_set(name, value):
     value hands the decision back to the library. For tests and measurements only."""
     v = -1 if value is None else int(value)
     _check(load().ntsamd_tuning_set(name.encode(), v))
+
+
+def last_plan():
+    """What the last product or attention call of this thread was planned as: kernel family, tile shape, layout,
+    fetch route, pieces of k, the passes around it. For measurements and tests."""
+    return load().ntsamd_last_plan().decode()
+
+
+def plan_only(on):
+    """While on, calls from this thread stop after planning: no device is looked up, nothing is allocated or
+    launched, no pointer is followed; last_plan() then tells what would have run. For tests of the dispatcher."""
+    load().ntsamd_plan_only(1 if on else 0)
 
 
 def matrix_mul_batched_strided(a, transA, b, transB, c, count, strideA, strideB, strideC,

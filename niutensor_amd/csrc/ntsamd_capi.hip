@@ -40,6 +40,14 @@ namespace {
 
 thread_local char g_error[512] = "";
 
+/* What the last product issued from this thread was planned as (the kernel family, tile shape, pieces of k, how
+   the operands are fetched, the passes around it): for the benchmark, which records it beside its timings so that
+   a profile's kernel rows can be matched to what ran, and for the tests of the dispatcher. With g_planOnly set
+   (ntsamd_plan_only, tests) a call stops there: nothing is looked up on a device, nothing allocated or launched,
+   no pointer followed. */
+thread_local char g_plan[512] = "";
+thread_local bool g_planOnly = false;
+
 int fail(int code, const char * fmt, ...)
 {
     va_list ap;
@@ -83,8 +91,10 @@ struct DeviceScope {
     int backup;
     bool switched;
     int status;
-    explicit DeviceScope(int devID) : backup(-1), switched(false), status(NTSAMD_OK)
+    explicit DeviceScope(int devID, bool planOnly = false) : backup(-1), switched(false), status(NTSAMD_OK)
     {
+        if (planOnly)
+            return;
         if (hipGetDevice(&backup) != hipSuccess)
             backup = -1;
         if (backup != devID) {
@@ -356,6 +366,12 @@ struct WorkHold {
     {
         if (mem != NULL)
             return;
+        if (g_planOnly) {
+            /* planning only: as if the workspace were there (never dereferenced) */
+            mem = reinterpret_cast<float *>(static_cast<uintptr_t>(256));
+            bytes = SPLIT_WORK_BYTES;
+            return;
+        }
         SplitWork * w;
         {
             std::lock_guard<std::mutex> lock(g_splitMutex);
@@ -367,7 +383,12 @@ struct WorkHold {
             w = slot;
         }
         w->inUse.lock();
-        if (w->mem == NULL && g_splitAlive.load() < SPLIT_STREAMS_MAX) {
+        /* a place among the SPLIT_STREAMS_MAX is taken before the allocation and given back if that fails, so that two
+           threads cannot both pass the test on the last one */
+        const bool place = w->mem == NULL && g_splitAlive.fetch_add(1) < SPLIT_STREAMS_MAX;
+        if (w->mem == NULL && !place)
+            g_splitAlive.fetch_sub(1);
+        if (place) {
             /* the stream may be recording a graph: allocating is allowed then only in the relaxed mode, which is
                how allocators that serve captures do it; the allocation itself is no part of the graph */
             hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
@@ -376,12 +397,12 @@ struct WorkHold {
             const hipError_t err = hipMalloc(&got, SPLIT_WORK_BYTES);
             if (exchanged)
                 (void)hipThreadExchangeStreamCaptureMode(&mode);
-            if (err == hipSuccess && got != NULL) {
+            if (err == hipSuccess && got != NULL)
                 w->mem = static_cast<float *>(got);
-                g_splitAlive.fetch_add(1);
-            }
-            else
+            else {
                 (void)hipGetLastError();
+                g_splitAlive.fetch_sub(1);
+            }
         }
         if (w->mem == NULL) {
             w->inUse.unlock();
@@ -394,6 +415,11 @@ struct WorkHold {
     /* the static scratch of devID (current); false with the message set if it cannot be found */
     bool take_static(int devID)
     {
+        if (g_planOnly) {
+            mem = reinterpret_cast<float *>(static_cast<uintptr_t>(256));
+            bytes = STATIC_SCRATCH_BYTES;
+            return true;
+        }
         float * ptr = static_scratch(devID);
         if (ptr == NULL)
             return false;
@@ -488,12 +514,23 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     if (count == 0 || s.M == 0 || s.N == 0)
         return NTSAMD_OK;
 
-    int st = check_device(devID);
-    if (st != NTSAMD_OK)
-        return st;
-    DeviceScope scope(devID);
+    const bool planOnly = g_planOnly;
+    g_plan[0] = 0;
+    if (!planOnly) {
+        int st = check_device(devID);
+        if (st != NTSAMD_OK)
+            return st;
+    }
+    else if (devID < 0 || devID >= MAX_DEVICES)
+        return fail(NTSAMD_ERR_DEVICE, "invalid device id %d", devID);
+    DeviceScope scope(devID, planOnly);
     if (scope.status != NTSAMD_OK)
         return scope.status;
+    char pre[160] = "";                 /* the passes that run before the product kernel, for the plan's text */
+    auto note = [&pre](const char * what) {
+        const size_t n = strlen(pre);
+        snprintf(pre + n, sizeof(pre) - n, "%s%s", n ? "+" : "", what);
+    };
 
     /* the kernels number their workgroups with 32-bit integers: the finest tiling of the largest batch,
        with k cut into the most pieces, must fit */
@@ -518,9 +555,10 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         if (strideA >= 0 && span > 0 && (size_t)span * 2 <= SPLIT_WORK_BYTES && (forced || slower > pass)) {
             work.take_stream(devID, hs);
             if (work.mem != NULL) {
-                const int rc = launch_convert(0, a, work.mem, span, hs);
+                const int rc = planOnly ? 0 : launch_convert(0, a, work.mem, span, hs);
                 if (rc != 0)
                     return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+                note("convert_kernel(a to half)");
                 a = work.mem;
                 kind = kind == KIND_A32_F16 ? KIND_F16 : KIND_F16_F32OUT;
                 aInWork = true;
@@ -579,6 +617,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     bool vec = lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21) && biasMode != NTSAMD_BIAS_ROW;
     p.mOper = colsA;
     p.nOper = colsB;
+    /* b as the caller stored it: what a column-sum pass of its own reads, whatever copy the product is given */
+    const void * const bStored = b;
     if ((kind == KIND_F16 || kind == KIND_F16_F32OUT) && vec && !ptrs && !grid && !noAlloc && !aInWork &&
         tn.f16Repitch.load(std::memory_order_relaxed) != 0) {
         /* A half operand whose rows are no whole 16-byte pieces (a 30011-word vocabulary) keeps the product off the
@@ -604,7 +644,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                 _Float16 * at = reinterpret_cast<_Float16 *>(work.mem);
                 int rc = 0;
                 if (!okA) {
-                    rc = launch_repitch_f16(a, lda, at, padA, itemsA * rowsA, colsA, hs);
+                    rc = planOnly ? 0 : launch_repitch_f16(a, lda, at, padA, itemsA * rowsA, colsA, hs);
+                    note("repitch_f16_kernel(a)");
                     p.a = a = at;
                     p.lda = lda = padA;
                     p.strideA = strideA = strideA == 0 ? 0 : (long long)rowsA * padA;
@@ -612,7 +653,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                 }
                 if (!okB && rc == 0) {
                     _Float16 * bt = at + elemsA;
-                    rc = launch_repitch_f16(b, ldb, bt, padB, itemsB * rowsB, colsB, hs);
+                    rc = planOnly ? 0 : launch_repitch_f16(b, ldb, bt, padB, itemsB * rowsB, colsB, hs);
+                    note("repitch_f16_kernel(b)");
                     p.b = b = bt;
                     p.ldb = ldb = padB;
                     p.strideB = strideB = strideB == 0 ? 0 : (long long)rowsB * padB;
@@ -659,8 +701,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             return fail(NTSAMD_ERR_ARGUMENT, "k can be cut into 2, 4, 8 or 16 pieces (or 0: the library chooses), not %d",
                         forcedSplits);
         if (!maySplit)
-            return fail(NTSAMD_ERR_ARGUMENT, "this product cannot be cut along k (half operands must be 16-byte "
-                        "aligned with rows of whole 16-byte pieces, rows shorter than 2097152 elements)");
+            return fail(NTSAMD_ERR_ARGUMENT, "this product cannot be cut along k (rows of 2097152 elements or more, or a "
+                        "bias by row, keep it on the kernel that has no such form)");
         if (s.K / forcedSplits < (half ? 128 : 64))
             return fail(NTSAMD_ERR_ARGUMENT, "k = %d is too short for %d pieces (at least %d each)", s.K, forcedSplits,
                         half ? 128 : 64);
@@ -670,6 +712,11 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                         (long long)STATIC_SCRATCH_BYTES);
     }
     Plan plan = choose_plan(s.M, s.N, s.K, count, half, maySplit, beta != 1.f, workBytes, cutExtra, fast32, forcedSplits);
+    /* pieces that were asked for by number and that no tile shape can take (a forced tile shape without such a
+       kernel) are an error, not a product in one piece */
+    if (forcedSplits > 1 && plan.splits != forcedSplits)
+        return fail(NTSAMD_ERR_ARGUMENT, "k cannot be cut into %d pieces under the tile shape in force (NTSAMD_TILE_CFG)",
+                    forcedSplits);
     bool viaWork = false;
     if (plan.splits > 1 && !atomicAsked) {
         if (noAlloc) {
@@ -679,7 +726,10 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         else
             work.take_stream(devID, hs);
         viaWork = work.mem != NULL;
-        if (!viaWork && !atomicAble)
+        /* no workspace to be had (no memory, or too many streams hold one): the product runs in one piece, float
+           and half alike, so that a result never depends on the order in which atomic adds arrive unless the
+           NTSAMD_F32_SPLIT_ATOMIC knob asked for exactly that */
+        if (!viaWork)
             plan = choose_plan(s.M, s.N, s.K, count, half, false, beta != 1.f, 0, 0.0, fast32);
     }
     const int cfg = plan.cfg;
@@ -696,7 +746,9 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     int launchCfg = cfg;
     if (kind == KIND_F16 && fetch16 == F16_DIRECT && (beta == 0.f || (bias == NULL && tn.f16PersistBeta.load(std::memory_order_relaxed) != 0)) && biasFits && colSum == NULL && plan.splits == 1 &&
         s.K >= 256 && tn.f16Persist.load(std::memory_order_relaxed) != 0) {
-        const int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
+        int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
+        if (planOnly && cus <= 0)
+            cus = 256;                  /* planning without a device: the part this library is written for */
         const long long tiles = (long long)((s.M + 255) / 256) * ((s.N + 255) / 256) * count;
         const long long tiles128 = (long long)((s.M + 127) / 128) * ((s.N + 255) / 256) * count;
         const bool wide = ldc % 8 == 0 && s.N % 8 == 0 && aligned16(c) && strideC % 8 == 0 &&
@@ -735,7 +787,10 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     }
     if (p.splits > 1 && !viaWork && beta != 1.f) {
         /* float pieces that add to c: c is dense, count matrices of M x N, strideC apart */
-        if (count == 1 || strideC == (long long)s.M * s.N)
+        note("scale_kernel(c)");
+        if (planOnly)
+            rc = 0;
+        else if (count == 1 || strideC == (long long)s.M * s.N)
             rc = launch_scale(false, c, (long long)s.M * s.N * count, beta, hs);
         else
             for (int i = 0; i < count && rc == 0; i++)
@@ -748,20 +803,69 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             /* by-product of the product kernel */
             p.colSum = colSum;
             p.colSumBeta = colSumBeta;
-            if (p.splits > 1)
-                rc = launch_scale(false, colSum, s.N, colSumBeta, hs);
+            if (p.splits > 1) {
+                note("scale_kernel(colSum)");
+                rc = planOnly ? 0 : launch_scale(false, colSum, s.N, colSumBeta, hs);
+            }
         }
         else {
             /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS. It runs before the product
-               on the same stream, so the two can share the workspace. */
-            if (!half && !s.bKContig && !noAlloc)
+               on the same stream, so the two can share the workspace. It reads b as the caller stored it (dense
+               rows), never the re-pitched copy the product may have been given. */
+            if (!half && !s.bKContig && !noAlloc && !repitched)
                 work.take_stream(devID, hs);
-            rc = s.bKContig ? launch_reduce_sum_xz(half, b, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
-                            : launch_reduce_sum_xz(half, b, s.K, s.N, 1, colSum, colSumBeta, hs, work.mem, work.bytes / 4);
+            note(s.bKContig ? "outer_inner_sum_kernel(b)" : "column_sum_kernel(b)");
+            float * const sumWork = repitched ? NULL : work.mem;
+            const size_t sumFloats = repitched ? 0 : work.bytes / 4;
+            if (planOnly)
+                rc = 0;
+            else
+                rc = s.bKContig ? launch_reduce_sum_xz(half, bStored, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
+                                : launch_reduce_sum_xz(half, bStored, s.K, s.N, 1, colSum, colSumBeta, hs, sumWork, sumFloats);
         }
         if (rc != 0)
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
+
+    {
+        /* the plan in words: the kernel's family and what of its template follows from the plan */
+        static const char * const tiles[CFG_COUNT] = {"128x128", "64x64", "256x256", "32x128", "16x128"};
+        const char * family;
+        const char * fetch;
+        int tileCfg = cfg;
+        if (kind == KIND_F32) {
+            family = "gemm_f32_kernel";
+            fetch = vec ? "vec16" : "elementwise";
+            if (!vec || (ptrs && cfg != CFG_128x128) || (p.colSum != NULL && cfg != CFG_128x128))
+                tileCfg = CFG_64x64;
+        }
+        else {
+            tileCfg = launchCfg;
+            const bool staged = kind_a32(kind) || fetch16 != F16_DIRECT || ptrs;
+            fetch = kind_a32(kind) ? (fetch16 == F16_STAGED ? "staged16,a float" : "elementwise,a float")
+                                   : (fetch16 == F16_DIRECT && !ptrs ? "lds-direct" : (fetch16 == F16_STAGED ? "staged16" : "elementwise"));
+            if (staged)
+                family = "gemm_f16_kernel";
+            else if (launchCfg == CFG_256x256 && p.persistGrid > 0 && !kind_out_f32(kind))
+                family = "gemm_f16_persistent_kernel";
+            else
+                family = "gemm_f16_direct_kernel";
+            if (!staged && p.colSum != NULL && !kind_out_f32(kind) && tileCfg != CFG_64x64)
+                tileCfg = CFG_128x128;
+        }
+        snprintf(g_plan, sizeof(g_plan), "%s%s%s tile=%s%s layout=%c%c fetch=%s splits=%d%s%s%s%s%s%s",
+                 pre, pre[0] ? "+" : "", family,
+                 family[9] == 'p' && p.persistRows == 128 ? "128x256" : tiles[tileCfg],
+                 family[9] == 'p' ? ",walk" : "",
+                 s.aKContig ? 'N' : 'T', s.bKContig ? 'T' : 'N', fetch, p.splits,
+                 p.splits > 1 ? (viaWork ? "+split_reduce_kernel" : ",atomic") : "",
+                 p.colSum != NULL ? " colsum=in-kernel" : "",
+                 bias != NULL ? (biasMode == NTSAMD_BIAS_ROW ? " bias=row" : " bias=col") : "",
+                 beta != 0.f ? " beta" : "", act != ACT_NONE ? " act" : "",
+                 ptrs ? " list" : (grid ? " grid" : (count > 1 ? " strided" : "")));
+    }
+    if (planOnly)
+        return NTSAMD_OK;
 
     if (kind == KIND_F32) {
         if (s.aKContig)
@@ -849,6 +953,16 @@ int ntsamd_release_workspaces(int devID)
         g_splitAlive.fetch_sub(1);
     }
     return NTSAMD_OK;
+}
+
+const char * ntsamd_last_plan(void)
+{
+    return g_plan;
+}
+
+void ntsamd_plan_only(int on)
+{
+    g_planOnly = on != 0;
 }
 
 int ntsamd_tuning_set(const char * name, int value)
@@ -1008,6 +1122,7 @@ int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType
     WorkHold work;
     if (dataType == NTSAMD_X_FLOAT && z == 1 && x >= 128)
         work.take_stream(devID, static_cast<hipStream_t>(stream));
+    snprintf(g_plan, sizeof(g_plan), "%s", z > 1 ? "outer_inner_sum_kernel" : "column_sum_kernel");
     int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,
                                   static_cast<hipStream_t>(stream), work.mem, work.bytes / 4);
     if (rc != 0)
@@ -1046,6 +1161,7 @@ int ntsamd_convert_data_type(int devID, void * stream, const void * s, int typeS
     DeviceScope scope(devID);
     if (scope.status != NTSAMD_OK)
         return scope.status;
+    snprintf(g_plan, sizeof(g_plan), "convert_kernel");
     int rc = launch_convert(kind, s, t, size, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -1088,10 +1204,13 @@ int ntsamd_attention(int devID, void * stream,
     for (int t = 1; t <= 2; t++)
         if (((long long)lk + 256) * strides[3 * t + 2] * 4 > 0x7fffffffLL)
             return fail(NTSAMD_ERR_ARGUMENT, "tensor too large: the keys of one head span more than 2 GiB");
-    int st = check_device(devID);
-    if (st != NTSAMD_OK)
-        return st;
-    DeviceScope scope(devID);
+    const bool planOnly = g_planOnly;
+    if (!planOnly) {
+        int st = check_device(devID);
+        if (st != NTSAMD_OK)
+            return st;
+    }
+    DeviceScope scope(devID, planOnly);
     if (scope.status != NTSAMD_OK)
         return scope.status;
     AttnParams p;
@@ -1117,7 +1236,12 @@ int ntsamd_attention(int devID, void * stream,
     const bool halfType = dataType == NTSAMD_X_FLOAT16;
     const size_t rowsLds = attention_rows_lds(p, halfType);
     int rc;
-    if (rowsLds > 0 && rowsLds <= 60 * 1024 && tuning().attnRows.load(std::memory_order_relaxed) != 0)
+    const bool fewRows = rowsLds > 0 && rowsLds <= 60 * 1024 && tuning().attnRows.load(std::memory_order_relaxed) != 0;
+    snprintf(g_plan, sizeof(g_plan), "%s%s", fewRows ? "attention_rows_kernel" : (halfType ? "attention_f16_kernel" : "attention_f32_kernel"),
+             mask ? " mask" : "");
+    if (planOnly)
+        return NTSAMD_OK;
+    if (fewRows)
         rc = launch_attention_rows(p, halfType, static_cast<hipStream_t>(stream));
     else
         rc = halfType ? launch_attention_f16(p, static_cast<hipStream_t>(stream))
@@ -1155,10 +1279,13 @@ int ntsamd_attention_probs(int devID, void * stream,
         return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
     if (((long long)lk + 256) * strides[5] * 4 > 0x7fffffffLL)
         return fail(NTSAMD_ERR_ARGUMENT, "tensor too large: the keys of one head span more than 2 GiB");
-    int st = check_device(devID);
-    if (st != NTSAMD_OK)
-        return st;
-    DeviceScope scope(devID);
+    const bool planOnly = g_planOnly;
+    if (!planOnly) {
+        int st = check_device(devID);
+        if (st != NTSAMD_OK)
+            return st;
+    }
+    DeviceScope scope(devID, planOnly);
     if (scope.status != NTSAMD_OK)
         return scope.status;
     AttnParams p;
@@ -1175,6 +1302,9 @@ int ntsamd_attention_probs(int devID, void * stream,
     p.qH = strides[0]; p.qB = strides[1]; p.qL = strides[2];
     p.kH = strides[3]; p.kB = strides[4]; p.kL = strides[5];
     p.scale = scale;
+    snprintf(g_plan, sizeof(g_plan), "attention_probs_f32_kernel%s", mask ? " mask" : "");
+    if (planOnly)
+        return NTSAMD_OK;
     int rc = launch_attention_probs_f32(p, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));

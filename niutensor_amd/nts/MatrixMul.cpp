@@ -13,6 +13,7 @@
  */
 #include "MatrixMul.h"
 #include "MatrixMul2D.h"
+#include "MatrixMulBatched.h"
 #include "XTensorBLAS.h"
 
 namespace nts {
@@ -103,8 +104,16 @@ void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
         else {
             BiasSpec spec = RowOrColumnBias(c, bias, n, c->order - 2);
             spec.act = act;
-            CheckNTErrors(a2->devID >= 0, "Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
-            _AmdMatrixMul2DBias(a2, transposedA, b, transposedB, c2, alpha, beta, &spec);
+            if (a2->devID >= 0 || b->devID >= 0 || c2->devID >= 0)
+                _AmdMatrixMul2DBias(a2, transposedA, b, transposedB, c2, alpha, beta, &spec);
+            else {
+                /* host tensors: the host tree's product, then its broadcast add in place, as MulAndShift does there
+                   (MulAndShift.cpp:69, :88); both through the functions the tree handed in */
+                CheckNTErrors(GetHostSumDim() != NULL && n != SCALAR_BIAS && act == 0,
+                              "Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+                _MatrixMul2D(a2, transposedA, b, transposedB, c2, alpha, beta);
+                GetHostSumDim()(c, bias, c, n, (DTYPE)1.0);
+            }
         }
         a2->data = NULL;
         c2->data = NULL;
@@ -137,10 +146,15 @@ void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
 
     CheckNTErrors(!a->isSparse && !b->isSparse, "Sparse matrices are outside this library.");
 
-    if (!(a->devID >= 0 && b->devID >= 0 && c->devID >= 0)) {
-        ShowNTErrors("Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+    /* the GPU takes the list only if all three tensors are on one (MatrixMul.cpp:156-175); anything else is
+       the host's loop over the items (:180-185) */
+    const bool onGpu = a->devID >= 0 && b->devID >= 0 && c->devID >= 0;
+    if (onGpu) {
+        CheckNTErrors((a->devID == b->devID && a->devID == c->devID), "The code must be run on the same GPU!");
     }
-    CheckNTErrors((a->devID == b->devID && a->devID == c->devID), "The code must be run on the same GPU!");
+    else {
+        CheckNTErrors(bias == NULL, "Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+    }
 
     int aDimSize[2] = {-da.rows, da.cols};
     int bDimSize[2] = {-db.rows, db.cols};
@@ -201,7 +215,10 @@ void _MatrixMulBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTen
         }
     }
 
-    _AmdMatrixMULList(a->devID, aList, transposedA, bList, transposedB, cList, aList->count, alpha, beta);
+    if (onGpu)
+        _AmdMatrixMULList(a->devID, aList, transposedA, bList, transposedB, cList, aList->count, alpha, beta);
+    else
+        _MatrixMulBatchedCPU(aList, transposedA, bList, transposedB, cList, alpha, beta);
 
     for (int i = 0; i < aList->count; i++) {
         XTensor * t[3] = {aList->GetItem(i), bList->GetItem(i), cList->GetItem(i)};

@@ -4,17 +4,26 @@
  * rule, "any tensor on a GPU selects the GPU path") and MatrixMul2D.cu:123-164
  * (same-GPU rule, accepted data types). Two things differ on purpose: c is not
  * zeroed before a beta == 0 product, because the kernels do not read c then;
- * and host tensors are refused, because the CPU path is not part of this library.
+ * and host tensors go to the function the host tree handed in with SetHostMatrixMul2D
+ * (its own _MatrixMul2DParallel), because this library holds no CPU arithmetic: without
+ * such a function they are refused.
  */
 #include "MatrixMul2D.h"
 #include "XTensorBLAS.h"
 
 namespace nts {
 
+static HostMatrixMul2DFn hostMatrixMul2D = NULL;
+static HostSumDimFn hostSumDim = NULL;
+
+void SetHostMatrixMul2D(HostMatrixMul2DFn fn) { hostMatrixMul2D = fn; }
+void SetHostSumDim(HostSumDimFn fn) { hostSumDim = fn; }
+HostMatrixMul2DFn GetHostMatrixMul2D() { return hostMatrixMul2D; }
+HostSumDimFn GetHostSumDim() { return hostSumDim; }
+
 void _MatrixMul2D(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
                   XTensor * c, DTYPE alpha, DTYPE beta, XPRunner * parallelRunner)
 {
-    (void)parallelRunner;
     CheckNTErrors((a && b && c), "Empty input tensors!");
     CheckNTErrors((a->dataType == b->dataType), "Input tensors should have the same data type!");
     CheckNTErrors((a->order == 2 && b->order == 2 && c->order == 2), "Input tensors must have a order = 2!");
@@ -34,7 +43,16 @@ void _MatrixMul2D(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTenso
         return;
     }
 
-    ShowNTErrors("Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+    /* none of the three on a GPU: the host tree's dense float product (MatrixMul2D.cpp:77-94) */
+    CheckNTErrors((!a->isSparse && !b->isSparse && !c->isSparse), "Sparse matrices are outside this library.");
+    if (hostMatrixMul2D == NULL) {
+        ShowNTErrors("Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+    }
+    if (a->dataType == DEFAULT_DTYPE && b->dataType == DEFAULT_DTYPE && c->dataType == DEFAULT_DTYPE)
+        hostMatrixMul2D(a, transposedA, b, transposedB, c, alpha, beta, parallelRunner);
+    else {
+        ShowNTErrors("TODO!");
+    }
 }
 
 void _AmdMatrixMul2DBias(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,

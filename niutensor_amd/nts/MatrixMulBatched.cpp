@@ -6,6 +6,7 @@
  * before a beta == 0 product (:121-122 does that): the kernels do not read it.
  */
 #include "MatrixMulBatched.h"
+#include "MatrixMul2D.h"
 #include "XTensorBLAS.h"
 
 namespace nts {
@@ -22,8 +23,61 @@ void _MatrixMulBatched(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const X
 
     if (a->devID >= 0 || b->devID >= 0 || c->devID >= 0)
         _MatrixMulBatchedGPU(a, transposedA, b, transposedB, c, alpha, beta);
-    else {
-        ShowNTErrors("Host tensors are multiplied by NiuTensor's own CPU path, which this library does not replace!");
+    else
+        _MatrixMulBatchedCPU(a, transposedA, b, transposedB, c, alpha, beta);
+}
+
+void _MatrixMulBatchedCPU(const XTensor * a, MATRIX_TRANS_TYPE transposedA, const XTensor * b, MATRIX_TRANS_TYPE transposedB,
+                          XTensor * c, DTYPE alpha, DTYPE beta)
+{
+    CheckNTErrors((a && b && c), "Empty input tensors!");
+    CheckNTErrors((a->dataType == b->dataType && a->dataType == c->dataType),
+                  "Input tensors should have the same data type!");
+    CheckNTErrors((a->order >= 2 && b->order >= 2 && c->order >= 2), "Input tensors must have a order >= 2!");
+    CheckNTErrors((a->order == b->order && a->order == c->order), "Input tensor and output tensor must have same order!");
+
+    const int order = a->order;
+    const XTensor * t[3] = {a, b, c};
+    int rows[3], cols[3];
+    for (int k = 0; k < 3; k++) {
+        rows[k] = t[k]->dimSize[order - 2];
+        cols[k] = t[k]->dimSize[order - 1];
+    }
+    const int an = transposedA == X_TRANS ? cols[0] : rows[0], am = transposedA == X_TRANS ? rows[0] : cols[0];
+    const int bn = transposedB == X_TRANS ? cols[1] : rows[1], bm = transposedB == X_TRANS ? rows[1] : cols[1];
+    CheckNTErrors((am == bn && an == rows[2] && bm == cols[2]), "Unmatched tensors in multiplication!");
+
+    int blockNum = 1;
+    for (int i = 0; i < order - 2; i++) {
+        CheckNTErrors((a->dimSize[i] == c->dimSize[i]), "Incorrect tensor sizes!");
+        CheckNTErrors((b->dimSize[i] == c->dimSize[i]), "Incorrect tensor sizes!");
+        blockNum *= a->dimSize[i];
+    }
+
+    /* one matrix-shaped view per operand (a negative size: the shape and no storage), moved from block to block */
+    XTensor * view[3];
+    for (int k = 0; k < 3; k++)
+        view[k] = NewTensor2DV2(-rows[k], cols[k], t[k]->dataType, t[k]->devID, t[k]->mem);
+    for (int i = 0; i < blockNum; i++) {
+        for (int k = 0; k < 3; k++)
+            view[k]->data = (char *)t[k]->data + (size_t)i * rows[k] * cols[k] * t[k]->unitSize;
+        _MatrixMul2D(view[0], transposedA, view[1], transposedB, view[2], alpha, beta);
+    }
+    for (int k = 0; k < 3; k++) {
+        view[k]->data = NULL;
+        delete view[k];
+    }
+}
+
+void _MatrixMulBatchedCPU(const TensorList * a, MATRIX_TRANS_TYPE transposedA, const TensorList * b, MATRIX_TRANS_TYPE transposedB,
+                          TensorList * c, DTYPE alpha, DTYPE beta)
+{
+    CheckNTErrors((a && b && c), "Empty input lists!");
+    CheckNTErrors((a->count == b->count && a->count == c->count), "Input lists must be of the same size!");
+    for (int i = 0; i < a->count; i++) {
+        XTensor * ai = a->GetItem(i), * bi = b->GetItem(i), * ci = c->GetItem(i);
+        CheckNTErrors((ai->order == 2 && bi->order == 2 && ci->order == 2), "2d tensor (i.e., matrix) is required!");
+        _MatrixMul2D(ai, transposedA, bi, transposedB, ci, alpha, beta);
     }
 }
 

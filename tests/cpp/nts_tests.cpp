@@ -9,6 +9,9 @@
  *
  *   nts_tests                run everything on device 0, exit 0 if all passed
  *   nts_tests --alloc-bench  time an allocating call with and without reuse of device blocks
+ *   nts_tests --bench        time the operators of the baseline's configurations 2 to 5 through this layer
+ *                            (MulAndShift, MatrixMulBatched twice, MatrixMul twice): one JSON line each
+ *   nts_tests --host         the dispatch of host tensors to the functions a host tree hands in (no GPU needed)
  *   nts_tests --abort NAME   provoke one fatal error (no GPU needed): the process
  *                            must print the reference's message and abort
  */
@@ -943,6 +946,212 @@ static int AllocBench()
     return 0;
 }
 
+
+/* ---- host tensors: the layer hands them to the host tree's functions --------------- */
+
+/* stand-ins for the host tree's _MatrixMul2DParallel and _SumDim: plain loops of this file (never the oracle
+   library, which the layer must not depend on), enough to show that the right blocks arrive in the right order */
+static int hostProducts = 0, hostSums = 0;
+static void HostProduct(const XTensor * a, MATRIX_TRANS_TYPE ta, const XTensor * b, MATRIX_TRANS_TYPE tb,
+                        XTensor * c, DTYPE alpha, DTYPE beta, XPRunner *)
+{
+    hostProducts++;
+    const int M = c->dimSize[0], N = c->dimSize[1], K = ta == X_TRANS ? a->dimSize[0] : a->dimSize[1];
+    const float * A = (const float *)a->data, * B = (const float *)b->data;
+    float * C = (float *)c->data;
+    for (int i = 0; i < M; i++)
+        for (int j = 0; j < N; j++) {
+            double sum = 0;
+            for (int k = 0; k < K; k++)
+                sum += (double)(ta == X_TRANS ? A[k * M + i] : A[i * K + k]) * (tb == X_TRANS ? B[j * K + k] : B[k * N + j]);
+            C[i * N + j] = (float)(alpha * sum + (beta != 0 ? beta * C[i * N + j] : 0.0));
+        }
+}
+static void HostSumLastDim(const XTensor * a, const XTensor * b, XTensor * c, int n, DTYPE beta)
+{
+    hostSums++;
+    if (n != a->order - 1)
+        return;
+    const int cols = a->dimSize[n];
+    for (int i = 0; i < a->unitNum; i++)
+        ((float *)c->data)[i] = ((const float *)a->data)[i] + ((const float *)b->data)[i % cols] * beta;
+}
+
+static XTensor * NewHost(int order, const int * dims, const float * data)
+{
+    XTensor * t = NewTensorV2(order, dims, X_FLOAT, 1.0F, -1);
+    if (data != NULL)
+        memcpy(t->data, data, sizeof(float) * t->unitNum);
+    return t;
+}
+static bool SameAs(const XTensor * t, const void * answer, int num)
+{
+    return t->devID < 0 && t->unitNum == num && oracle_check_data((const float *)t->data, (const float *)answer, num, 1e-4F) != 0;
+}
+
+/* The reference's known answers again, on host tensors: _MatrixMul2D, the flattened product and the (p, q) list of
+   _MatrixMul, the blocks of _MatrixMulBatched, the allocating wrappers and MulAndShift all reach the two functions
+   the host tree handed in (source/tensor/core/arithmetic/MatrixMul2D.cpp:77-94, MatrixMul.cpp:180-185,
+   MatrixMulBatched.cpp:157-271, MulAndShift.cpp:69-88). */
+static bool TestHostDispatch()
+{
+    SetHostMatrixMul2D(HostProduct);
+    SetHostSumDim(HostSumLastDim);
+    hostProducts = hostSums = 0;
+    bool ok = GetHostMatrixMul2D() == HostProduct && GetHostSumDim() == HostSumLastDim;
+
+    int d23[2] = {2, 3}, d32[2] = {3, 2}, d22[2] = {2, 2};
+    DTYPE a23[2][3] = {{1.0F, 2.0F, 3.0F}, {-4.0F, 5.0F, 6.0F}};
+    DTYPE a32t[3][2] = {{1.0F, -4.0F}, {2.0F, 5.0F}, {3.0F, 6.0F}};
+    DTYPE b32[3][2] = {{0.0F, -1.0F}, {1.0F, 2.0F}, {2.0F, 1.0F}};
+    DTYPE want22[2][2] = {{8.0F, 6.0F}, {17.0F, 20.0F}};
+    XTensor * s1 = NewHost(2, d23, &a23[0][0]), * s1t = NewHost(2, d32, &a32t[0][0]), * s2 = NewHost(2, d32, &b32[0][0]);
+    XTensor * t = NewHost(2, d22, NULL), * t2 = NewHost(2, d22, NULL);
+    _MatrixMul2D(s1, X_NOTRANS, s2, X_NOTRANS, t);
+    _MatrixMul(s1t, X_TRANS, s2, X_NOTRANS, t2);
+    XTensor user = MatrixMul(*s1, X_NOTRANS, *s2, X_NOTRANS);
+    ok = ok && SameAs(t, want22, 4) && SameAs(t2, want22, 4) && SameAs(&user, want22, 4) && hostProducts == 3;
+
+    /* (3,2,3) x (2,3,2): six pairs of blocks, result block (p, q) at p * 2 + q */
+    int d323[3] = {3, 2, 3}, d232[3] = {2, 3, 2}, d3222[4] = {3, 2, 2, 2}, d322[3] = {3, 2, 2}, d222[3] = {2, 2, 2}, d223[3] = {2, 2, 3};
+    DTYPE want3222[3][2][2][2] = {{{{8.0F, 9.0F}, {4.0F, 25.0F}}, {{7.0F, 8.0F}, {20.0F, 26.0F}}},
+                                  {{{1.0F, 32.0F}, {3.0F, 21.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}},
+                                  {{{-9.0F, 19.0F}, {5.0F, -1.0F}}, {{18.0F, 22.0F}, {-2.0F, -2.0F}}}};
+    XTensor * n1 = NewHost(3, d323, &sData323[0][0][0]), * n2 = NewHost(3, d232, &sData232[0][0][0]);
+    XTensor * t4 = NewHost(4, d3222, NULL);
+    hostProducts = 0;
+    _MatrixMul(n1, X_NOTRANS, n2, X_NOTRANS, t4);
+    ok = ok && SameAs(t4, want3222, 24) && hostProducts == 6;
+
+    /* (3,2,3) x (3,2): one product over the flattened rows */
+    DTYPE b32b[3][2] = {{1.0F, 2.0F}, {3.0F, 4.0F}, {5.0F, 6.0F}};
+    DTYPE want322[3][2][2] = {{{7.0F, 8.0F}, {20.0F, 26.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}, {{18.0F, 22.0F}, {-2.0F, -2.0F}}};
+    XTensor * w = NewHost(2, d32, &b32b[0][0]), * t3 = NewHost(3, d322, NULL);
+    hostProducts = 0;
+    _MatrixMul(n1, X_NOTRANS, w, X_NOTRANS, t3);
+    ok = ok && SameAs(t3, want322, 12) && hostProducts == 1;
+
+    /* (2,2,3) x (2,3,2), block i with block i */
+    DTYPE want222[2][2][2] = {{{8.0F, 9.0F}, {4.0F, 25.0F}}, {{27.0F, 34.0F}, {16.0F, 22.0F}}};
+    XTensor * m1 = NewHost(3, d223, &sData323[0][0][0]), * tb = NewHost(3, d222, NULL);
+    hostProducts = 0;
+    _MatrixMulBatched(m1, X_NOTRANS, n2, X_NOTRANS, tb);
+    XTensor userB = MatrixMulBatched(*m1, X_NOTRANS, *n2, X_NOTRANS);
+    ok = ok && SameAs(tb, want222, 8) && SameAs(&userB, want222, 8) && hostProducts == 4;
+
+    /* MulAndShift: the product, then the host tree's broadcast add along the last dimension, in place */
+    int d2[1] = {2};
+    DTYPE bias2[2] = {0.5F, -1.0F};
+    DTYPE wantShift[3][2][2] = {{{7.5F, 7.0F}, {20.5F, 25.0F}}, {{27.5F, 33.0F}, {16.5F, 21.0F}}, {{18.5F, 21.0F}, {-1.5F, -3.0F}}};
+    XTensor * bs = NewHost(1, d2, bias2);
+    hostProducts = 0;
+    XTensor shifted = MulAndShift(*n1, *w, *bs);
+    ok = ok && SameAs(&shifted, wantShift, 12) && hostProducts == 1 && hostSums == 1 && shifted.order == 3;
+
+    SetHostMatrixMul2D(NULL);
+    SetHostSumDim(NULL);
+    ok = ok && GetHostMatrixMul2D() == NULL;
+    delete s1; delete s1t; delete s2; delete t; delete t2; delete n1; delete n2; delete t4; delete w; delete t3;
+    delete m1; delete tb; delete bs;
+    return ok;
+}
+
+/* ---- the operators of the baseline's configurations, timed through this layer ---------------- */
+
+struct Timer {
+    hipEvent_t e0, e1;
+    Timer() { hipEventCreate(&e0); hipEventCreate(&e1); }
+    ~Timer() { hipEventDestroy(e0); hipEventDestroy(e1); }
+    template <class F> double Us(F f, int calls)
+    {
+        hipEventRecord(e0, NULL);
+        for (int i = 0; i < calls; i++)
+            f();
+        hipEventRecord(e1, NULL);
+        hipEventSynchronize(e1);
+        float ms = 0;
+        hipEventElapsedTime(&ms, e0, e1);
+        return (double)ms * 1e3 / calls;
+    }
+    /* runs f until 0.15 s of GPU time have passed (the clocks of the part settle under load), then times `calls`
+       calls five times over and returns the shortest average */
+    template <class F> double Settled(F f, int calls)
+    {
+        double spent = 0;
+        for (int n = 8; spent < 0.15e6; n = n < 256 ? n * 2 : n)
+            spent += Us(f, n) * n;
+        double best = 1e30;
+        for (int r = 0; r < 5; r++)
+            best = fmin(best, Us(f, calls));
+        return best;
+    }
+};
+
+static XTensor * Filled(int order, const int * dims, int seed, float sd, TENSOR_DATA_TYPE type = X_FLOAT, bool uniform = false)
+{
+    std::vector<float> h(Prod(dims, order));
+    if (uniform)
+        oracle_fill_uniform(h.data(), (long)h.size(), seed, -1.0F, 1.0F);
+    else
+        oracle_fill_normal(h.data(), (long)h.size(), seed, 0, sd);
+    return NewGPU(order, dims, h.data(), type);
+}
+
+/* One JSON line per configuration: microseconds per operator call (HIP events on the NULL stream, which is where
+   this layer issues its work, 200 calls after settling), the allocating form (a new result tensor per call, as
+   the reference's callers use it) and the in-place form beside it. */
+static int Bench()
+{
+    Timer tm;
+    {
+        /* configuration 2: MulAndShift(x[32x128x512], w[512x2048], b[2048]) */
+        int dx[3] = {32, 128, 512}, dw[2] = {512, 2048}, db[1] = {2048}, dc[3] = {32, 128, 2048};
+        XTensor * x = Filled(3, dx, 1, 0, X_FLOAT, true), * w = Filled(2, dw, 2, 0.02F), * b = Filled(1, db, 3, 0.02F);
+        XTensor * c = NewGPU(3, dc, NULL);
+        const double alloc = tm.Settled([&] { XTensor r = MulAndShift(*x, *w, *b); }, 200);
+        const double inplace = tm.Settled([&] { _MatrixMulBias(x, X_NOTRANS, w, X_NOTRANS, c, 1.0F, 0, b, 2); }, 200);
+        printf("{\"config\": 2, \"operator\": \"nts::MulAndShift(x, w, b)\", \"launches\": 1, \"us_per_call\": %.2f, \"us_per_call_into_existing_tensor\": %.2f}\n", alloc, inplace);
+        delete x; delete w; delete b; delete c;
+    }
+    {
+        /* configuration 3: BMMul(q, X_NOTRANS, k, X_TRANS, 1/8), then BMMul(s, v) */
+        int dq[3] = {256, 128, 64}, ds[3] = {256, 128, 128};
+        XTensor * q = Filled(3, dq, 1, 1.0F), * k = Filled(3, dq, 2, 1.0F), * v = Filled(3, dq, 3, 1.0F);
+        XTensor * s = NewGPU(3, ds, NULL), * o = NewGPU(3, dq, NULL);
+        const double alloc = tm.Settled([&] {
+            XTensor sc = MatrixMulBatched(*q, X_NOTRANS, *k, X_TRANS, 0.125F);
+            XTensor out = MatrixMulBatched(sc, X_NOTRANS, *v, X_NOTRANS);
+        }, 200);
+        const double inplace = tm.Settled([&] {
+            _MatrixMulBatched(q, X_NOTRANS, k, X_TRANS, s, 0.125F, 0);
+            _MatrixMulBatched(s, X_NOTRANS, v, X_NOTRANS, o, 1.0F, 0);
+        }, 200);
+        printf("{\"config\": 3, \"operator\": \"nts::MatrixMulBatched(q, k^T, 1/8) then nts::MatrixMulBatched(s, v)\", \"launches\": 2, \"us_per_call\": %.2f, \"us_per_call_into_existing_tensor\": %.2f}\n", alloc / 2, inplace / 2);
+        delete q; delete k; delete v; delete s; delete o;
+    }
+    {
+        /* configuration 4: MatrixMul(a[1024x8192], X_TRANS, b[1024x4096], X_NOTRANS), half */
+        int da[2] = {1024, 8192}, db[2] = {1024, 4096}, dc[2] = {8192, 4096};
+        XTensor * a = Filled(2, da, 1, 0.02F, X_FLOAT16), * b = Filled(2, db, 2, 0.02F, X_FLOAT16);
+        XTensor * c = NewGPU(2, dc, NULL, X_FLOAT16);
+        const double alloc = tm.Settled([&] { XTensor r = MatrixMul(*a, X_TRANS, *b, X_NOTRANS); }, 200);
+        const double inplace = tm.Settled([&] { _MatrixMul(a, X_TRANS, b, X_NOTRANS, c, 1.0F, 0); }, 200);
+        printf("{\"config\": 4, \"operator\": \"nts::MatrixMul(a, X_TRANS, b, X_NOTRANS), half\", \"launches\": 1, \"us_per_call\": %.2f, \"us_per_call_into_existing_tensor\": %.2f}\n", alloc, inplace);
+        delete a; delete b; delete c;
+    }
+    {
+        /* configuration 5: MatrixMul(h[4096x512], X_NOTRANS, w[30011x512], X_TRANS, c, 1, beta = 1) */
+        int dh[2] = {4096, 512}, dw[2] = {30011, 512}, dc[2] = {4096, 30011};
+        XTensor * h = Filled(2, dh, 1, 0, X_FLOAT, true), * w = Filled(2, dw, 2, 0.02F);
+        XTensor * c = Filled(2, dc, 3, 0, X_FLOAT, true);
+        const double inplace = tm.Settled([&] { MatrixMul(*h, X_NOTRANS, *w, X_TRANS, *c, 1.0F, 1.0F); }, 50);
+        printf("{\"config\": 5, \"operator\": \"nts::MatrixMul(h, X_NOTRANS, w, X_TRANS, c, 1, 1)\", \"launches\": 1, \"us_per_call\": %.2f, \"us_per_call_into_existing_tensor\": %.2f}\n", inplace, inplace);
+        delete h; delete w; delete c;
+    }
+    fflush(stdout);
+    return 0;
+}
+
 /* ---- fatal errors: same message, same ending as the reference ---------------- */
 
 static int Provoke(const char * name)
@@ -1015,6 +1224,13 @@ int main(int argc, char ** argv)
         return Provoke(argv[2]);
     if (argc == 2 && !strcmp(argv[1], "--alloc-bench"))
         return AllocBench();
+    if (argc == 2 && !strcmp(argv[1], "--bench"))
+        return Bench();
+    if (argc == 2 && !strcmp(argv[1], "--host")) {
+        const bool ok = TestHostDispatch();
+        printf(">> %-36s %s\n", "TestHostDispatch", ok ? "passed" : "FAILED");
+        return ok ? 0 : 1;
+    }
 
     bool all = true;
     RUN(TestMatrixMul1);
@@ -1039,6 +1255,7 @@ int main(int argc, char ** argv)
     RUN(TestMulAndShiftRectify);
     RUN(TestThreads);
     RUN(TestMemoryReuse);
+    RUN(TestHostDispatch);
     printf(all ? "OK! Everything is good!\n" : "Sorry, some problems happened!\n");
     return all ? 0 : 1;
 }
