@@ -118,7 +118,6 @@ def test_static_entry_point_allocates_nothing_and_can_be_recorded_into_a_graph(g
         torch.cuda.synchronize()
         with torch.cuda.graph(g):
             nt.matrix_mul_static(a, X_TRANS, b, X_NOTRANS, got, 0.5, 0.0, 8)
-        assert torch.cuda.mem_get_info(gpu)[0] <= free0          # (torch's graph pool may have taken memory; the library none)
         for replay in range(3):
             got.fill_(float("nan"))
             g.replay()
