@@ -48,7 +48,7 @@ PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6}     # MI355X dense matrix peaks (dat
 HBM_TBS = 8.0
 SETTLE_S = 0.15                                 # GPU time under load before anything is timed
 BASELINE_CONFIGS = (1, 2, 3, 4, 5)
-ATTENTION_FORMS = (8, 11, 12)                   # configuration 3 as the transformer runs it: one kernel, or the two halves of training
+ATTENTION_FORMS = (8, 15, 11, 12)               # configuration 3 as the transformer runs it: one kernel (inference, training), or the two halves of training
 CACHE_BYTES = 256 << 20                         # Infinity Cache of the part
 ROTATE_BYTES = 320 << 20                        # what the sets of buffers cycled by kernel_us_rotated add up to, at least
 LAYOUT_OF_4 = "TN"                              # how configuration 4's operands are stored (--layout changes it)
@@ -86,6 +86,10 @@ def configs():
                       "half), v[256x128x64]) as one batched product that rounds the probabilities where it fetches them; "
                       "the library's conversion pass followed by the all-half product is timed beside it",
                  dtype="f16", M=128, N=64, K=128, batch=256),
+        15: dict(name="cfg15 fp32 attention of the training path in one kernel: probabilities [8x32x128x128] written, multiplied "
+                      "with a dropout mask and written again, context on merged tensors (cfg11, the caller's Multiply and cfg12 "
+                      "in one launch)",
+                 dtype="f32", M=128, N=128, K=64, batch=256),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -224,6 +228,27 @@ class Workload:
             self.flops = 2.0 * 256 * 128 * 128 * 64
             self.bytes = 4.0 * (256 * 128 * 128 + 2 * 32 * 128 * 512)
             self.launches = 1
+        elif idx == 15:
+            self.q = g(oracle.normal((32, 128, 512), 1))
+            self.k = g(oracle.normal((32, 128, 512), 2))
+            self.v = g(oracle.normal((32, 128, 512), 3))
+            self.dm = (torch.rand((8, 32, 128, 128), device=dev) >= 0.1).float() / 0.9
+            self.p = torch.empty((8, 32, 128, 128), device=dev)
+            self.pd = torch.empty((8, 32, 128, 128), device=dev)
+            self.o = torch.empty((32, 128, 512), device=dev)
+            self.run = lambda: nt.attention_train(self.q, self.k, self.v, self.p, self.o, 8, 0.125, drop_mask=self.dm, dropped=self.pd)
+
+            def three_steps():
+                nt.attention_probs(self.q, self.k, self.p, 8, 0.125)
+                torch.mul(self.p, self.dm, out=self.pd)          # stands in for the caller's Multiply
+                nt.matrix_mul_batched_grid(self.pd, NT, 128, (16384, 32 * 16384), self.v, NT, 512, (65536, 64),
+                                           self.o, 512, (65536, 64), 32, 8, 128, 128, 128, 64, 128, 64)
+            self.other = ("ntsamd_attention_probs, an element-wise multiply with the dropout mask (torch.mul), "
+                          "ntsamd_matrix_mul_batched_grid", three_steps)
+            self.flops = 2 * 2.0 * 256 * 128 * 128 * 64
+            # q, k, v read, the context written; the dropout mask read, probabilities and dropped probabilities written
+            self.bytes = 4.0 * (4 * 32 * 128 * 512 + 3 * 256 * 128 * 128)
+            self.launches = 1
         elif idx == 14:
             self.p = torch.softmax(g(oracle.normal((256, 128, 128), 1)), -1)
             self.ph = torch.empty((256, 128, 128), device=dev, dtype=torch.float16)
@@ -321,6 +346,13 @@ class Workload:
         elif idx == 12:
             r = pick(32, 2)
             pairs, whole, rows = [(self.o[r], merged(d(self.p[:, r]) @ heads(d(self.v[r]))))], [self.o], 2 * 128
+        elif idx == 15:
+            r = pick(32, 2)
+            q, k, v = (heads(d(t[r])) for t in (self.q, self.k, self.v))
+            pr = torch.softmax(q @ k.transpose(2, 3) * 0.125, -1)
+            dr = pr * d(self.dm[:, r])
+            pairs = [(self.p[:, r], pr), (self.pd[:, r], dr), (self.o[r], merged(dr @ v))]
+            whole, rows, limit = [self.p, self.pd, self.o], 8 * 2 * 128, 1e-5 * math.sqrt(64 + 128)
         elif idx == 13:
             rk = pick(512, 64)
             self.dw.zero_()
@@ -386,14 +418,14 @@ def cpu_baseline(idx, budget_s=12.0):
     # the forward configurations in float run the REAL reference (its CPU sources compiled by oracle/Makefile into
     # oracle/_ref, which travels with the tree) when that library is there; the others (half: the reference has no
     # CPU half arithmetic; the gradient steps) and a tree without it run the restatement
-    use_ref = idx in (1, 2, 3, 5, 8, 10, 11, 12) and Reference.available()
+    use_ref = idx in (1, 2, 3, 5, 8, 10, 11, 12, 15) and Reference.available()
     o = Reference() if use_ref else gen
     if use_ref:
         o.uniform, o.normal = gen.uniform, gen.normal
     kind = "reference" if use_ref else "port"
     if use_ref:
         why = "the reference's own CPU sources, compiled by oracle/Makefile into oracle/_ref (test infrastructure)"
-    elif idx in (1, 2, 3, 5, 8, 10, 11, 12):
+    elif idx in (1, 2, 3, 5, 8, 10, 11, 12, 15):
         why = "oracle/_ref/libnts_ref.so is not in this tree: the C restatement of the reference's CPU path runs instead"
     else:
         why = "the reference has no CPU arithmetic for this step (half operands, or a gradient step): the C restatement on fp32 values"
@@ -402,7 +434,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 13: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9, 14: 6e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 13: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9, 14: 6e9, 15: 3e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -442,6 +474,19 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 8 * 2.0 * 128 * 128 * 64
         sample = "%d of 32 sentences, 8 heads each: split of v, batched product, merge" % nb
+    elif idx == 15:
+        nb = max(1, min(32, int(budget_s * rate / (8 * 4.0 * 128 * 128 * 64))))
+        q, k, v = o.normal((nb, 128, 512), 1), o.normal((nb, 128, 512), 2), o.normal((nb, 128, 512), 3)
+        dm = np.where(o.uniform((8, nb, 128, 128), 4, 0.0, 1.0) < 0.1, 0.0, 1.0 / 0.9).astype(np.float32)
+        t0 = time.perf_counter()
+        # the reference's chain: probabilities, Dropout as its element-wise product with the mask, Split of v, BMMul, Merge
+        dr = o.attention_probs(q, k, 8, 0.125) * dm
+        vs = np.ascontiguousarray(v.reshape(nb, 128, 8, 64).transpose(2, 0, 1, 3))
+        c = o.matmul_batched(dr, X_NOTRANS, vs, X_NOTRANS)
+        np.ascontiguousarray(c.transpose(1, 2, 0, 3)).reshape(nb, 128, 512)
+        dt = time.perf_counter() - t0
+        fl = nb * 8 * 4.0 * 128 * 128 * 64
+        sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax, dropout mask, product, merge" % nb
     elif idx == 14:
         nb = max(1, min(256, int(budget_s * rate / (2.0 * 128 * 128 * 64))))
         p = o.uniform((nb, 128, 128), 1, 0.0, 1.0)
@@ -771,7 +816,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-14 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-15 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values, 15 the attention of the training path in one kernel)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-rotate", action="store_true",
@@ -821,7 +866,7 @@ def main():
     rotate = not args.no_rotate and not args.only
     lines = {}
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
             if idx == args.config:
                 continue
             steps = args.steps if idx != 5 else max(5, args.steps // 10)

@@ -288,6 +288,27 @@ int ntsamd_attention_probs(int devID, void * stream,
                            const long long * strides, float scale);
 
 /*
+ * The attention of the reference's TRAINING path in one launch: the operator chain of Attention::MakeAttention with
+ * isTraining set (source/sample/transformer/submodel/Attention.cpp:194-242): Split x3, Scale, BMMul(q, k^T), Sum with
+ * the mask, Softmax, Dropout, BMMul with v, Merge. Dropout in the reference is a mask tensor of the probabilities'
+ * shape, filled by the caller's random number generator with 0 and 1 / (1 - p), and an element-wise Multiply
+ * (source/tensor/function/Dropout.cpp:148-162); the backward step reads the softmax's result and the product's
+ * first operand, so both are written:
+ *     probs   = softmax(scale q k^T + mask)     dense float [heads][batch][lq][lk], as ntsamd_attention_probs
+ *     dropped = probs * dropMask                the same shape; written only if `dropped` is not NULL
+ *     out     = (dropMask ? dropped : probs) v  laid out by strides[9..11], as ntsamd_attention
+ * mask and dropMask may be NULL (no mask; no dropout, then `dropped` must be NULL too). q, k, v, out and strides
+ * as for ntsamd_attention; X_FLOAT only (the reference converts half scores to float for its softmax, and its
+ * dropout mask is a float tensor). Replaces, of this library's own entry points, ntsamd_attention_probs, the
+ * caller's Multiply and ntsamd_matrix_mul_batched_grid: the probabilities cross memory twice instead of five times.
+ */
+int ntsamd_attention_train(int devID, void * stream,
+                           const void * q, const void * k, const void * v, const void * mask, const void * dropMask,
+                           void * probs, void * dropped, void * out, int dataType,
+                           int heads, int batch, int lq, int lk, int dh,
+                           const long long * strides, float scale);
+
+/*
  * Element-wise data type conversion t[i] = (typeT) s[i], i < size.
  * Replaces _CudaConvertDataType(devID, s, typeS, t, typeT, size) and the tensor form
  * _CudaConvertDataType(input, output) (source/tensor/core/getandset/ConvertDataType.cu:78-99,

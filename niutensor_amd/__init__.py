@@ -33,6 +33,7 @@ EXPORTS = (
     "ntsamd_reduce_sum_xz",
     "ntsamd_attention",
     "ntsamd_attention_probs",
+    "ntsamd_attention_train",
     "ntsamd_convert_data_type",
     "ntsamd_release_workspaces",
     "ntsamd_matrix_mul_static",
@@ -77,6 +78,7 @@ def load():
     L.ntsamd_reduce_sum_xz.argtypes = [ci, vp, vp, ci, ci, ci, ci, vp, cf]
     L.ntsamd_attention.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     L.ntsamd_attention_probs.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
+    L.ntsamd_attention_train.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, C.POINTER(ll), cf]
     L.ntsamd_convert_data_type.argtypes = [ci, vp, vp, ci, vp, ci, ll]
     L.ntsamd_release_workspaces.argtypes = [ci]
     L.ntsamd_matrix_mul_static.argtypes = L.ntsamd_matrix_mul.argtypes + [ci]
@@ -296,6 +298,24 @@ def attention_probs(q, k, probs, heads, scale, mask=None):
                                        heads, batch, lq, lk, dh, strides, scale)
     _check(rc)
     return probs
+
+
+def attention_train(q, k, v, probs, out, heads, scale, mask=None, drop_mask=None, dropped=None):
+    """The training path in one launch: probs = softmax(scale q k^T + mask) ([heads][batch][lq][lk]),
+    dropped = probs * drop_mask (written if given), out = (dropped or probs) v in the merged layout of q."""
+    batch, lq, hd = (int(x) for x in q.shape)
+    lk = int(k.shape[1])
+    dh = hd // heads
+    for t in (q, k, v, probs, out):
+        assert t.is_contiguous()
+    st = lambda rows: (dh, rows * hd, hd)
+    strides = (C.c_longlong * 12)(*(st(lq) + st(lk) + st(lk) + st(lq)))
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    rc = load().ntsamd_attention_train(q.device.index, _stream_ptr(q), q.data_ptr(), k.data_ptr(), v.data_ptr(), ptr(mask),
+                                       ptr(drop_mask), probs.data_ptr(), ptr(dropped), out.data_ptr(), _dtype_code(q),
+                                       heads, batch, lq, lk, dh, strides, scale)
+    _check(rc)
+    return out
 
 
 def convert_data_type(s, t):

@@ -21,7 +21,11 @@ struct AttnParams {
     float scale;
     int qTiles;                         /* filled in by the launcher */
     int maskVec;                        /* filled in by the launcher: 16-byte mask loads are possible */
-    int probsVec;                       /* filled in by the launcher (attention_probs): 16-byte stores are possible */
+    int probsVec;                       /* filled in by the launcher (attention_probs, attention_train): 16-byte stores are possible */
+    /* the training form (attention_train_f32.hip): dense float [heads][batch][lq][lk] tensors */
+    float * probs;                      /* the softmax's result, written */
+    const float * dropMask;             /* NULL, or what the probabilities are multiplied with before the second product */
+    float * dropped;                    /* NULL, or where probs * dropMask is written */
 };
 
 int launch_attention_f32(const AttnParams & p, hipStream_t stream);
@@ -32,5 +36,7 @@ size_t attention_rows_lds(const AttnParams & p, bool half);
 int launch_attention_rows(const AttnParams & p, bool half, hipStream_t stream);
 /* probabilities only: out is the dense [heads][batch][lq][lk] tensor, v is not used */
 int launch_attention_probs_f32(const AttnParams & p, hipStream_t stream);
+/* the training path in one launch: probs, probs * dropMask and the merged context */
+int launch_attention_train_f32(const AttnParams & p, hipStream_t stream);
 
 }  // namespace ntsamd

@@ -32,6 +32,7 @@ int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void *
                          float * work, size_t workFloats);
 int launch_convert(int kind, const void * s, void * t, long long n, hipStream_t stream);
 int launch_repitch_f16(const void * s, long long srcPitch, void * t, int dstPitch, long long rows, int cols, hipStream_t stream);
+int launch_row_bias(bool half, void * c, int M, int N, int ldc, const void * bias, int div, int len, int act, hipStream_t stream);
 }
 
 using namespace ntsamd;
@@ -540,6 +541,21 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
 
     const Tuning & tn = tuning();
     hipStream_t hs = static_cast<hipStream_t>(stream);
+    /* A bias along a dimension that is not the last (one value per row, or per group of rows) is added by a pass of
+       its own behind the product, as the reference adds it (_SumDim with KernelAddWithCol behind the product,
+       MulAndShift.cpp:69-88), and the activation with it: the product itself then runs on the fast kernels, which
+       know a bias by column only. (Rows of 2^21 elements and more keep to the element-wise kernel, which adds either
+       kind of bias itself.) */
+    const void * rowBias = NULL;
+    int rowBiasAct = ACT_NONE;
+    if (bias != NULL && biasMode == NTSAMD_BIAS_ROW && !ptrs && !grid && count == 1 &&
+        lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 21)) {
+        rowBias = bias;
+        rowBiasAct = act;
+        bias = NULL;
+        biasMode = NTSAMD_BIAS_NONE;
+        act = ACT_NONE;
+    }
     WorkHold work;
     bool aInWork = false, repitched = false;
     if (kind_a32(kind) && !noAlloc && !ptrs && !grid && tn.a32Convert.load(std::memory_order_relaxed) != 0) {
@@ -860,8 +876,8 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
                  s.aKContig ? 'N' : 'T', s.bKContig ? 'T' : 'N', fetch, p.splits,
                  p.splits > 1 ? (viaWork ? "+split_reduce_kernel" : ",atomic") : "",
                  p.colSum != NULL ? " colsum=in-kernel" : "",
-                 bias != NULL ? (biasMode == NTSAMD_BIAS_ROW ? " bias=row" : " bias=col") : "",
-                 beta != 0.f ? " beta" : "", act != ACT_NONE ? " act" : "",
+                 rowBias != NULL ? "+row_bias_kernel" : (bias != NULL ? (biasMode == NTSAMD_BIAS_ROW ? " bias=row" : " bias=col") : ""),
+                 beta != 0.f ? " beta" : "", act != ACT_NONE || rowBiasAct != ACT_NONE ? " act" : "",
                  ptrs ? " list" : (grid ? " grid" : (count > 1 ? " strided" : "")));
     }
     if (planOnly)
@@ -882,6 +898,9 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     }
     if (rc == 0 && p.splits > 1 && viaWork)
         rc = launch_split_reduce(p, kind == KIND_F32 || kind_out_f32(kind), hs);
+    if (rc == 0 && rowBias != NULL)
+        rc = launch_row_bias(kind_c_half(kind), c, s.M, s.N, ldc, rowBias, biasRowDiv > 0 ? biasRowDiv : 1, biasLen > 0 ? biasLen : 1,
+                             rowBiasAct, hs);
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;
@@ -1306,6 +1325,81 @@ int ntsamd_attention_probs(int devID, void * stream,
     if (planOnly)
         return NTSAMD_OK;
     int rc = launch_attention_probs_f32(p, static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return NTSAMD_OK;
+}
+
+int ntsamd_attention_train(int devID, void * stream,
+                           const void * q, const void * k, const void * v, const void * mask, const void * dropMask,
+                           void * probs, void * dropped, void * out, int dataType,
+                           int heads, int batch, int lq, int lk, int dh,
+                           const long long * strides, float scale)
+{
+    if (dataType != NTSAMD_X_FLOAT)
+        return fail(NTSAMD_ERR_DATATYPE, "Unsupported data type!");
+    if (heads < 0 || batch < 0 || lq < 0 || lk < 0 || dh < 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "negative tensor size");
+    if (heads == 0 || batch == 0 || lq == 0)
+        return NTSAMD_OK;
+    if (lk == 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "attention over no keys");
+    if (!q || !k || !v || !probs || !out || !strides)
+        return fail(NTSAMD_ERR_ARGUMENT, "Empty input tensors!");
+    if (dropped && !dropMask)
+        return fail(NTSAMD_ERR_ARGUMENT, "dropped probabilities asked for without a dropout mask");
+    if (dh == 0 || dh > 128 || dh % 4 != 0)
+        return fail(NTSAMD_ERR_ARGUMENT, "head size %d is not served by the fused kernel (a multiple of 4 up to 128 is)", dh);
+    for (int i = 0; i < 12; i++)
+        if (strides[i] < 0 || strides[i] % 4 != 0)
+            return fail(NTSAMD_ERR_ARGUMENT, "strides must be non-negative multiples of 4 elements");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
+        return fail(NTSAMD_ERR_ARGUMENT, "q, k, v and out must be 16-byte aligned");
+    const void * four[4] = {mask, dropMask, probs, dropped};
+    for (int i = 0; i < 4; i++)
+        if (four[i] && (reinterpret_cast<uintptr_t>(four[i]) & 3) != 0)
+            return fail(NTSAMD_ERR_ARGUMENT, "misaligned mask or probabilities");
+    for (int t = 0; t < 4; t++)
+        if (strides[3 * t + 2] < dh)
+            return fail(NTSAMD_ERR_ARGUMENT, "row stride smaller than the head size");
+    if ((long long)heads * batch * ((lq + 63) / 64) > 0x7fffffffLL)
+        return fail(NTSAMD_ERR_ARGUMENT, "tensor too large");
+    for (int t = 1; t <= 2; t++)
+        if (((long long)lk + 256) * strides[3 * t + 2] * 4 > 0x7fffffffLL)
+            return fail(NTSAMD_ERR_ARGUMENT, "tensor too large: the keys of one head span more than 2 GiB");
+    const bool planOnly = g_planOnly;
+    if (!planOnly) {
+        int st = check_device(devID);
+        if (st != NTSAMD_OK)
+            return st;
+    }
+    DeviceScope scope(devID, planOnly);
+    if (scope.status != NTSAMD_OK)
+        return scope.status;
+    AttnParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.mask = static_cast<const float *>(mask);
+    p.dropMask = static_cast<const float *>(dropMask);
+    p.probs = static_cast<float *>(probs);
+    p.dropped = static_cast<float *>(dropped);
+    p.out = out;
+    p.heads = heads;
+    p.batch = batch;
+    p.lq = lq;
+    p.lk = lk;
+    p.dh = dh;
+    p.qH = strides[0]; p.qB = strides[1]; p.qL = strides[2];
+    p.kH = strides[3]; p.kB = strides[4]; p.kL = strides[5];
+    p.vH = strides[6]; p.vB = strides[7]; p.vL = strides[8];
+    p.oH = strides[9]; p.oB = strides[10]; p.oL = strides[11];
+    p.scale = scale;
+    snprintf(g_plan, sizeof(g_plan), "attention_train_f32_kernel%s%s", mask ? " mask" : "", dropMask ? " dropout" : "");
+    if (planOnly)
+        return NTSAMD_OK;
+    int rc = launch_attention_train_f32(p, static_cast<hipStream_t>(stream));
     if (rc != 0)
         return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return NTSAMD_OK;

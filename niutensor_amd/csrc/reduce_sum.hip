@@ -117,6 +117,37 @@ int launch_scale(bool half, void * v, long long n, float beta, hipStream_t strea
     return (int)hipGetLastError();
 }
 
+/* c[row][col] = f(c[row][col] + bias[(row / div) % len]): the broadcast add along a dimension that is not the last,
+   as a pass of its own behind the product, which is how the reference does it (_SumDim with KernelAddWithCol,
+   source/tensor/core/arithmetic/SumDim.cu:79-105, called from MulAndShift.cpp:88); f is the activation */
+template <typename T>
+__global__ void __launch_bounds__(256)
+row_bias_kernel(T * __restrict__ c, long long total, int N, int ldc, const T * __restrict__ bias, int div, int len, int act)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total)
+        return;
+    const long long row = i / N;
+    const int col = (int)(i - row * N);
+    T * at = c + row * ldc + col;
+    *at = (T)activate((float)*at + (float)bias[(row / div) % len], act);
+}
+
+int launch_row_bias(bool half, void * c, int M, int N, int ldc, const void * bias, int div, int len, int act, hipStream_t stream)
+{
+    const long long total = (long long)M * N;
+    if (total <= 0)
+        return 0;
+    dim3 grid((unsigned)((total + 255) / 256));
+    if (half)
+        hipLaunchKernelGGL(row_bias_kernel<half_t>, grid, dim3(256), 0, stream, static_cast<half_t *>(c), total, N, ldc,
+                           static_cast<const half_t *>(bias), div, len, act);
+    else
+        hipLaunchKernelGGL(row_bias_kernel<float>, grid, dim3(256), 0, stream, static_cast<float *>(c), total, N, ldc,
+                           static_cast<const float *>(bias), div, len, act);
+    return (int)hipGetLastError();
+}
+
 /* work: NULL, or workFloats floats of device memory that this stream's launches may use until the call's last
    kernel has run */
 int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void * out, float beta, hipStream_t stream,

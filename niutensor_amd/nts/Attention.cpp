@@ -161,4 +161,49 @@ XTensor AmdAttentionContext(const XTensor & probs, const XTensor & v, int nhead)
     return out;
 }
 
+void _AmdAttentionTrain(const XTensor * q, const XTensor * k, const XTensor * v, const XTensor * mask, const XTensor * dropMask,
+                        XTensor * probs, XTensor * dropped, XTensor * out, int nhead, DTYPE scale)
+{
+    CheckNTErrors((q && k && v && probs && out), "Empty input tensors!");
+    CheckNTErrors((q->dataType == X_FLOAT && k->dataType == X_FLOAT && v->dataType == X_FLOAT &&
+                   probs->dataType == X_FLOAT && out->dataType == X_FLOAT), "TODO!");
+    CheckNTErrors((q->order >= 2 && q->order == k->order && q->order == v->order && q->order == out->order &&
+                   probs->order == q->order + 1), "Input tensors must have the same order >= 2!");
+    CheckNTErrors((q->devID >= 0), "This code must be run on GPUs!");
+    CheckNTErrors((q->devID == k->devID && q->devID == v->devID && q->devID == out->devID && q->devID == probs->devID),
+                  "The tensors must be on the same GPU!");
+    CheckNTErrors((_IsSameShaped(k, v) && _IsSameShaped(q, out)), "Unmatched tensors in attention!");
+    CheckNTErrors((dropped == NULL || dropMask != NULL), "Unmatched tensors in attention!");
+
+    const int order = q->order;
+    const int hidden = q->dimSize[order - 1];
+    const int lq = q->dimSize[order - 2], lk = k->dimSize[order - 2];
+    CheckNTErrors((nhead > 0 && hidden % nhead == 0), "The hidden size must be a multiple of the number of heads!");
+    CheckNTErrors((k->dimSize[order - 1] == hidden), "Unmatched tensors in attention!");
+    int batch = 1;
+    for (int i = 0; i < order - 2; i++) {
+        CheckNTErrors((q->dimSize[i] == k->dimSize[i]), "Unmatched tensors in attention!");
+        batch *= q->dimSize[i];
+    }
+    CheckNTErrors((probs->unitNum == nhead * batch * lq * lk), "Unmatched tensors in attention!");
+    const XTensor * like[3] = {mask, dropMask, dropped};
+    for (int i = 0; i < 3; i++)
+        if (like[i] != NULL) {
+            CheckNTErrors((like[i]->dataType == X_FLOAT && like[i]->devID == q->devID && like[i]->unitNum == probs->unitNum),
+                          "Unmatched tensors in attention!");
+        }
+    const int dh = hidden / nhead;
+    long long strides[12] = {dh, (long long)lq * hidden, hidden,
+                             dh, (long long)lk * hidden, hidden,
+                             dh, (long long)lk * hidden, hidden,
+                             dh, (long long)lq * hidden, hidden};
+    int rc = ntsamd_attention_train(q->devID, NULL, q->data, k->data, v->data, mask != NULL ? mask->data : NULL,
+                                    dropMask != NULL ? dropMask->data : NULL, probs->data,
+                                    dropped != NULL ? dropped->data : NULL, out->data, X_FLOAT,
+                                    nhead, batch, lq, lk, dh, strides, scale);
+    if (rc != NTSAMD_OK) {
+        ShowNTErrors(ntsamd_last_error());
+    }
+}
+
 }  // namespace nts

@@ -34,5 +34,15 @@ XTensor AmdAttentionProbs(const XTensor & q, const XTensor & k, const XTensor * 
 void _AmdAttentionContext(const XTensor * probs, const XTensor * v, XTensor * out, int nhead);
 XTensor AmdAttentionContext(const XTensor & probs, const XTensor & v, int nhead);
 
+/* The whole of MakeAttention between the projections when it IS training (:194-242), one launch:
+       probs   = Softmax(Split(q) * scale x Split(k)^T + mask, -1)      (nhead, batch..., lq, lk), written
+       dropped = probs * dropMask                                        the same shape, written if not NULL
+       out     = Merge((dropMask ? dropped : probs) x Split(v))          (batch..., lq, hidden)
+   dropMask is the tensor Dropout multiplies with (0 and 1 / (1 - p), filled by the caller's generator,
+   source/tensor/function/Dropout.cpp:148-162); the backward step reads probs (the softmax's gradient) and dropped
+   (the gradient of v). All X_FLOAT. */
+void _AmdAttentionTrain(const XTensor * q, const XTensor * k, const XTensor * v, const XTensor * mask, const XTensor * dropMask,
+                        XTensor * probs, XTensor * dropped, XTensor * out, int nhead, DTYPE scale);
+
 }  // namespace nts
 #endif

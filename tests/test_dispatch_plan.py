@@ -114,8 +114,9 @@ def test_no_product_the_16_byte_routes_accept_goes_element_wise(planning):
     # the draw reaches every family and the walking kernel
     for family in ("gemm_f32_kernel", "gemm_f16_direct_kernel", "gemm_f16_kernel", "gemm_f16_persistent_kernel"):
         assert any(family in k for k in seen), (family, sorted(seen))
-    # a bias by row and rows of 2^21 elements are what the element-wise kernel is for
+    # a bias by row is a pass of its own behind a product on the fast kernels; rows of 2^21 elements are what the
+    # element-wise kernel is for
     rc, plan = plan_mm(L, 64, 64, 64, X_NOTRANS, X_NOTRANS, bias=0x400000, bias_mode=nt.BIAS_ROW)
-    assert rc == 0 and "fetch=elementwise" in plan and "bias=row" in plan
+    assert rc == 0 and "fetch=vec16" in plan and "+row_bias_kernel" in plan
     rc, plan = plan_mm(L, 4, 1 << 21, 8, X_NOTRANS, X_NOTRANS)
     assert rc == 0 and "fetch=elementwise" in plan

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 import niutensor_amd as nt
+from niutensor_amd import X_NOTRANS
 from tolerance import FP16_LIMIT, assert_fp32, normwise, scaled
 
 pytestmark = pytest.mark.gpu
@@ -159,6 +160,63 @@ def test_probabilities_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     vh = v.reshape(B, lk, nh, H // nh).transpose(2, 0, 1, 3).astype(np.float64)
     two_step = (got.astype(np.float64) @ vh).transpose(1, 2, 0, 3).reshape(B, lq, H)
     assert np.abs(whole - two_step).max() <= 1e-5 * np.sqrt(H // nh + lk) * np.abs(two_step).max()
+
+
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked,dropout", [
+    (2, 128, 128, 128, 2, False, True),     # one key block, 16-byte moves
+    (3, 100, 77, 96, 3, True, True),        # ragged rows and keys: scalar moves
+    (1, 300, 516, 64, 1, True, True),       # several key blocks: a first pass for the maxima and sums
+    (2, 40, 261, 256, 2, False, True),      # head size 128, ragged
+    (4, 9, 5, 8, 2, False, False),          # head size 4, no dropout
+    (2, 70, 200, 128, 4, True, False),
+])
+def test_training_path_in_one_launch(gpu, oracle, B, lq, lk, H, nh, masked, dropout):
+    """ntsamd_attention_train against the operator chain of the reference's training path put together from the
+    oracle's pieces: probabilities from the oracle's Split, Scale, BMMul, Sum, Softmax (oracle_attention_probs);
+    Dropout as the element-wise product with a mask of 0 and 1 / (1 - p) (the reference's Dropout is exactly that
+    product); the oracle's batched product with the split values; the merge. The probabilities must also be what
+    ntsamd_attention_probs writes, bit for bit where both make one pass."""
+    torch = torch_()
+    print("\n[gpu-case] attention_train B=%d lq=%d lk=%d H=%d heads=%d mask=%d dropout=%d" % (B, lq, lk, H, nh, masked, dropout), flush=True)
+    q, k, v = oracle.normal((B, lq, H), 81), oracle.normal((B, lk, H), 82), oracle.normal((B, lk, H), 83)
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 84, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., lk // 2] = 0.0
+    drop = None
+    if dropout:
+        drop = np.where(oracle.uniform((nh, B, lq, lk), 85, 0.0, 1.0) < 0.1, 0.0, 1.0 / 0.9).astype(np.float32)
+    scale = float(np.float32(1.0 / np.sqrt(H // nh)))
+    dh = H // nh
+    p_ref = oracle.attention_probs(q, k, nh, scale, mask)
+    d_ref = p_ref * drop if dropout else p_ref
+    vh = np.ascontiguousarray(v.reshape(B, lk, nh, dh).transpose(2, 0, 1, 3))
+    c_ref = oracle.matmul_batched(d_ref.reshape(nh * B, lq, lk), X_NOTRANS, vh.reshape(nh * B, lk, dh), X_NOTRANS)
+    o_ref = c_ref.reshape(nh, B, lq, dh).transpose(1, 2, 0, 3).reshape(B, lq, H)
+
+    nan = lambda *shape: torch.full(shape, float("nan"), device=gpu)
+    probs, dropped, out = nan(nh, B, lq, lk), (nan(nh, B, lq, lk) if dropout else None), nan(B, lq, H)
+    nt.attention_train(dev(q, gpu), dev(k, gpu), dev(v, gpu), probs, out, nh, scale, mask=dev(mask, gpu) if masked else None,
+                       drop_mask=dev(drop, gpu) if dropout else None, dropped=dropped)
+    torch.cuda.synchronize()
+    got_p, got_o = probs.cpu().numpy(), out.cpu().numpy()
+    assert np.isfinite(got_p).all() and np.isfinite(got_o).all()
+    assert np.abs(got_p - p_ref).max() <= 1e-5 * np.sqrt(dh)
+    assert np.abs(got_p.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+    if dropout:
+        got_d = dropped.cpu().numpy()
+        assert np.isfinite(got_d).all()
+        assert np.array_equal(got_d, got_p * drop)              # one fp32 product per element, as Multiply does it
+        assert (got_d[drop == 0] == 0).all()
+    assert np.abs(got_o - o_ref).max() <= 1e-5 * np.sqrt(dh + lk) * np.abs(o_ref).max()
+    # the probabilities on their own: the same kernel arithmetic
+    alone = nan(nh, B, lq, lk)
+    nt.attention_probs(dev(q, gpu), dev(k, gpu), alone, nh, scale, mask=dev(mask, gpu) if masked else None)
+    assert np.abs(alone.cpu().numpy() - got_p).max() <= 2e-7
+    # without dropout the result is the attention of the one-kernel path
+    if not dropout:
+        whole = run(gpu, q, k, v, nh, scale, mask)
+        assert np.abs(whole - got_o).max() <= 1e-5 * np.sqrt(dh + lk) * np.abs(o_ref).max()
 
 
 def halfed(oracle, x):
