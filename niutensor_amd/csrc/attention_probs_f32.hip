@@ -96,35 +96,47 @@ attention_probs_f32_kernel(const AttnParams p)
 #pragma unroll
         for (int j = 0; j < NJ; j++)
             accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        f32x4 kf[2][NJ];
+        /* The key fragments come from LDS two blocks of 16 keys at a time, one step ahead of the eight products
+           that use them (16 registers, where fragments for a whole group would be 64). What that frees holds a mask
+           that moves 16 bytes at a time, asked for before the product begins and without a branch (keys past the
+           end read the row's last ones and are overwritten below), so that its loads travel together and behind
+           the product. */
+        constexpr int PAIRS = NJ / 2, STEPS = NT * PAIRS;
+        const bool maskEarly = MK != nullptr && p.maskVec;
+        f32x4 kf[2][2], mk[NJ];
+        if (maskEarly) {
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-            kf[0][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 4 * g]);
+            for (int j = 0; j < NJ; j++) {
+                const int key = kb0 + 16 * j + 4 * g;
+                mk[j] = *reinterpret_cast<const f32x4 *>(MK + (key < lk ? key : lk - 4));
+            }
+        }
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            if (t + 1 < NT) {
+        for (int i = 0; i < 2; i++)
+            kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KP + 4 * g]);
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
-                    kf[(t + 1) & 1][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 16 * (t + 1) + 4 * g]);
+        for (int st = 0; st < STEPS; st++) {
+            const int t = st / PAIRS, j0 = 2 * (st % PAIRS);
+            if (st + 1 < STEPS) {
+                const int t1 = (st + 1) / PAIRS, j1 = 2 * ((st + 1) % PAIRS);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KP + 16 * t1 + 4 * g]);
             }
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
-                    accS[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t & 1][j][e], qf[t][e], accS[j], 0, 0, 0);
+                for (int i = 0; i < 2; i++)
+                    accS[j0 + i] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st & 1][i][e], qf[t][e], accS[j0 + i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (MK != nullptr) {
             if (p.maskVec) {
 #pragma unroll
-                for (int j = 0; j < NJ; j++) {
-                    const int key = kb0 + 16 * j + 4 * g;
-                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK + key) : z;
+                for (int j = 0; j < NJ; j++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        accS[j][r] = fmaf(mk[r], LOG2E, accS[j][r] * scale2);
-                }
+                        accS[j][r] = fmaf(mk[j][r], LOG2E, accS[j][r] * scale2);
             }
             else {
 #pragma unroll

@@ -115,39 +115,55 @@ attention_train_f32_kernel(const AttnParams p)
     float rowMax = -INFINITY, rowSum = 0.f;              /* in units of log2: the scores are scaled by log2(e) */
 
     /* the scaled and masked scores (times log2 e) of this wave's rows against the block of keys in LDS */
-    auto scores = [&](int kb0, f32x4 (&accS)[NJ]) {
+    /* The key fragments come from LDS two blocks of 16 keys at a time, one step ahead of the eight products that
+       use them: 16 registers, where fragments for a whole slice of the head dimension would be 64. What that frees
+       holds the loads that travel behind this product: a mask that moves 16 bytes at a time and the first values
+       (firstV) from its start, the dropout mask (dropMask) from the start of its last slice. The mask is read
+       without a branch (keys past the end read the row's last ones and are overwritten below), so that its loads
+       travel together. */
+    const bool maskEarly = MK != nullptr && p.maskVec;
+    auto scores = [&](int kb0, f32x4 (&accS)[NJ], auto && firstV, auto && dropMask) {
+        constexpr int PAIRS = NJ / 2, STEPS = NT * PAIRS;
 #pragma unroll
         for (int j = 0; j < NJ; j++)
             accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        f32x4 kf[2][NJ];
+        f32x4 kf[2][2], mk[NJ];
+        if (maskEarly) {
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-            kf[0][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 4 * g]);
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            if (t + 1 < NT) {
-#pragma unroll
-                for (int j = 0; j < NJ; j++)
-                    kf[(t + 1) & 1][j] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * j + m) * KP + 16 * (t + 1) + 4 * g]);
+            for (int j = 0; j < NJ; j++) {
+                const int key = kb0 + 16 * j + 4 * g;
+                mk[j] = *reinterpret_cast<const f32x4 *>(MK + rowAt + (key < lk ? key : lk - 4));
             }
+        }
+        firstV();
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KP + 4 * g]);
+#pragma unroll
+        for (int st = 0; st < STEPS; st++) {
+            const int t = st / PAIRS, j0 = 2 * (st % PAIRS);
+            if (st + 1 < STEPS) {
+                const int t1 = (st + 1) / PAIRS, j1 = 2 * ((st + 1) % PAIRS);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KP + 16 * t1 + 4 * g]);
+            }
+            if (st == STEPS - PAIRS)
+                dropMask();
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
-                    accS[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t & 1][j][e], qf[t][e], accS[j], 0, 0, 0);
+                for (int i = 0; i < 2; i++)
+                    accS[j0 + i] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st & 1][i][e], qf[t][e], accS[j0 + i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (MK != nullptr) {
             if (p.maskVec) {
 #pragma unroll
-                for (int j = 0; j < NJ; j++) {
-                    const int key = kb0 + 16 * j + 4 * g;
-                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK + rowAt + key) : z;
+                for (int j = 0; j < NJ; j++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        accS[j][r] = fmaf(mk[r], LOG2E, accS[j][r] * scale2);
-                }
+                        accS[j][r] = fmaf(mk[j][r], LOG2E, accS[j][r] * scale2);
             }
             else {
 #pragma unroll
@@ -207,7 +223,7 @@ attention_train_f32_kernel(const AttnParams p)
             __syncthreads();
             load_k(kb0 + KB < lk ? kb0 + KB : 0);            /* the next block, or the first again for the second pass */
             f32x4 accS[NJ];
-            scores(kb0, accS);
+            scores(kb0, accS, [] {}, [] {});
             fold(accS);
             __syncthreads();                                 /* every wave is done with this block of keys */
         }
@@ -224,32 +240,33 @@ attention_train_f32_kernel(const AttnParams p)
         for (int s = 0; s < LOADS; s++)
             *reinterpret_cast<f32x4 *>(&Ks[sLds + s * RSTEP * KP]) = kreg[s];
         __syncthreads();                                 /* also: every wave has finished the previous block's Vs */
-        if (kb0 == 0)
-            load_v(0);
         if (more)
             load_k(kb0 + KB);
 
-        f32x4 accS[NJ];
-        scores(kb0, accS);
-        /* the dropout mask of this block is asked for now, when the key fragments' registers are free, and
-           travels while the softmax is worked out */
-        f32x4 dm[NJ];
-        __builtin_amdgcn_sched_barrier(0);               /* (not earlier: the first product has no registers to spare) */
-        if (DM != nullptr) {
+        f32x4 accS[NJ], dm[NJ];
+        scores(kb0, accS, [&] {
+            if (kb0 == 0)
+                load_v(0);
+        }, [&] {
+            if (DM == nullptr)
+                return;
+            if (p.probsVec) {                  /* (keys past the end: any finite value, their probabilities are 0) */
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                const int key = kb0 + 16 * j + 4 * g;
-                if (p.probsVec) {
-                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    dm[j] = key < lk ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(DM + rowAt + key)) : z;
-                }
-                else {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        dm[j][r] = DM[rowAt + (key + r < lk ? key + r : lk - 1)];
+                for (int j = 0; j < NJ; j++) {
+                    const int key = kb0 + 16 * j + 4 * g;
+                    dm[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(DM + rowAt + (key < lk ? key : lk - 4)));
                 }
             }
-        }
+            else {
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int key = kb0 + 16 * j + 4 * g + r;
+                        dm[j][r] = DM[rowAt + (key < lk ? key : lk - 1)];
+                    }
+            }
+        });
         if (oneBlock)
             fold(accS);
         const float shift = rowMax == -INFINITY ? 0.f : rowMax;

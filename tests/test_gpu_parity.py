@@ -13,7 +13,7 @@ import pytest
 
 import niutensor_amd as nt
 from niutensor_amd import BIAS_COL, BIAS_ROW, X_NOTRANS, X_TRANS
-from tolerance import assert_fp16, assert_fp32, fp32_limit, normwise
+from tolerance import FP16_LIMIT, assert_fp16, assert_fp32, fp32_limit, normwise, scaled
 
 pytestmark = pytest.mark.gpu
 
@@ -668,10 +668,16 @@ def test_fused_bias(gpu, oracle, half):
         nt.matrix_mul(dev_tensor(x.reshape(120, 48), gpu, half), X_NOTRANS, dev_tensor(w, gpu, half), X_NOTRANS, c, 0.5, 0.0,
                       bias=dev_tensor(bias.ravel(), gpu, half), bias_mode=mode, bias_row_div=div)
         got = c.float().cpu().numpy().reshape(ref.shape)
-        if half:
+        mag = 0.5 * oracle.matmul(np.abs(x), X_NOTRANS, np.abs(w), X_NOTRANS) + np.abs(ref - oracle.matmul(x, X_NOTRANS, w, X_NOTRANS, None, 0.5))
+        if half and mode == BIAS_ROW:
+            # a bias by row is added behind the product, as the reference adds it (_SumDim on the half result,
+            # MulAndShift.cpp:69-88): the product is rounded to half before the sum is, so where the two nearly
+            # cancel the error is a half ulp of the product, not of the sum
+            assert np.isfinite(got).all()
+            assert normwise(got, ref) <= FP16_LIMIT and scaled(got, ref, mag) <= FP16_LIMIT, str(bshape)
+        elif half:
             assert_fp16(got, ref, what=str(bshape))
         else:
-            mag = 0.5 * oracle.matmul(np.abs(x), X_NOTRANS, np.abs(w), X_NOTRANS) + np.abs(ref - oracle.matmul(x, X_NOTRANS, w, X_NOTRANS, None, 0.5))
             assert_fp32(got, ref, 48, mag, what=str(bshape))
 
 
