@@ -85,6 +85,7 @@ struct GemmParams {
     float * splitWork;
     int act;                               /* Activation of the epilogue */
     int wideRowsOnly;                      /* fp32, measurements: no 16-row MFMAs for products of at most 16 rows */
+    int f16Slab64;                         /* half, 64 x 64 tile on the LDS-direct path: slabs of 64 along k */
     int f16PingPong;                       /* half, 256 x 256 tile: the two wave groups run one phase apart */
     int storeHint;                         /* != 0: the fast epilogues write c through (STORE_WRITE_THROUGH) */
     int persistGrid;                       /* half, 256 x 256 tile: > 0 = that many workgroups walk over all tiles */

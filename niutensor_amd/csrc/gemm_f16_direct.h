@@ -19,6 +19,9 @@
  *       column c at position c ^ ((r >> 2) & 3): rows r, r+4, r+8, r+12 share their
  *       64 bytes of a 256-byte line, and sixteen consecutive rows reading the same
  *       logical column hit sixteen different 16-byte bank groups.
+ *       With slabs of 64 along k (BKT_ = 64, the 64 x 64 tile only) a row is a whole
+ *       128-byte line, a chunk is 8 rows, and column c of row r sits at position
+ *       c ^ ((r >> 1) & 7): rows of equal parity share their half of a 256-byte line.
  *   MN-contiguous operand (rows of k): a chunk holds rows k, k + NCH, k + 2 NCH ...
  *       (NCH chunks per slab), and chunks are 1 KB + 64 bytes apart, so the four
  *       consecutive k rows of one transposing read sit in four different chunks,
@@ -86,22 +89,25 @@ __device__ __forceinline__ void lds_dma16(i32x4 desc, unsigned ldsAddr, int byte
    as plain fp32 (no alpha, beta, bias or activation) in p.splitWork, which holds p.splits x p.batch dense M x N
    matrices; split_reduce.hip adds the pieces up and does what the epilogue would have done. */
 template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4,
-          bool PP = false>
+          bool PP = false, int BKT_ = 32>
 __global__ void __launch_bounds__(WGM * WGN * 64, MINW)
 gemm_f16_direct_kernel(const GemmParams p)
 {
     static_assert(!CS || std::is_same<OutT, half_t>::value, "column sums have the type of b and of c");
     static_assert(!(CS && SPLIT), "column sums are not gathered from pieces of k");
     static_assert(!SPLIT || std::is_same<OutT, float>::value, "partial tiles are fp32");
-    constexpr int BKT = 32, KS = 2;
+    constexpr int BKT = BKT_, KS = BKT / 16;               /* slab depth, MFMA k steps per slab */
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TI = WM / 32, TJ = WN / 32;
+    static_assert(BKT == 32 || (BKT == 64 && TI == 1 && TJ == 1 && !PP), "slabs of 64: the one-block wave tile only");
     /* per-operand LDS geometry, bytes */
-    constexpr int A_RPC = AKC ? 16 : 512 / BM;             /* rows per chunk */
-    constexpr int B_RPC = BKC ? 16 : 512 / BN;
-    constexpr int A_NCH = AKC ? BM / 16 : BKT / A_RPC;     /* chunks per slab */
-    constexpr int B_NCH = BKC ? BN / 16 : BKT / B_RPC;
+    constexpr int ROWB = BKT * 2;                          /* a K-contiguous row of a slab */
+    constexpr int LPRK = BKT / 8;                          /* lanes per such row */
+    constexpr int A_RPC = AKC ? 1024 / ROWB : 512 / BM;    /* rows per chunk */
+    constexpr int B_RPC = BKC ? 1024 / ROWB : 512 / BN;
+    constexpr int A_NCH = AKC ? BM / A_RPC : BKT / A_RPC;  /* chunks per slab */
+    constexpr int B_NCH = BKC ? BN / B_RPC : BKT / B_RPC;
     constexpr int A_CP = AKC ? 1024 : 1088;                /* chunk pitch */
     constexpr int B_CP = BKC ? 1024 : 1088;
     constexpr int A_BYTES = A_NCH * A_CP;
@@ -141,8 +147,8 @@ gemm_f16_direct_kernel(const GemmParams p)
     for (int q = 0; q < NLA; q++) {
         const int ch = wave * NLA + q;
         if (AKC) {
-            int row = ch * 16 + (lane >> 2);
-            int col = (lane & 3) ^ ((row >> 2) & 3);
+            int row = ch * A_RPC + lane / LPRK;
+            int col = (lane % LPRK) ^ (BKT == 32 ? (row >> 2) & 3 : (row >> 1) & 7);
             aKc[q] = col * 8;
             int r = m0 + row < M - 1 ? row : M - 1 - m0;
             aOff[q] = (r * p.lda + col * 8) * 2;
@@ -160,8 +166,8 @@ gemm_f16_direct_kernel(const GemmParams p)
     for (int q = 0; q < NLB; q++) {
         const int ch = wave * NLB + q;
         if (BKC) {
-            int row = ch * 16 + (lane >> 2);
-            int col = (lane & 3) ^ ((row >> 2) & 3);
+            int row = ch * B_RPC + lane / LPRK;
+            int col = (lane % LPRK) ^ (BKT == 32 ? (row >> 2) & 3 : (row >> 1) & 7);
             bKc[q] = col * 8;
             int r = n0 + row < N - 1 ? row : N - 1 - n0;
             bOff[q] = (r * p.ldb + col * 8) * 2;
@@ -218,9 +224,9 @@ gemm_f16_direct_kernel(const GemmParams p)
     int aTr[KS][2], bTr[KS][2];    /* MN-contiguous: offset for k step kk, half h, block 0 */
 #pragma unroll
     for (int kk = 0; kk < KS; kk++) {
-        const int sw = (l32 >> 2) & 3;
-        aFrag[kk] = (wm0 + l32) * 64 + ((kk * 2 + lh) ^ sw) * 16;
-        bFrag[kk] = A_BYTES + (wn0 + l32) * 64 + ((kk * 2 + lh) ^ sw) * 16;
+        const int sw = BKT == 32 ? (l32 >> 2) & 3 : (l32 >> 1) & 7;
+        aFrag[kk] = (wm0 + l32) * ROWB + ((kk * 2 + lh) ^ sw) * 16;
+        bFrag[kk] = A_BYTES + (wn0 + l32) * ROWB + ((kk * 2 + lh) ^ sw) * 16;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const int kr = 16 * kk + 8 * lh + 4 * h + trRow;
@@ -237,7 +243,7 @@ gemm_f16_direct_kernel(const GemmParams p)
         if (f < TI) {
             const int i = f;
             if constexpr (AKC)
-                fa[kk][i] = *reinterpret_cast<const f16x8 *>(stage + aFrag[kk] + i * 32 * 64);
+                fa[kk][i] = *reinterpret_cast<const f16x8 *>(stage + aFrag[kk] + i * 32 * ROWB);
             else {
                 f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][0] + i * 64));
                 f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + aTr[kk][1] + i * 64));
@@ -247,7 +253,7 @@ gemm_f16_direct_kernel(const GemmParams p)
         else {
             const int j = f - TI;
             if constexpr (BKC)
-                fb[kk][j] = *reinterpret_cast<const f16x8 *>(stage + bFrag[kk] + j * 32 * 64);
+                fb[kk][j] = *reinterpret_cast<const f16x8 *>(stage + bFrag[kk] + j * 32 * ROWB);
             else {
                 f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][0] + j * 64));
                 f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(stage + bTr[kk][1] + j * 64));
@@ -363,6 +369,10 @@ gemm_f16_direct_kernel(const GemmParams p)
     constexpr bool DEEP = TI == 1 && TJ == 1;
     if constexpr (DEEP) {
         f16x8 da[2][KS], db[2][KS];                  /* [set][k step] */
+        f32x16 accOdd;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            accOdd[r] = 0.f;
         auto read_set = [&](auto SETC, const char * stage) {
             constexpr int S = decltype(SETC)::value;
 #pragma unroll
@@ -402,7 +412,12 @@ gemm_f16_direct_kernel(const GemmParams p)
             }
 #pragma unroll
             for (int kk = 0; kk < KS; kk++) {
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(da[S][kk], db[S][kk], acc[0][0], 0, 0, 0);
+                /* slabs of four k steps: odd steps add into a second accumulator, so that no MFMA waits for the
+                   one before it (a lone wave on its SIMD has nobody to fill that wait) */
+                if (KS == 4 && (kk & 1))
+                    accOdd = __builtin_amdgcn_mfma_f32_32x32x16_f16(da[S][kk], db[S][kk], accOdd, 0, 0, 0);
+                else
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(da[S][kk], db[S][kk], acc[0][0], 0, 0, 0);
                 if constexpr (CS) {
                     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
                     const h2 ones = {(_Float16)1, (_Float16)1};
@@ -468,6 +483,11 @@ gemm_f16_direct_kernel(const GemmParams p)
                 rest(rest, IntC<NSTAGE + 1>(), IntC<1>());
             else
                 rest(rest, IntC<NSTAGE + 1>(), IntC<0>());
+        }
+        if constexpr (KS == 4) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[0][0][r] += accOdd[r];
         }
     }
     else if constexpr (PP) {
@@ -783,7 +803,7 @@ gemm_f16_direct_kernel(const GemmParams p)
 }
 
 template <typename OutT, int BM, int BN, int WGM, int WGN, int MINW, bool AKC, bool BKC, bool CS, bool SPLIT = false, int NSTAGE = 4,
-          bool PP = false>
+          bool PP = false, int BKT = 32>
 static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
 {
     GemmParams p = p0;
@@ -792,7 +812,7 @@ static int launch_f16_direct_shape(const GemmParams & p0, hipStream_t stream)
     if (!SPLIT)
         p.splits = 1;
     dim3 grid((unsigned)(p.tilesM * p.tilesN * p.batch * p.splits));
-    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT, NSTAGE, PP>),
+    hipLaunchKernelGGL((gemm_f16_direct_kernel<OutT, BM, BN, WGM, WGN, MINW, AKC, BKC, CS, SPLIT, NSTAGE, PP, BKT>),
                        grid, dim3(WGM * WGN * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -814,9 +834,19 @@ static int launch_f16_direct(const GemmParams & p, hipStream_t stream)
     }
     else if constexpr (!CS) {
         /* pieces of k leave fp32 partial tiles, whatever the type of c */
-        if (p.splits > 1 && p.splitWork != NULL)
+        if (p.splits > 1 && p.splitWork != NULL) {
+            if constexpr (CFG == CFG_64x64)
+                if (p.f16Slab64)
+                    return launch_f16_direct_shape<float, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS, true, 4, false, 64>(p, stream);
             return launch_f16_direct_shape<float, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS, true>(p, stream);
+        }
     }
+    /* the small tile with slabs of 64: whole 128-byte lines of a K-contiguous operand per load, half the barriers
+       and waits per k, four stages of 16-17 KB (three or six stages cost a division by a number that is no power
+       of two where a stage's address is worked out, and ran slower than four; eight leave one workgroup to a CU) */
+    if constexpr (CFG == CFG_64x64)
+        if (p.f16Slab64)
+            return launch_f16_direct_shape<OutT, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS, false, 4, false, 64>(p, stream);
     return launch_f16_direct_shape<OutT, S::BM, S::BN, S::WGM, S::WGN, S::MINW16, AKC, BKC, CS>(p, stream);
 }
 

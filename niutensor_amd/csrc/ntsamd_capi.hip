@@ -219,7 +219,7 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
 double tile_cost_f16(int M, int N, int K, int count, int bm, int splits)
 {
     if (splits > 1) {
-        const int kPiece = ((K + splits - 1) / splits + 31) / 32 * 32;
+        const int kPiece = ((K + splits - 1) / splits + 63) / 64 * 64;
         return tile_cost_f16(M, N, kPiece, count * splits, bm, 1) + SPLIT_FIXED_US +
                8.0 * M * N * count * splits / SPLIT_BYTES_PER_US;
     }
@@ -239,9 +239,10 @@ double tile_cost_f16(int M, int N, int K, int count, int bm, int splits)
         }
         return (double)rounds * 0.0086 * K + 4.3 + 1.4 * (double)(rounds - 1);
     }
+    /* up to two workgroups to a CU run with slabs of 64 (see where f16Slab64 is set) */
     if (alone)
-        return 0.0045 * K + (groups <= 128 ? 3.15 : 3.45);
-    return (double)rounds * 0.00368 * K + 3.5 + 0.47 * (double)(rounds - 1);
+        return 0.0034 * K + (groups <= 128 ? 3.15 : 3.45);
+    return (double)rounds * (rounds <= 2 ? 0.0026 : 0.00368) * K + 3.5 + 0.47 * (double)(rounds - 1);
 }
 
 struct Plan {
@@ -266,10 +267,12 @@ struct Plan {
      NTSAMD_A32_CONVERT=0|1      float a with half b: never / whenever it fits the workspace, round a to half in a pass
                                  of its own before the product
      NTSAMD_F16_PERSIST_BETA=0   half products that read the old c keep to the one-tile kernels
+     NTSAMD_F16_SLAB64=0|1       half, 64 x 64 tile on the 16-byte path: slabs of 32 / of 64 along k, however many
+                                 workgroups share a CU
      NTSAMD_F16_REPITCH=0|1      half operands with rows that are no whole 16-byte pieces: never / whenever they fit the
                                  workspace, copied there with padded rows so that the product takes the 16-byte path */
 struct Tuning {
-    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert, f16Repitch, f16PersistBeta;
+    std::atomic<int> tileCfg, splitK, f16Fetch, attnRows, f32R16, f32SplitAtomic, f16PingPong, f16Persist, storeHint, groupM, a32Convert, f16Repitch, f16PersistBeta, f16Slab64;
 };
 Tuning g_tuning;
 std::once_flag g_tuningOnce;
@@ -285,7 +288,7 @@ const Knob g_knobs[] = {
     {"NTSAMD_F16_PINGPONG", &Tuning::f16PingPong}, {"NTSAMD_F16_PERSIST", &Tuning::f16Persist},
     {"NTSAMD_STORE_HINT", &Tuning::storeHint}, {"NTSAMD_GROUP_M", &Tuning::groupM},
     {"NTSAMD_A32_CONVERT", &Tuning::a32Convert}, {"NTSAMD_F16_REPITCH", &Tuning::f16Repitch},
-    {"NTSAMD_F16_PERSIST_BETA", &Tuning::f16PersistBeta},
+    {"NTSAMD_F16_PERSIST_BETA", &Tuning::f16PersistBeta}, {"NTSAMD_F16_SLAB64", &Tuning::f16Slab64},
 };
 
 const Tuning & tuning()
@@ -797,9 +800,23 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
     }
     p.splits = 1;
     if (plan.splits > 1) {
-        p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 31) / 32 * 32;
+        p.kPerSplit = ((s.K + plan.splits - 1) / plan.splits + 63) / 64 * 64;
         p.splits = (s.K + p.kPerSplit - 1) / p.kPerSplit;
         p.splitWork = viaWork ? work.mem : NULL;
+    }
+    {
+        /* The small half tile on the LDS-direct path with slabs of 64 along k (whole 128-byte lines of a k-contiguous
+           operand per load, twice the bytes on their way per workgroup) as long as a CU has at most two workgroups:
+           its four stages take 68 KB of LDS, so two fit where four of the 32-deep kernel do. Measured, all layouts:
+           1024 x 1024 x 4096 22.2 -> 17.1 us, 4096 x 512 x 2048 16.6 -> 14.5, 4096 x 512 x 512 6.8 -> 6.2,
+           512 x 512 x 4096 in four pieces 11.8 -> 10.8; with four workgroups to a CU (8192 x 512 x 512 on this tile)
+           10.3 -> 12.4. */
+        const int knob = tn.f16Slab64.load(std::memory_order_relaxed);
+        int cus = g_deviceCUs[devID].load(std::memory_order_relaxed);
+        if (cus <= 0)
+            cus = 256;
+        const long long groups = (long long)((s.M + 63) / 64) * ((s.N + 63) / 64) * count * p.splits;
+        p.f16Slab64 = knob >= 0 ? knob : (groups <= 2LL * cus ? 1 : 0);
     }
     if (p.splits > 1 && !viaWork && beta != 1.f) {
         /* float pieces that add to c: c is dense, count matrices of M x N, strideC apart */
@@ -872,7 +889,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
         snprintf(g_plan, sizeof(g_plan), "%s%s%s tile=%s%s layout=%c%c fetch=%s splits=%d%s%s%s%s%s%s",
                  pre, pre[0] ? "+" : "", family,
                  family[9] == 'p' && p.persistRows == 128 ? "128x256" : tiles[tileCfg],
-                 family[9] == 'p' ? ",walk" : "",
+                 family[9] == 'p' ? ",walk" : (family[9] == 'd' && tileCfg == CFG_64x64 && p.f16Slab64 ? ",slab64" : ""),
                  s.aKContig ? 'N' : 'T', s.bKContig ? 'T' : 'N', fetch, p.splits,
                  p.splits > 1 ? (viaWork ? "+split_reduce_kernel" : ",atomic") : "",
                  p.colSum != NULL ? " colsum=in-kernel" : "",

@@ -18,7 +18,7 @@ F32, F16 = nt.X_FLOAT, nt.X_FLOAT16
 def planning():
     nt.load()
     for knob in ("NTSAMD_TILE_CFG", "NTSAMD_SPLIT_K", "NTSAMD_F16_FETCH", "NTSAMD_F16_PERSIST", "NTSAMD_F16_REPITCH",
-                 "NTSAMD_A32_CONVERT", "NTSAMD_F32_SPLIT_ATOMIC"):
+                 "NTSAMD_A32_CONVERT", "NTSAMD_F32_SPLIT_ATOMIC", "NTSAMD_F16_SLAB64"):
         nt.tuning_set(knob, None)
     nt.plan_only(True)
     yield nt.load()
@@ -67,6 +67,13 @@ def test_plans_name_the_passes_around_the_product(planning):
     # a long product with a float a: rounded once, then all half
     rc, plan = plan_mm(L, 8192, 4096, 1024, X_NOTRANS, X_NOTRANS, (F32, F16, F16))
     assert rc == 0 and plan.startswith("convert_kernel(a to half)+gemm_f16_persistent_kernel")
+    # few tiles of the small half shape: slabs of 64 along k; four workgroups to a CU: slabs of 32
+    rc, plan = plan_mm(L, 1024, 1024, 4096, X_NOTRANS, X_TRANS, (F16, F16, F16))
+    assert rc == 0 and plan.startswith("gemm_f16_direct_kernel tile=64x64,slab64 ")
+    nt.tuning_set("NTSAMD_TILE_CFG", 1)
+    rc, plan = plan_mm(L, 4096, 1024, 512, X_NOTRANS, X_TRANS, (F16, F16, F16))
+    assert rc == 0 and plan.startswith("gemm_f16_direct_kernel tile=64x64 ")
+    nt.tuning_set("NTSAMD_TILE_CFG", None)
     # a short one: rounded where it is fetched
     rc, plan = plan_mm(L, 128, 64, 128, X_NOTRANS, X_NOTRANS, (F32, F16, F16))
     assert rc == 0 and plan == "gemm_f16_kernel tile=64x64 layout=NN fetch=staged16,a float splits=1"

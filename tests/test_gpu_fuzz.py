@@ -26,6 +26,7 @@ KNOBS = {
     "NTSAMD_F32_R16": (None, None, 0),
     "NTSAMD_STORE_HINT": (None, None, 0, 1),
     "NTSAMD_GROUP_M": (None, None, 1, 3),
+    "NTSAMD_F16_SLAB64": (None, None, 0, 1),
 }
 
 

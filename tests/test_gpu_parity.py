@@ -179,9 +179,11 @@ def test_fp32_against_oracle(gpu, oracle, ta, tb):
 @pytest.mark.parametrize("ta,tb", TRANS)
 def test_fp16_against_oracle(gpu, oracle, ta, tb):
     torch = torch_()
-    # 128 x 128, 64 x 64, 256 x 256 (eight waves up to k = 2048, four beyond: the last shape)
-    for cfg in ("0", "1", "2"):
+    # 128 x 128, 64 x 64 with slabs of 32 and of 64 along k, 256 x 256 (eight waves up to k = 2048, four beyond: the
+    # last shape)
+    for cfg, slab64 in (("0", None), ("1", "0"), ("1", "1"), ("2", None)):
         nt.tuning_set("NTSAMD_TILE_CFG", cfg)
+        nt.tuning_set("NTSAMD_F16_SLAB64", slab64)
         for i, (M, N, K) in enumerate(SHAPES + [(264, 520, 2304)]):
             # round the inputs to half first; the oracle then runs in fp32 on those values
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 4000 + i, 0, 0.5)))
@@ -191,7 +193,8 @@ def test_fp16_against_oracle(gpu, oracle, ta, tb):
                 ref = oracle.matmul2d(a, ta, b, tb, c0.copy(), alpha, beta)
                 c = dev_tensor(c0, gpu, True) if beta != 0 else torch.full((M, N), float("nan"), device=gpu).half()
                 nt.matrix_mul(dev_tensor(a, gpu, True), ta, dev_tensor(b, gpu, True), tb, c, alpha, beta)
-                assert_fp16(c.float().cpu().numpy(), ref, what="cfg%s %dx%dx%d alpha=%g beta=%g" % (cfg, M, N, K, alpha, beta))
+                assert_fp16(c.float().cpu().numpy(), ref, what="cfg%s slab64=%s %dx%dx%d alpha=%g beta=%g" % (cfg, slab64, M, N, K, alpha, beta))
+    nt.tuning_set("NTSAMD_F16_SLAB64", None)
 
 
 @pytest.mark.parametrize("ta,tb", TRANS)
@@ -204,8 +207,8 @@ def test_half_products_cut_along_k(gpu, oracle, ta, tb):
     # 51 columns: rows of c that the adding kernel cannot take four elements at a time (cut only where b is stored
     # n x k: the 16-byte path needs whole 16-byte pieces along the rows of b)
     shapes = [(8, 8, 264), (72, 136, 1000), (40, 51, 1024), (200, 24, 4096), (16, 512, 2048), (256, 256, 2304)]
-    for cfg, pieces in ((None, None), ("0", "2"), ("0", "16"), ("1", "2"), ("1", "16")):
-        for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces)):
+    for cfg, pieces, slab64 in ((None, None, None), ("0", "2", None), ("0", "16", None), ("1", "2", "1"), ("1", "16", "1"), ("1", "2", "0"), ("1", "16", "0")):
+        for key, val in (("NTSAMD_TILE_CFG", cfg), ("NTSAMD_SPLIT_K", pieces), ("NTSAMD_F16_SLAB64", slab64)):
             nt.tuning_set(key, val)
         for i, (M, N, K) in enumerate(shapes if cfg else shapes[-2:]):
             a = oracle.from_f16_bits(oracle.to_f16_bits(oracle.normal(stored((M, K), ta), 8000 + i, 0, 0.5)))
