@@ -120,31 +120,53 @@ int launch_scale(bool half, void * v, long long n, float beta, hipStream_t strea
 /* c[row][col] = f(c[row][col] + bias[(row / div) % len]): the broadcast add along a dimension that is not the last,
    as a pass of its own behind the product, which is how the reference does it (_SumDim with KernelAddWithCol,
    source/tensor/core/arithmetic/SumDim.cu:79-105, called from MulAndShift.cpp:88); f is the activation */
-template <typename T>
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
-row_bias_kernel(T * __restrict__ c, long long total, int N, int ldc, const T * __restrict__ bias, int div, int len, int act)
+row_bias_kernel(T * __restrict__ c, int M, int colsV, int ldc, const T * __restrict__ bias, int div, int len, int act)
 {
-    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total)
+    /* a block is 64 pieces of VEC columns by 4 rows; rows beyond what the grid's second dimension holds are
+       reached by striding */
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
+    const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+    if (col >= colsV)
         return;
-    const long long row = i / N;
-    const int col = (int)(i - row * N);
-    T * at = c + row * ldc + col;
-    *at = (T)activate((float)*at + (float)bias[(row / div) % len], act);
+    for (int row = blockIdx.y * 4 + (threadIdx.x >> 6); row < M; row += gridDim.y * 4) {
+        const float bv = (float)bias[(row / div) % len];
+        T * at = c + (long long)row * ldc + col * VEC;
+        if constexpr (VEC == 1)
+            *at = (T)activate((float)*at + bv, act);
+        else {
+            vec_t v = *reinterpret_cast<const vec_t *>(at);
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+                v[e] = (T)activate((float)v[e] + bv, act);
+            *reinterpret_cast<vec_t *>(at) = v;
+        }
+    }
+}
+
+template <typename T>
+static void launch_row_bias_t(T * c, int M, int N, int ldc, const T * bias, int div, int len, int act, hipStream_t stream)
+{
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const bool wide = N % VEC == 0 && ldc % VEC == 0 && (reinterpret_cast<uintptr_t>(c) & 15) == 0;
+    const int colsV = wide ? N / VEC : N;
+    const int rowBlocks = (M + 3) / 4;
+    dim3 grid((unsigned)((colsV + 63) / 64), (unsigned)(rowBlocks < 65535 ? rowBlocks : 65535));
+    if (wide)
+        hipLaunchKernelGGL((row_bias_kernel<T, VEC>), grid, dim3(256), 0, stream, c, M, colsV, ldc, bias, div, len, act);
+    else
+        hipLaunchKernelGGL((row_bias_kernel<T, 1>), grid, dim3(256), 0, stream, c, M, colsV, ldc, bias, div, len, act);
 }
 
 int launch_row_bias(bool half, void * c, int M, int N, int ldc, const void * bias, int div, int len, int act, hipStream_t stream)
 {
-    const long long total = (long long)M * N;
-    if (total <= 0)
+    if (M <= 0 || N <= 0)
         return 0;
-    dim3 grid((unsigned)((total + 255) / 256));
     if (half)
-        hipLaunchKernelGGL(row_bias_kernel<half_t>, grid, dim3(256), 0, stream, static_cast<half_t *>(c), total, N, ldc,
-                           static_cast<const half_t *>(bias), div, len, act);
+        launch_row_bias_t(static_cast<half_t *>(c), M, N, ldc, static_cast<const half_t *>(bias), div, len, act, stream);
     else
-        hipLaunchKernelGGL(row_bias_kernel<float>, grid, dim3(256), 0, stream, static_cast<float *>(c), total, N, ldc,
-                           static_cast<const float *>(bias), div, len, act);
+        launch_row_bias_t(static_cast<float *>(c), M, N, ldc, static_cast<const float *>(bias), div, len, act, stream);
     return (int)hipGetLastError();
 }
 
