@@ -549,18 +549,19 @@ def cpu_baseline(idx, budget_s=12.0):
 
 
 def measured_traffic(idx):
-    """HBM-side bytes per step from the committed rocprofv3 counter runs: the table in
-    profiles/hbm_traffic_per_step.md (rows "| configuration | bytes |"), or None."""
+    """HBM-side bytes per step from the committed rocprofv3 counter runs and what the library launched when they
+    were read: the row of this configuration in profiles/hbm_traffic_per_step.md
+    ("| configuration | bytes | algorithmic bytes | plans |"), or (None, None)."""
     import re
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic_per_step.md")) as f:
             for line in f:
-                m = re.match(r"\|\s*(\d+)\s*\|\s*(\d+)\s*\|", line)
+                m = re.match(r"\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*\d+\s*\|\s*(.*?)\s*\|\s*$", line)
                 if m and int(m.group(1)) == idx:
-                    return int(m.group(2))
+                    return int(m.group(2)), m.group(3)
     except OSError:
         pass
-    return None
+    return None, None
 
 
 def graph_replayed(wl, dev, ev, steps_in_graph=50, replays=20):
@@ -738,10 +739,18 @@ def bench_one(idx, steps, warmup, dev, oracle, with_cpu, cpu_budget_s=12.0, rota
     # beside it.
     roof = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
             "frac": round(achieved / peak, 4)}
-    traffic = measured_traffic(idx)
+    traffic, taken_with = measured_traffic(idx)
+    source = None
+    if traffic is not None:
+        if kernels is not None and taken_with != " ; ".join(kernels):
+            source = ("stale: the committed table's counters were read when the library launched [%s]; it now launches [%s]"
+                      % (taken_with, " ; ".join(kernels)))
+            traffic = None
+        else:
+            source = ("committed rocprofv3 FETCH_SIZE/WRITE_SIZE table (profiles/hbm_traffic_per_step.md), read with the "
+                      "kernels this run launched, not measured in this run")
     roof.update({"traffic": traffic,
-                 "traffic_source": None if traffic is None else
-                 "committed rocprofv3 FETCH_SIZE/WRITE_SIZE table (profiles/hbm_traffic_per_step.md), not measured in this run",
+                 "traffic_source": source,
                  "kernel_us": round(kt / wl.launches * 1e6, 2),
                  "kernel_us_best": round(kt_best / wl.launches * 1e6, 2),
                  "hbm_frac": round(wl.bytes / kt / 1e12 / HBM_TBS, 4),

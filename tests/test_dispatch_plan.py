@@ -127,3 +127,18 @@ def test_no_product_the_16_byte_routes_accept_goes_element_wise(planning):
     assert rc == 0 and "fetch=vec16" in plan and "+row_bias_kernel" in plan
     rc, plan = plan_mm(L, 4, 1 << 21, 8, X_NOTRANS, X_NOTRANS)
     assert rc == 0 and "fetch=elementwise" in plan
+
+
+def test_the_traffic_table_was_read_with_todays_kernels(planning):
+    """profiles/hbm_traffic_per_step.md names, per configuration, what the library launched when its counters were
+    read; bench.py reports a row as stale when that differs from what it launches. Here, without a GPU: the rows of
+    the baseline's single products still name what the dispatcher plans for them."""
+    import bench
+    L = planning
+    for idx, args, kw in ((1, (4096, 2048, 512, X_NOTRANS, X_NOTRANS), {}),
+                          (2, (4096, 2048, 512, X_NOTRANS, X_NOTRANS), {"bias": 0x400000}),
+                          (4, (8192, 4096, 1024, X_TRANS, X_NOTRANS, (F16, F16, F16)), {}),
+                          (5, (4096, 30011, 512, X_NOTRANS, X_TRANS), {"beta": 1.0})):
+        rc, plan = plan_mm(L, *args, **kw)
+        traffic, taken_with = bench.measured_traffic(idx)
+        assert rc == 0 and traffic and taken_with == plan, (idx, plan, taken_with)
