@@ -832,6 +832,9 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             return fail(NTSAMD_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
     if (colSum != NULL) {
+        /* (Float: the workgroups of the first tile row gather the sums from their b fragments and run about a fifth
+           longer for it, 66.4 -> 77.9 us at 512 x 2048 over 4096 rows; a pass of its own over b before the product
+           was measured against that: two launches more, 76.8 us, and b once more from memory. The by-product stays.) */
         if (vec && count == 1 && !(p.splits > 1 && viaWork)) {
             /* by-product of the product kernel */
             p.colSum = colSum;
@@ -845,7 +848,7 @@ int run(int devID, void * stream, Kind kind, const Shape & s,
             /* a pass of its own over b: rows of k for X_NOTRANS, rows of n for X_TRANS. It runs before the product
                on the same stream, so the two can share the workspace. It reads b as the caller stored it (dense
                rows), never the re-pitched copy the product may have been given. */
-            if (!half && !s.bKContig && !noAlloc && !repitched)
+            if (!s.bKContig && !noAlloc && !repitched)
                 work.take_stream(devID, hs);
             note(s.bKContig ? "outer_inner_sum_kernel(b)" : "column_sum_kernel(b)");
             float * const sumWork = repitched ? NULL : work.mem;
@@ -1122,7 +1125,7 @@ int ntsamd_matrix_mul_colsum(int devID, void * stream,
             return scope.status;
         hipStream_t hs = static_cast<hipStream_t>(stream);
         WorkHold work;
-        if (kind == KIND_F32 && !s.bKContig && s.K >= 128)
+        if (!s.bKContig && s.K >= 128)
             work.take_stream(devID, hs);
         int rc = s.bKContig ? launch_reduce_sum_xz(kind != KIND_F32, b, 1, s.N, s.K, colSum, colSumBeta, hs, NULL, 0)
                             : launch_reduce_sum_xz(kind != KIND_F32, b, s.K, s.N, 1, colSum, colSumBeta, hs,
@@ -1154,9 +1157,9 @@ int ntsamd_reduce_sum_xz(int devID, void * stream, const void * in, int dataType
     DeviceScope scope(devID);
     if (scope.status != NTSAMD_OK)
         return scope.status;
-    /* float column sums over many rows are cut into pieces of the rows, which meet in the stream's workspace */
+    /* column sums over many rows are cut into pieces of the rows, which meet in the stream's workspace as fp32 */
     WorkHold work;
-    if (dataType == NTSAMD_X_FLOAT && z == 1 && x >= 128)
+    if (z == 1 && x >= 128)
         work.take_stream(devID, static_cast<hipStream_t>(stream));
     snprintf(g_plan, sizeof(g_plan), "%s", z > 1 ? "outer_inner_sum_kernel" : "column_sum_kernel");
     int rc = launch_reduce_sum_xz(dataType == NTSAMD_X_FLOAT16, in, x, y, z > 0 ? z : 1, out, beta,

@@ -22,7 +22,8 @@ namespace ntsamd {
    read 4 columns each (256 contiguous bytes of a row for fp32), 16 such rows per step. */
 enum { SUM_WHOLE = 0, SUM_ATOMIC = 1, SUM_PIECE = 2 };   /* what a workgroup does with its sums */
 
-template <typename T, int MODE>
+/* WIDE: rows are whole groups of four columns and start on 4-column boundaries of memory (one load per thread and row) */
+template <typename T, int MODE, bool WIDE = false>
 __global__ void __launch_bounds__(256)
 column_sum_kernel(const T * __restrict__ in, int X, int Y, int rowsPerPiece, T * __restrict__ out, float beta)
 {
@@ -32,7 +33,17 @@ column_sum_kernel(const T * __restrict__ in, int X, int Y, int rowsPerPiece, T *
     const int xBeg = blockIdx.y * rowsPerPiece;
     const int xEnd = xBeg + rowsPerPiece < X ? xBeg + rowsPerPiece : X;
     float s[4] = {0.f, 0.f, 0.f, 0.f};
-    if (col0 + 3 < Y) {
+    if (WIDE && col0 + 3 < Y) {
+        typedef T vec_t __attribute__((ext_vector_type(4)));
+#pragma unroll 4
+        for (int x = xBeg + rl; x < xEnd; x += 16) {
+            const vec_t v = *reinterpret_cast<const vec_t *>(in + (size_t)x * Y + col0);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                s[e] += (float)v[e];
+        }
+    }
+    else if (col0 + 3 < Y) {
 #pragma unroll 4
         for (int x = xBeg + rl; x < xEnd; x += 16) {
             const T * rp = in + (size_t)x * Y + col0;
@@ -187,30 +198,32 @@ int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void *
         return (int)hipGetLastError();
     }
     const int colGroups = (Y + 63) / 64;
-    if (half) {
-        /* one piece: half sums are rounded once, from the fp32 total */
-        hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_WHOLE>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
-                           static_cast<const half_t *>(in), X, Y, X > 0 ? X : 1, static_cast<half_t *>(out), beta);
-        return (int)hipGetLastError();
-    }
     /* enough pieces to give every CU a few workgroups, at least 64 rows each */
     int pieces = (1024 + colGroups - 1) / colGroups;
     if (pieces > (X + 63) / 64)
         pieces = (X + 63) / 64;
-    if (pieces <= 1) {
-        hipLaunchKernelGGL((column_sum_kernel<float, SUM_WHOLE>), dim3((unsigned)colGroups, 1), dim3(256), 0, stream,
-                           static_cast<const float *>(in), X, Y, X > 0 ? X : 1, static_cast<float *>(out), beta);
-        return (int)hipGetLastError();
-    }
-    if (work != NULL && (size_t)Y * 2 <= workFloats) {
-        /* the pieces meet in the workspace and are added in their order */
+    const bool wide = Y % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & (half ? 7 : 15)) == 0;
+    if (work != NULL && pieces > 1 && (size_t)Y * 2 <= workFloats) {
+        /* the pieces meet in the workspace as fp32 and are added in their order; a half result is rounded once,
+           from the fp32 total */
         const int most = (size_t)Y * 16 <= workFloats ? 16 : (int)(workFloats / (size_t)Y);
         if (pieces > most)
             pieces = most;
         const int rows = (X + pieces - 1) / pieces;
         pieces = (X + rows - 1) / rows;
-        hipLaunchKernelGGL((column_sum_kernel<float, SUM_PIECE>), dim3((unsigned)colGroups, (unsigned)pieces), dim3(256), 0,
-                           stream, static_cast<const float *>(in), X, Y, rows, reinterpret_cast<float *>(work), 1.f);
+        const dim3 grid((unsigned)colGroups, (unsigned)pieces);
+        if (half && wide)
+            hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_PIECE, true>), grid, dim3(256), 0, stream,
+                               static_cast<const half_t *>(in), X, Y, rows, reinterpret_cast<half_t *>(work), 1.f);
+        else if (half)
+            hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_PIECE>), grid, dim3(256), 0, stream,
+                               static_cast<const half_t *>(in), X, Y, rows, reinterpret_cast<half_t *>(work), 1.f);
+        else if (wide)
+            hipLaunchKernelGGL((column_sum_kernel<float, SUM_PIECE, true>), grid, dim3(256), 0, stream,
+                               static_cast<const float *>(in), X, Y, rows, reinterpret_cast<float *>(work), 1.f);
+        else
+            hipLaunchKernelGGL((column_sum_kernel<float, SUM_PIECE>), grid, dim3(256), 0, stream,
+                               static_cast<const float *>(in), X, Y, rows, reinterpret_cast<float *>(work), 1.f);
         int rc = (int)hipGetLastError();
         if (rc != 0)
             return rc;
@@ -224,7 +237,24 @@ int launch_reduce_sum_xz(bool half, const void * in, int X, int Y, int Z, void *
         p.beta = beta;
         p.splits = pieces;
         p.splitWork = work;
-        return launch_split_reduce(p, true, stream);
+        return launch_split_reduce(p, !half, stream);
+    }
+    if (half || pieces <= 1) {
+        /* one piece (half without a workspace: the sums are rounded once, from the fp32 total) */
+        const dim3 grid((unsigned)colGroups, 1);
+        if (half && wide)
+            hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_WHOLE, true>), grid, dim3(256), 0, stream,
+                               static_cast<const half_t *>(in), X, Y, X > 0 ? X : 1, static_cast<half_t *>(out), beta);
+        else if (half)
+            hipLaunchKernelGGL((column_sum_kernel<half_t, SUM_WHOLE>), grid, dim3(256), 0, stream,
+                               static_cast<const half_t *>(in), X, Y, X > 0 ? X : 1, static_cast<half_t *>(out), beta);
+        else if (wide)
+            hipLaunchKernelGGL((column_sum_kernel<float, SUM_WHOLE, true>), grid, dim3(256), 0, stream,
+                               static_cast<const float *>(in), X, Y, X > 0 ? X : 1, static_cast<float *>(out), beta);
+        else
+            hipLaunchKernelGGL((column_sum_kernel<float, SUM_WHOLE>), grid, dim3(256), 0, stream,
+                               static_cast<const float *>(in), X, Y, X > 0 ? X : 1, static_cast<float *>(out), beta);
+        return (int)hipGetLastError();
     }
     int rc = launch_scale(false, out, Y, beta, stream);
     if (rc != 0)
