@@ -177,10 +177,14 @@ bool aligned16(const void * p)
    a workgroup spends before its first and after its last MFMA (4 us; 1.5 us for the small tile) is exposed
    once and partly hidden behind the other workgroups of the CU after that. Cutting k sends the fp32 partial
    products across memory once (about 5 TB/s, much of it behind the multiplications) on their way to a second
-   launch (2.3 us) that adds them up in a fixed order. Without a workspace the pieces add to c with atomics
+   launch that adds them up in a fixed order. The constants of the 16-row shape (0.55 of the rate, 1 us of ends) and of the
+   cut (4.5 us) are those of a second fit, over 102 products from 64 x 512 x 512 to
+   2048 x 2048 x 2048 with every shape and 1 to 16 pieces measured: the plan they choose is within 3.5 % of the best
+   measured plan on every one of them (the first fit's: 24 % off on the worst, small products that it cut into
+   pieces where the 16-row shape in one piece is faster). Without a workspace the pieces add to c with atomics
    instead (about 2.7 TB/s) and, unless beta is 1, a pass over c applies beta first: a launch (2.5 us) and c
    read and written. */
-constexpr double SPLIT_FIXED_US = 2.3, SPLIT_BYTES_PER_US = 5.0e6;
+constexpr double SPLIT_FIXED_US = 2.3, SPLIT_FIXED_F32_US = 4.5, SPLIT_BYTES_PER_US = 5.0e6;
 
 double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits, bool betaPass, bool viaWork)
 {
@@ -189,14 +193,14 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     const long long rounds = (groups + 255) / 256;
     /* 16 rows per workgroup: every workgroup stages 128 columns of b for 16 rows of c, twice what the others move
        per MFMA (measured: 0.7 of the rate, and a longer start) */
-    const double rate = big ? 1.0 : (bm == 16 ? 0.7 : (rounds > 1 ? 0.965 : 0.89));
+    const double rate = big ? 1.0 : (bm == 16 ? 0.55 : (rounds > 1 ? 0.965 : 0.89));
     /* the 32-row tile multiplies only 16 rows when there are no more (16-row MFMAs) */
     const double mfma = (double)(bm == 32 && M <= 16 ? 16 : bm) * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
-    const double ends = (big ? 4.0 : (bm == 16 ? 2.5 : 1.5)) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
+    const double ends = (big ? 4.0 : (bm == 16 ? 1.0 : 1.5)) * (1.0 + (double)(rounds - 1) * (big ? 0.5 : 0.25));
     const double cBytes = 4.0 * M * N * count;
     double cut = 0.0;
     if (splits > 1 && viaWork)
-        cut = SPLIT_FIXED_US + 2.0 * cBytes * splits / SPLIT_BYTES_PER_US;
+        cut = SPLIT_FIXED_F32_US + 2.0 * cBytes * splits / SPLIT_BYTES_PER_US;
     else if (splits > 1)
         cut = cBytes * splits / 2.7e6 + (betaPass ? 2.5 + cBytes * 2 / 2.7e6 : 0.0);
     return (double)rounds * mfma + ends + cut;
