@@ -685,6 +685,30 @@ def test_fused_bias(gpu, oracle, half):
 
 
 @pytest.mark.parametrize("half", (False, True))
+def test_bias_by_row_on_many_rows_and_odd_columns(gpu, oracle, half):
+    """The pass that adds a bias by row behind the product: more rows than its grid holds in one sweep (it strides),
+    columns that are no whole 16-byte pieces (element by element), a row group of 3 and a rectifier; against float64."""
+    torch = torch_()
+    dt = torch.float16 if half else torch.float32
+    for M, N, K, div in ((300000, 8, 8, 3), (1000, 37, 16, 1), (4100, 72, 24, 7)):
+        g = torch.Generator(device="cpu").manual_seed(M + N)
+        a = torch.randn(M, K, generator=g).to(dt).to(gpu)
+        b = torch.randn(K, N, generator=g).to(dt).to(gpu)
+        length = (M + div - 1) // div
+        bias = torch.randn(length, generator=g).to(dt).to(gpu)
+        c = torch.full((M, N), float("nan"), device=gpu, dtype=dt)
+        nt.matrix_mul(a, X_NOTRANS, b, X_NOTRANS, c, 1.0, 0.0, bias=bias, bias_mode=BIAS_ROW, bias_row_div=div, act=nt.ACT_RECTIFY)
+        assert "+row_bias_kernel" in nt.last_plan()
+        rows = torch.arange(M, device=gpu) // div
+        prod = a.double() @ b.double()
+        if half:
+            prod = prod.half().double()          # the product is rounded before the bias is added, as in the reference
+        ref = (prod + bias.double()[rows][:, None]).clamp(min=0)
+        err = float((c.double() - ref).abs().max() / ref.abs().max())
+        assert err <= (2e-3 if half else 1e-5), (M, N, K, div, err)
+
+
+@pytest.mark.parametrize("half", (False, True))
 def test_fused_bias_and_rectify(gpu, oracle, half):
     """Rectify(MulAndShift(x, w, b)) in the epilogue (the first step of the reference's feed-forward block):
     against the oracle's product + broadcast add + rectify, on the main path and on the generic one
