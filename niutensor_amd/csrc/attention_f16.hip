@@ -17,10 +17,10 @@
  *   S^T = K Q^T   v_mfma_f32_16x16x32_f16: lane (m, g) = (l%16, l/16) feeds key m / query m with the
  *                 eight columns 32 t + 8 g .. + 7 (one 16-byte read) and receives the scores of query m
  *                 against keys 16 j + 4 g + r, r = 0..3.
- *   O^T = V^T P^T v_mfma_f32_16x16x16_f16: B wants four consecutive k per lane, k = 4 g + r: the four
- *                 scores above, rounded to half. A wants V[key 16 j + 4 g + r][column m], four values
- *                 one LDS row apart: a transposing read (ds_read_b64_tr_b16) of the 4 x 16 block whose
- *                 rows the lane groups 0-3, 4-7, 8-11, 12-15 of every 16 lanes point at.
+ *   O^T = V^T P^T v_mfma_f32_16x16x32_f16 over pairs of 16-key blocks: B wants eight k per lane: the four
+ *                 scores above of either block, rounded to half. A wants V[key 16 j + 4 g + r][column m],
+ *                 four values one LDS row apart per block: a transposing read (ds_read_b64_tr_b16) of the
+ *                 4 x 16 block whose rows the lane groups 0-3, 4-7, 8-11, 12-15 of every 16 lanes point at.
  */
 #include "gemm_common.h"
 #include "gemm_f16.h"       /* half_t, make_rsrc, buffer_load_f16x8, lds_read_tr16 */
@@ -223,13 +223,19 @@ attention_f16_kernel(const AttnParams p)
         if (more)
             load_v(kb0 + KB);
 
-        /* ---- O^T += V^T P^T ---- */
+        /* ---- O^T += V^T P^T, 32 keys per MFMA: the k index 8 g + e of v_mfma_f32_16x16x32_f16 stands for key
+           4 g + e of the first 16-key block of a pair for e < 4 and for key 4 g + e - 4 of the second for e >= 4 (the
+           order in which a sum runs over the keys is free), so a lane's operands are its two blocks' four
+           probabilities and two transposing reads side by side. (The 16x16x16 form runs at half the rate.) ---- */
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
+        for (int j = 0; j < NJ; j += 2)
 #pragma unroll
             for (int d = 0; d < ND; d++) {
-                const f16x4 vf = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * j * PITCH + trOff + 32 * d]));
-                accO[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf[j], accO[d], 0, 0, 0);
+                const f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * j * PITCH + trOff + 32 * d]));
+                const f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * (j + 1) * PITCH + trOff + 32 * d]));
+                const f16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                const f16x8 pp = __builtin_shufflevector(pf[j], pf[j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                accO[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pp, accO[d], 0, 0, 0);
             }
     }
 
