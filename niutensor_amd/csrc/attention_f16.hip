@@ -40,12 +40,18 @@ __device__ __forceinline__ float groups_sum(float x)
     return x + __shfl_xor(x, 32);
 }
 
-/* DHM: head size the kernel is built for (dh <= DHM, a multiple of 8; columns past dh are zero) */
-template <int DHM>
-__global__ void __launch_bounds__(256, 2)
+/* DHM: head size the kernel is built for (dh <= DHM, a multiple of 8; columns past dh are zero).
+   QR: blocks of 16 query rows per wave. With two, a key or value fragment that a wave reads from LDS feeds two MFMAs
+   instead of one: every wave of a workgroup reads every key and every value of a block, and at long sequences those
+   reads, not the matrix pipe, are what the kernel waits for (LDS busy 53 % of the kernel's cycles with one block per
+   wave). A workgroup then takes 128 query rows, so short sequences, which need the workgroups, keep one block.
+   Two blocks of query rows go with blocks of 64 keys: scores and probabilities of 2 x 128 keys at once spilled 37
+   registers and ran slower than one block of rows; with 64 keys the kernel fits 168 registers, three waves to a SIMD. */
+template <int DHM, int QR>
+__global__ void __launch_bounds__(256, QR == 2 ? 3 : 2)
 attention_f16_kernel(const AttnParams p)
 {
-    constexpr int KB = 128;                  /* keys per block */
+    constexpr int KB = QR == 2 ? 64 : 128;   /* keys per block in LDS */
     constexpr int PITCH = DHM * 2 + 16;      /* bytes per LDS row: 16 mod 128, so 16-byte reads of consecutive rows
                                                 walk through the banks */
     constexpr int NT = DHM / 32;             /* k steps of the first product */
@@ -74,9 +80,16 @@ attention_f16_kernel(const AttnParams p)
     const half_t * V = static_cast<const half_t *>(p.v) + h * p.vH + b * p.vB;
     half_t * O = static_cast<half_t *>(p.out) + h * p.oH + b * p.oB;
 
-    const int row = qt * 64 + wave * 16 + m;
-    const int rowc = row < lq ? row : lq - 1;
-    const float * MK = p.mask ? p.mask + ((long long)pair * lq + rowc) * lk : nullptr;
+    /* this lane's query rows, one per block of 16 */
+    int row[QR];
+    const float * MK[QR];
+#pragma unroll
+    for (int q = 0; q < QR; q++) {
+        row[q] = qt * (64 * QR) + wave * (16 * QR) + 16 * q + m;
+        const int rowc = row[q] < lq ? row[q] : lq - 1;
+        MK[q] = p.mask ? p.mask + ((long long)pair * lq + rowc) * lk : nullptr;
+    }
+    const bool masked = p.mask != nullptr;
 
     /* ---- staging of keys and values, as in the fp32 kernel ---- */
     const int sr0 = tid / TPR, sc = (tid % TPR) * 8;
@@ -99,22 +112,28 @@ attention_f16_kernel(const AttnParams p)
     load_k(0);
 
     /* ---- Q fragments ---- */
-    f16x8 qf[NT];
-    {
-        const half_t * qr = Q + (long long)rowc * p.qL;
+    f16x8 qf[QR][NT];
+#pragma unroll
+    for (int q = 0; q < QR; q++) {
+        const half_t * qr = Q + (long long)(row[q] < lq ? row[q] : lq - 1) * p.qL;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const int c = 32 * t + 8 * g;
             f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-            qf[t] = c < dh ? *reinterpret_cast<const f16x8 *>(qr + c) : z;
+            qf[q][t] = c < dh ? *reinterpret_cast<const f16x8 *>(qr + c) : z;
         }
     }
 
-    f32x4 accO[ND];
+    f32x4 accO[QR][ND];
+    float rowMax[QR], rowSum[QR];
 #pragma unroll
-    for (int d = 0; d < ND; d++)
-        accO[d] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float rowMax = -INFINITY, rowSum = 0.f;
+    for (int q = 0; q < QR; q++) {
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+            accO[q][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+        rowMax[q] = -INFINITY;
+        rowSum[q] = 0.f;
+    }
     const float scale2 = p.scale * LOG2E;
 
     /* where this lane points for the transposing reads: row 4 g + (m / 4) of a 16-key block, columns 4 (m % 4) .. + 3 */
@@ -134,87 +153,94 @@ attention_f16_kernel(const AttnParams p)
         if (more)
             load_k(kb0 + KB);
 
-        /* ---- S^T = K Q^T ---- */
-        f32x4 accS[NJ];
+        /* ---- S^T = K Q^T: a key fragment feeds the products of all of the lane's query rows ---- */
+        f32x4 accS[QR][NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-            accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < QR; q++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+                accS[q][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < NT; t++) {
 #pragma unroll
             for (int j = 0; j < NJ; j++) {
                 const f16x8 kf = *reinterpret_cast<const f16x8 *>(&Ks[(16 * j + m) * PITCH + 64 * t + 16 * g]);
-                accS[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t], accS[j], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < QR; q++)
+                    accS[q][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[q][t], accS[q][j], 0, 0, 0);
             }
         }
 
-        /* ---- scale and mask ---- */
-        if (MK != nullptr) {
-            if (p.maskVec) {
+        f16x4 pf[QR][NJ];                                /* the probabilities as the second product's operand */
 #pragma unroll
-                for (int j = 0; j < NJ; j++) {
-                    const int key = kb0 + 16 * j + 4 * g;
-                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK + key) : z;
+        for (int q = 0; q < QR; q++) {
+            /* ---- scale and mask ---- */
+            if (masked) {
+                if (p.maskVec) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        accS[j][r] = fmaf(mk[r], LOG2E, accS[j][r] * scale2);
+                    for (int j = 0; j < NJ; j++) {
+                        const int key = kb0 + 16 * j + 4 * g;
+                        f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                        const f32x4 mk = key < lk ? *reinterpret_cast<const f32x4 *>(MK[q] + key) : z;
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            accS[q][j][r] = fmaf(mk[r], LOG2E, accS[q][j][r] * scale2);
+                    }
+                }
+                else {
+#pragma unroll
+                    for (int j = 0; j < NJ; j++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            int key = kb0 + 16 * j + 4 * g + r;
+                            key = key < lk ? key : lk - 1;
+                            accS[q][j][r] = fmaf(MK[q][key], LOG2E, accS[q][j][r] * scale2);
+                        }
                 }
             }
             else {
 #pragma unroll
                 for (int j = 0; j < NJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        int key = kb0 + 16 * j + 4 * g + r;
-                        key = key < lk ? key : lk - 1;
-                        accS[j][r] = fmaf(MK[key], LOG2E, accS[j][r] * scale2);
-                    }
+                    for (int r = 0; r < 4; r++)
+                        accS[q][j][r] *= scale2;
             }
-        }
-        else {
+            if (kb0 + KB > lk) {
 #pragma unroll
-            for (int j = 0; j < NJ; j++)
+                for (int j = 0; j < NJ; j++)
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    accS[j][r] *= scale2;
-        }
-        if (kb0 + KB > lk) {
-#pragma unroll
-            for (int j = 0; j < NJ; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (kb0 + 16 * j + 4 * g + r >= lk)
-                        accS[j][r] = -INFINITY;
-        }
+                    for (int r = 0; r < 4; r++)
+                        if (kb0 + 16 * j + 4 * g + r >= lk)
+                            accS[q][j][r] = -INFINITY;
+            }
 
-        /* ---- running softmax of this lane's query row, in fp32 ---- */
-        float mx = accS[0][0];
+            /* ---- running softmax of this lane's query row, in fp32 ---- */
+            float mx = accS[q][0][0];
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                mx = fmaxf(mx, accS[j][r]);
-        mx = groups_max(mx);
-        const float newMax = fmaxf(rowMax, mx);
-        const float shift = newMax == -INFINITY ? 0.f : newMax;
-        const float corr = __builtin_amdgcn_exp2f(rowMax - shift);
-        float sum = 0.f;
-        f16x4 pf[NJ];                                    /* the probabilities as the second product's operand */
+                for (int r = 0; r < 4; r++)
+                    mx = fmaxf(mx, accS[q][j][r]);
+            mx = groups_max(mx);
+            const float newMax = fmaxf(rowMax[q], mx);
+            const float shift = newMax == -INFINITY ? 0.f : newMax;
+            const float corr = __builtin_amdgcn_exp2f(rowMax[q] - shift);
+            float sum = 0.f;
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float e = __builtin_amdgcn_exp2f(accS[j][r] - shift);
-                sum += e;
-                pf[j][r] = (half_t)e;
-            }
-        sum = groups_sum(sum);
-        rowSum = rowSum * corr + sum;
-        rowMax = newMax;
+                for (int r = 0; r < 4; r++) {
+                    const float e = __builtin_amdgcn_exp2f(accS[q][j][r] - shift);
+                    sum += e;
+                    pf[q][j][r] = (half_t)e;
+                }
+            sum = groups_sum(sum);
+            rowSum[q] = rowSum[q] * corr + sum;
+            rowMax[q] = newMax;
 #pragma unroll
-        for (int d = 0; d < ND; d++)
-            accO[d] *= corr;
+            for (int d = 0; d < ND; d++)
+                accO[q][d] *= corr;
+        }
 
 #pragma unroll
         for (int s = 0; s < LOADS; s++)
@@ -226,7 +252,8 @@ attention_f16_kernel(const AttnParams p)
         /* ---- O^T += V^T P^T, 32 keys per MFMA: the k index 8 g + e of v_mfma_f32_16x16x32_f16 stands for key
            4 g + e of the first 16-key block of a pair for e < 4 and for key 4 g + e - 4 of the second for e >= 4 (the
            order in which a sum runs over the keys is free), so a lane's operands are its two blocks' four
-           probabilities and two transposing reads side by side. (The 16x16x16 form runs at half the rate.) ---- */
+           probabilities and two transposing reads side by side. (The 16x16x16 form runs at half the rate.) A
+           value fragment feeds the products of all of the lane's query rows. ---- */
 #pragma unroll
         for (int j = 0; j < NJ; j += 2)
 #pragma unroll
@@ -234,24 +261,30 @@ attention_f16_kernel(const AttnParams p)
                 const f16x4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * j * PITCH + trOff + 32 * d]));
                 const f16x4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(&Vs[16 * (j + 1) * PITCH + trOff + 32 * d]));
                 const f16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                const f16x8 pp = __builtin_shufflevector(pf[j], pf[j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                accO[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pp, accO[d], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < QR; q++) {
+                    const f16x8 pp = __builtin_shufflevector(pf[q][j], pf[q][j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    accO[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pp, accO[q][d], 0, 0, 0);
+                }
             }
     }
 
     /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
-    if (row < lq) {
-        const float inv = rowSum > 0.f ? 1.f / rowSum : 0.f;
-        half_t * orow = O + (long long)row * p.oL;
 #pragma unroll
-        for (int d = 0; d < ND; d++) {
-            const int c = 16 * d + 4 * g;
-            if (c < dh) {
-                f16x4 o;
+    for (int q = 0; q < QR; q++) {
+        if (row[q] < lq) {
+            const float inv = rowSum[q] > 0.f ? 1.f / rowSum[q] : 0.f;
+            half_t * orow = O + (long long)row[q] * p.oL;
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    o[r] = (half_t)(accO[d][r] * inv);
-                *reinterpret_cast<f16x4 *>(orow + c) = o;
+            for (int d = 0; d < ND; d++) {
+                const int c = 16 * d + 4 * g;
+                if (c < dh) {
+                    f16x4 o;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        o[r] = (half_t)(accO[q][d][r] * inv);
+                    *reinterpret_cast<f16x4 *>(orow + c) = o;
+                }
             }
         }
     }
@@ -260,15 +293,25 @@ attention_f16_kernel(const AttnParams p)
 int launch_attention_f16(const AttnParams & p0, hipStream_t stream)
 {
     AttnParams p = p0;
-    p.qTiles = (p.lq + 63) / 64;
     p.maskVec = (p.mask != nullptr && p.lk % 4 == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 15) == 0) ? 1 : 0;
+    /* 128 query rows per workgroup (two blocks of 16 per wave) where that still leaves two workgroups for every CU
+       of the part; heads of 128 keep one block (their registers) */
+    const long long groups128 = (long long)p.heads * p.batch * ((p.lq + 127) / 128);
+    const bool two = p.dh <= 64 && p.lq > 64 && groups128 >= 512;
+    p.qTiles = two ? (p.lq + 127) / 128 : (p.lq + 63) / 64;
     dim3 grid((unsigned)(p.heads * p.batch * p.qTiles));
-    if (p.dh <= 32)
-        hipLaunchKernelGGL((attention_f16_kernel<32>), grid, dim3(256), 0, stream, p);
+    if (two) {
+        if (p.dh <= 32)
+            hipLaunchKernelGGL((attention_f16_kernel<32, 2>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_f16_kernel<64, 2>), grid, dim3(256), 0, stream, p);
+    }
+    else if (p.dh <= 32)
+        hipLaunchKernelGGL((attention_f16_kernel<32, 1>), grid, dim3(256), 0, stream, p);
     else if (p.dh <= 64)
-        hipLaunchKernelGGL((attention_f16_kernel<64>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((attention_f16_kernel<64, 1>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((attention_f16_kernel<128>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((attention_f16_kernel<128, 1>), grid, dim3(256), 0, stream, p);
     return (int)hipGetLastError();
 }
 
