@@ -192,7 +192,7 @@ double tile_cost_f32(int M, int N, int K, int count, int bm, int bn, int splits,
     const long long groups = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * count * splits;
     const long long rounds = (groups + 255) / 256;
     /* 16 rows per workgroup: every workgroup stages 128 columns of b for 16 rows of c, twice what the others move
-       per MFMA (measured: 0.7 of the rate, and a longer start) */
+       per MFMA (fitted: 0.55 of the rate) */
     const double rate = big ? 1.0 : (bm == 16 ? 0.55 : (rounds > 1 ? 0.965 : 0.89));
     /* the 32-row tile multiplies only 16 rows when there are no more (16-row MFMAs) */
     const double mfma = (double)(bm == 32 && M <= 16 ? 16 : bm) * bn * ((K + splits - 1) / splits) * 3.48e-6 / rate;
