@@ -268,6 +268,31 @@ def test_half_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     assert_half(got, ref, mag, str((B, lq, lk, H, nh, masked)))
 
 
+@pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
+    (4, 1000, 136, 1024, 16, True),    # head size 64, 512 workgroups of 128 rows, a ragged last block of 64 keys
+    (32, 520, 70, 128, 4, False),      # head size 32, a last workgroup with 8 live rows
+])
+def test_half_with_two_blocks_of_query_rows_per_wave(gpu, oracle, B, lq, lk, H, nh, masked):
+    """Long sequences in half run with 128 query rows per workgroup, two blocks of 16 per wave against blocks of 64
+    keys (taken when such workgroups still give every CU two): against the oracle like the other half cases, and
+    bit for bit the same rows when the sentences are fed in two halves that are too few for that form."""
+    q, k, v = (halfed(oracle, oracle.normal(s, seed)) for s, seed in (((B, lq, H), 71), ((B, lk, H), 72), ((B, lk, H), 73)))
+    mask = None
+    if masked:
+        mask = np.where(oracle.uniform((nh, B, lq, lk), 74, 0.0, 1.0) < 0.3, -1e9, 0.0).astype(np.float32)
+        mask[..., lk // 2] = 0.0
+    scale = float(np.float32(1.0 / np.sqrt(H // nh)))
+    assert nh * B * ((lq + 127) // 128) >= 512
+    ref = oracle.attention(q, k, v, nh, scale, mask)
+    mag = oracle.attention(q, k, np.abs(v), nh, scale, mask)
+    got = run_half(gpu, q, k, v, nh, scale, mask)
+    assert_half(got, ref, mag, str((B, lq, lk, H, nh, masked)))
+    # the one-block form on a part of the batch: the same arithmetic per row up to the order of the key blocks, so the
+    # rows agree to the limit as well
+    part = run_half(gpu, q[:1], k[:1], v[:1], nh, scale, None if mask is None else np.ascontiguousarray(mask[:, :1]))
+    assert_half(part, ref[:1], mag[:1], "one sentence of " + str((B, lq, lk, H, nh, masked)))
+
+
 def test_half_exact_cases_and_benchmark_shape(gpu, oracle):
     torch = torch_()
     # one key: probabilities exactly 1, the result is v's row, bit for bit
