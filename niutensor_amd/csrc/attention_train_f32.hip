@@ -117,10 +117,10 @@ attention_train_f32_kernel(const AttnParams p)
     /* the scaled and masked scores (times log2 e) of this wave's rows against the block of keys in LDS */
     /* The key fragments come from LDS two blocks of 16 keys at a time, one step ahead of the eight products that
        use them: 16 registers, where fragments for a whole slice of the head dimension would be 64. What that frees
-       holds the loads that travel behind this product: a mask that moves 16 bytes at a time and the first values
-       (firstV) from its start, the dropout mask (dropMask) from the start of its last slice. The mask is read
-       without a branch (keys past the end read the row's last ones and are overwritten below), so that its loads
-       travel together. */
+       holds the loads that travel behind this product: the first values (firstV) from its start, with them a mask
+       that moves 16 bytes at a time, or else the dropout mask (dropMask); with such a mask the dropout mask follows
+       from the start of the product's last slice. The mask is read without a branch (keys past the end read the
+       row's last ones and are overwritten below), so that its loads travel together. */
     const bool maskEarly = MK != nullptr && p.maskVec;
     auto scores = [&](int kb0, f32x4 (&accS)[NJ], auto && firstV, auto && dropMask) {
         constexpr int PAIRS = NJ / 2, STEPS = NT * PAIRS;
@@ -136,6 +136,8 @@ attention_train_f32_kernel(const AttnParams p)
             }
         }
         firstV();
+        if (!maskEarly)
+            dropMask();
 #pragma unroll
         for (int i = 0; i < 2; i++)
             kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KP + 4 * g]);
@@ -148,7 +150,7 @@ attention_train_f32_kernel(const AttnParams p)
                 for (int i = 0; i < 2; i++)
                     kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KP + 16 * t1 + 4 * g]);
             }
-            if (st == STEPS - PAIRS)
+            if (maskEarly && st == STEPS - PAIRS)
                 dropMask();
 #pragma unroll
             for (int e = 0; e < 4; e++)
