@@ -35,13 +35,17 @@ template <int DHM, int KB>
 __global__ void __launch_bounds__(256, 2)
 attention_probs_f32_kernel(const AttnParams p)
 {
-    constexpr int KP = DHM + 4;
+    constexpr int KPK = DHM + 8;         /* row pitch of the key block in floats: a 16-byte read takes lanes 0-7 and 16-23 together
+                                            (rows m = 0..7, columns g = 0, 1), then 8-15 with 24-31 and so on: with a
+                                            pitch of 2 mod 16 pieces of 16 bytes those sixteen lanes hit sixteen
+                                            different pieces of the 256 bytes a cycle serves; with a pitch of 1 mod 16
+                                            pieces every such read took two turns (counted: SQ_LDS_BANK_CONFLICT) */
     constexpr int NT = DHM / 16;
     constexpr int NJ = KB / 16;
     constexpr int LOADS = KB * DHM / 4 / 256;
     constexpr float LOG2E = 1.4426950408889634f;
 
-    __shared__ __attribute__((aligned(16))) float Ks[KB * KP];
+    __shared__ __attribute__((aligned(16))) float Ks[KB * KPK];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -64,7 +68,7 @@ attention_probs_f32_kernel(const AttnParams p)
     constexpr int TPR = DHM / 4;
     constexpr int RSTEP = 256 / TPR;
     const int sr0 = tid / TPR, sc = (tid % TPR) * 4;
-    const int sLds = sr0 * KP + sc;
+    const int sLdsK = sr0 * KPK + sc;
     const __amdgpu_buffer_rsrc_t kRsrc = make_rsrc(K, ((long long)(lk - 1) * p.kL + dh) * 4);
     const int kL4 = (int)p.kL * 4;
     const int kOff0 = sc < dh ? sr0 * kL4 + sc * 4 : NTSAMD_OOB_OFFSET;
@@ -113,7 +117,7 @@ attention_probs_f32_kernel(const AttnParams p)
         }
 #pragma unroll
         for (int i = 0; i < 2; i++)
-            kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KP + 4 * g]);
+            kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KPK + 4 * g]);
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
             const int t = st / PAIRS, j0 = 2 * (st % PAIRS);
@@ -121,7 +125,7 @@ attention_probs_f32_kernel(const AttnParams p)
                 const int t1 = (st + 1) / PAIRS, j1 = 2 * ((st + 1) % PAIRS);
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KP + 16 * t1 + 4 * g]);
+                    kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KPK + 16 * t1 + 4 * g]);
             }
 #pragma unroll
             for (int e = 0; e < 4; e++)
@@ -194,7 +198,7 @@ attention_probs_f32_kernel(const AttnParams p)
     for (int kb0 = 0; kb0 < lk; kb0 += KB) {
 #pragma unroll
         for (int s = 0; s < LOADS; s++)
-            *reinterpret_cast<f32x4 *>(&Ks[sLds + s * RSTEP * KP]) = kreg[s];
+            *reinterpret_cast<f32x4 *>(&Ks[sLdsK + s * RSTEP * KPK]) = kreg[s];
         __syncthreads();
         /* the next block of this pass, or the first block again for the second pass */
         if (kb0 + KB < lk)
@@ -235,7 +239,7 @@ attention_probs_f32_kernel(const AttnParams p)
     for (int kb0 = 0; kb0 < lk; kb0 += KB) {
 #pragma unroll
         for (int s = 0; s < LOADS; s++)
-            *reinterpret_cast<f32x4 *>(&Ks[sLds + s * RSTEP * KP]) = kreg[s];
+            *reinterpret_cast<f32x4 *>(&Ks[sLdsK + s * RSTEP * KPK]) = kreg[s];
         __syncthreads();
         if (kb0 + KB < lk)
             load_k(kb0 + KB);
