@@ -37,6 +37,7 @@ Each JSON line carries
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import sys
 import time
@@ -90,6 +91,9 @@ def configs():
                       "with a dropout mask and written again, context on merged tensors (cfg11, the caller's Multiply and cfg12 "
                       "in one launch)",
                  dtype="f32", M=128, N=128, K=64, batch=256),
+        16: dict(name="cfg16 fp16 attention in one kernel at long sequences: softmax(Q.K^T/sqrt(128)).V per head, q,k,v half "
+                      "[2x4096x1024], 8 heads of 128 (the steady state of the half kernel: 64 blocks of 64 keys per workgroup)",
+                 dtype="f16", M=4096, N=4096, K=128, batch=16),
         9: dict(name="cfg9 fp16 attention in one kernel: softmax(Q.K^T/8).V per head, q,k,v half [32x128x512], 8 heads, "
                      "fp32 accumulation and softmax",
                 dtype="f16", M=128, N=128, K=64, batch=256),
@@ -264,6 +268,16 @@ class Workload:
             self.flops = 2.0 * 256 * 128 * 128 * 64
             self.bytes = 4.0 * 256 * 128 * 128 + 2.0 * 2 * 256 * 128 * 64
             self.launches = 1
+        elif idx == 16:
+            self.q = g(oracle.normal((2, 4096, 1024), 1)).half()
+            self.k = g(oracle.normal((2, 4096, 1024), 2)).half()
+            self.v = g(oracle.normal((2, 4096, 1024), 3)).half()
+            self.o = torch.empty((2, 4096, 1024), device=dev, dtype=torch.float16)
+            self.scale = 1.0 / math.sqrt(128.0)
+            self.run = lambda: nt.attention(self.q, self.k, self.v, self.o, 8, self.scale)
+            self.flops = 2 * 2.0 * 16 * 4096 * 4096 * 128
+            self.bytes = 4 * 2.0 * 2 * 4096 * 1024
+            self.launches = 1
         else:
             raise SystemExit("no such configuration: %d" % idx)
 
@@ -361,6 +375,11 @@ class Workload:
         elif idx == 14:
             r = pick(256, 8)
             pairs, whole, rows = [(self.o[r], d(self.p[r].half()) @ d(self.v[r]))], [self.o], 8 * 128
+        elif idx == 16:
+            rq = pick(4096, 64)
+            q, k, v = (d(t[:1]).reshape(1, -1, 8, 128).transpose(1, 2) for t in (self.q[:, rq], self.k, self.v))
+            ref = (torch.softmax(q @ k.transpose(2, 3) * self.scale, -1) @ v).transpose(1, 2).reshape(1, 64, 1024)
+            pairs, whole, rows, limit = [(self.o[:1, rq], ref)], [self.o], 64, 1e-2
         err = max(float((d(got) - ref).abs().max() / ref.abs().max()) for got, ref in pairs)
         finite = all(bool(torch.isfinite(t).all()) for t in whole)
         ok = finite and err <= limit
@@ -434,7 +453,7 @@ def cpu_baseline(idx, budget_s=12.0):
     M, N, K = cfg["M"], cfg["N"], cfg["K"]
     # measured rates of this path on the GPU box's host: ~0.4 GFLOP/s when an operand is walked by column
     # (NN, TN), ~5 GFLOP/s when both are walked along rows (NT)
-    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 13: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9, 14: 6e9, 15: 3e9}[idx]
+    rate = {1: 0.42e9, 2: 0.42e9, 10: 0.42e9, 3: 6e9, 4: 0.43e9, 13: 0.43e9, 5: 2.3e9 if use_ref else 5e9, 6: 0.75e9, 7: 2e9, 8: 4e9, 9: 4e9, 11: 4e9, 12: 2e9, 14: 6e9, 15: 3e9, 16: 4e9}[idx]
     if idx == 3:
         nb = max(1, min(256, int(budget_s * rate / (4.0 * 128 * 128 * 64))))
         q, k, v = o.normal((nb, 128, 64), 1), o.normal((nb, 128, 64), 2), o.normal((nb, 128, 64), 3)
@@ -487,6 +506,15 @@ def cpu_baseline(idx, budget_s=12.0):
         dt = time.perf_counter() - t0
         fl = nb * 8 * 4.0 * 128 * 128 * 64
         sample = "%d of 32 sentences, 8 heads each: split, scale, product, softmax, dropout mask, product, merge" % nb
+    elif idx == 16:
+        rows = max(16, min(4096, int(budget_s * rate / (8 * 4.0 * 4096 * 128)) // 16 * 16))
+        # fp32 arithmetic on the half-rounded values: the reference has no CPU half path
+        q, k, v = (o.from_f16_bits(o.to_f16_bits(o.normal((1, n, 1024), seed))) for n, seed in ((rows, 1), (4096, 2), (4096, 3)))
+        t0 = time.perf_counter()
+        o.attention(q, k, v, 8, 1.0 / math.sqrt(128.0))
+        dt = time.perf_counter() - t0
+        fl = rows * 8 * 4.0 * 4096 * 128
+        sample = "%d of 4096 query rows of one of the 2 sentences against all of its keys, 8 heads: split, scale, product, softmax, product, merge" % rows
     elif idx == 14:
         nb = max(1, min(256, int(budget_s * rate / (2.0 * 128 * 128 * 64))))
         p = o.uniform((nb, 128, 128), 1, 0.0, 1.0)
@@ -825,7 +853,7 @@ def main():
     # the clocks need tens of milliseconds of load to settle: a short warm-up times the ramp
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--config", type=int, default=2, help="configuration 1-15 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values, 15 the attention of the training path in one kernel)")
+    ap.add_argument("--config", type=int, default=2, help="configuration 1-16 (default 2, the MulAndShift linear layer; 6 and 7 are backward steps, 8 and 9 the one-kernel attention in float and half, 10 the linear layer with Rectify, 11 the attention probabilities, 12 the product of the probabilities with the merged values, 13 a half weight gradient cut along k, 14 the attention context with float probabilities and half values, 15 the attention of the training path in one kernel, 16 the half attention at 4096 positions and heads of 128)")
     ap.add_argument("--all", action="store_true", help="one line per configuration, then the headline line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-rotate", action="store_true",
@@ -875,7 +903,7 @@ def main():
     rotate = not args.no_rotate and not args.only
     lines = {}
     if args.all:
-        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
+        for idx in (1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16):
             if idx == args.config:
                 continue
             steps = args.steps if idx != 5 else max(5, args.steps // 10)

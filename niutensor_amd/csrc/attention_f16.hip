@@ -46,9 +46,10 @@ __device__ __forceinline__ float groups_sum(float x)
    reads, not the matrix pipe, are what the kernel waits for (LDS busy 53 % of the kernel's cycles with one block per
    wave). A workgroup then takes 128 query rows, so short sequences, which need the workgroups, keep one block.
    Two blocks of query rows go with blocks of 64 keys: scores and probabilities of 2 x 128 keys at once spilled 37
-   registers and ran slower than one block of rows; with 64 keys the kernel fits 168 registers, three waves to a SIMD. */
+   registers and ran slower than one block of rows; with 64 keys the kernel fits 168 registers, three waves to a SIMD
+   (heads of 128: 242 registers, two waves, as with one block of rows). */
 template <int DHM, int QR>
-__global__ void __launch_bounds__(256, QR == 2 ? 3 : 2)
+__global__ void __launch_bounds__(256, QR == 2 && DHM <= 64 ? 3 : 2)
 attention_f16_kernel(const AttnParams p)
 {
     constexpr int KB = QR == 2 ? 64 : 128;   /* keys per block in LDS */
@@ -295,16 +296,18 @@ int launch_attention_f16(const AttnParams & p0, hipStream_t stream)
     AttnParams p = p0;
     p.maskVec = (p.mask != nullptr && p.lk % 4 == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 15) == 0) ? 1 : 0;
     /* 128 query rows per workgroup (two blocks of 16 per wave) where that still leaves two workgroups for every CU
-       of the part; heads of 128 keep one block (their registers) */
+       of the part */
     const long long groups128 = (long long)p.heads * p.batch * ((p.lq + 127) / 128);
-    const bool two = p.dh <= 64 && p.lq > 64 && groups128 >= 512;
+    const bool two = p.lq > 64 && groups128 >= 512;
     p.qTiles = two ? (p.lq + 127) / 128 : (p.lq + 63) / 64;
     dim3 grid((unsigned)(p.heads * p.batch * p.qTiles));
     if (two) {
         if (p.dh <= 32)
             hipLaunchKernelGGL((attention_f16_kernel<32, 2>), grid, dim3(256), 0, stream, p);
-        else
+        else if (p.dh <= 64)
             hipLaunchKernelGGL((attention_f16_kernel<64, 2>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_f16_kernel<128, 2>), grid, dim3(256), 0, stream, p);
     }
     else if (p.dh <= 32)
         hipLaunchKernelGGL((attention_f16_kernel<32, 1>), grid, dim3(256), 0, stream, p);

@@ -271,6 +271,8 @@ def test_half_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
 @pytest.mark.parametrize("B,lq,lk,H,nh,masked", [
     (4, 1000, 136, 1024, 16, True),    # head size 64, 512 workgroups of 128 rows, a ragged last block of 64 keys
     (32, 520, 70, 128, 4, False),      # head size 32, a last workgroup with 8 live rows
+    (8, 1000, 136, 1024, 8, True),     # head size 128
+    (8, 900, 200, 832, 8, False),      # head size 104 in the kernel built for 128
 ])
 def test_half_with_two_blocks_of_query_rows_per_wave(gpu, oracle, B, lq, lk, H, nh, masked):
     """Long sequences in half run with 128 query rows per workgroup, two blocks of 16 per wave against blocks of 64
