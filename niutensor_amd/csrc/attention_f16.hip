@@ -28,18 +28,6 @@
 
 namespace ntsamd {
 
-__device__ __forceinline__ float groups_max(float x)
-{
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-
-__device__ __forceinline__ float groups_sum(float x)
-{
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
-}
-
 /* DHM: head size the kernel is built for (dh <= DHM, a multiple of 8; columns past dh are zero).
    QR: blocks of 16 query rows per wave. With two, a key or value fragment that a wave reads from LDS feeds two MFMAs
    instead of one: every wave of a workgroup reads every key and every value of a block, and at long sequences those
@@ -222,7 +210,7 @@ attention_f16_kernel(const AttnParams p)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                     mx = fmaxf(mx, accS[q][j][r]);
-            mx = groups_max(mx);
+            mx = lane_groups_max(mx);
             const float newMax = fmaxf(rowMax[q], mx);
             const float shift = newMax == -INFINITY ? 0.f : newMax;
             const float corr = __builtin_amdgcn_exp2f(rowMax[q] - shift);
@@ -235,8 +223,7 @@ attention_f16_kernel(const AttnParams p)
                     sum += e;
                     pf[q][j][r] = (half_t)e;
                 }
-            sum = groups_sum(sum);
-            rowSum[q] = rowSum[q] * corr + sum;
+            rowSum[q] = rowSum[q] * corr + sum;          /* this lane's keys only: the four lanes of a row meet at the end */
             rowMax[q] = newMax;
 #pragma unroll
             for (int d = 0; d < ND; d++)
@@ -273,8 +260,9 @@ attention_f16_kernel(const AttnParams p)
     /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
 #pragma unroll
     for (int q = 0; q < QR; q++) {
+        const float total = lane_groups_sum(rowSum[q]);
         if (row[q] < lq) {
-            const float inv = rowSum[q] > 0.f ? 1.f / rowSum[q] : 0.f;
+            const float inv = total > 0.f ? 1.f / total : 0.f;
             half_t * orow = O + (long long)row[q] * p.oL;
 #pragma unroll
             for (int d = 0; d < ND; d++) {

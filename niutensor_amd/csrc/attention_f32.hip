@@ -35,18 +35,6 @@
 
 namespace ntsamd {
 
-__device__ __forceinline__ float across_groups_max(float x)
-{
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-
-__device__ __forceinline__ float across_groups_sum(float x)
-{
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
-}
-
 /* DHM: head size the kernel is built for (dh <= DHM; columns past dh are zero in LDS and in the
    q fragments, and are multiplied like the others: the launcher picks the smallest DHM that holds dh);
    KB: keys per block */
@@ -231,7 +219,7 @@ attention_f32_kernel(const AttnParams p)
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 mx = fmaxf(mx, accS[j][r]);
-        mx = across_groups_max(mx);
+        mx = lane_groups_max(mx);
         const float newMax = fmaxf(rowMax, mx);
         const float shift = newMax == -INFINITY ? 0.f : newMax;      /* a row with nothing to see yet */
         const float corr = __builtin_amdgcn_exp2f(rowMax - shift);     /* 2^-inf = 0 on the first block */
@@ -244,8 +232,7 @@ attention_f32_kernel(const AttnParams p)
                 accS[j][r] = e;
                 sum += e;
             }
-        sum = across_groups_sum(sum);
-        rowSum = rowSum * corr + sum;
+        rowSum = rowSum * corr + sum;                    /* this lane's keys only: the four lanes of a row meet at the end */
         rowMax = newMax;
 #pragma unroll
         for (int d = 0; d < NT; d++)
@@ -285,6 +272,7 @@ attention_f32_kernel(const AttnParams p)
     }
 
     /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
+    rowSum = lane_groups_sum(rowSum);
     if (row < lq) {
         const float inv = rowSum > 0.f ? 1.f / rowSum : 0.f;
         float * orow = O + (long long)row * p.oL;

@@ -26,18 +26,6 @@
 
 namespace ntsamd {
 
-__device__ __forceinline__ float train_groups_max(float x)
-{
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-
-__device__ __forceinline__ float train_groups_sum(float x)
-{
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
-}
-
 template <int DHM, int KB>
 __global__ void __launch_bounds__(256, 2)
 attention_train_f32_kernel(const AttnParams p)
@@ -207,7 +195,7 @@ attention_train_f32_kernel(const AttnParams p)
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 mx = fmaxf(mx, accS[j][r]);
-        mx = train_groups_max(mx);
+        mx = lane_groups_max(mx);
         const float newMax = fmaxf(rowMax, mx);
         const float shift = newMax == -INFINITY ? 0.f : newMax;
         float sum = 0.f;
@@ -216,7 +204,7 @@ attention_train_f32_kernel(const AttnParams p)
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 sum += __builtin_amdgcn_exp2f(accS[j][r] - shift);
-        sum = train_groups_sum(sum);
+        sum = lane_groups_sum(sum);
         rowSum = rowSum * __builtin_amdgcn_exp2f(rowMax - shift) + sum;
         rowMax = newMax;
     };
