@@ -90,17 +90,18 @@ attention_f32_kernel(const AttnParams p)
     const int kOff0 = sc < dh ? sr0 * kL4 + sc * 4 : NTSAMD_OOB_OFFSET;
     const int vOff0 = sc < dh ? sr0 * vL4 + sc * 4 : NTSAMD_OOB_OFFSET;
     f32x4 kreg[LOADS], vreg[LOADS];
-    auto load_k = [&](int kb0) {
+    auto load_k = [&](int kb0, int first, int last) {
 #pragma unroll
         for (int s = 0; s < LOADS; s++)
-            kreg[s] = buffer_load_f32x4(kRsrc, sc < dh ? kOff0 + (kb0 + s * RSTEP) * kL4 : NTSAMD_OOB_OFFSET);
+            if (s >= first && s < last)
+                kreg[s] = buffer_load_f32x4(kRsrc, sc < dh ? kOff0 + (kb0 + s * RSTEP) * kL4 : NTSAMD_OOB_OFFSET);
     };
     auto load_v = [&](int kb0) {
 #pragma unroll
         for (int s = 0; s < LOADS; s++)
             vreg[s] = buffer_load_f32x4(vRsrc, sc < dh ? vOff0 + (kb0 + s * RSTEP) * vL4 : NTSAMD_OOB_OFFSET);
     };
-    load_k(0);
+    load_k(0, 0, LOADS / 2);     /* the second half of the first keys is asked for when the first has arrived */
 
     /* ---- Q fragments: lane (m, g) feeds query m with columns 16 t + 4 g + e in step e of group t ---- */
     f32x4 qf[NT];
@@ -121,96 +122,143 @@ attention_f32_kernel(const AttnParams p)
     float rowMax = -INFINITY, rowSum = 0.f;              /* in units of log2: the scores are scaled by log2(e) */
     const float scale2 = p.scale * LOG2E;
 
+    /* The keys of a block reach LDS in two halves, and the first product begins when the first half is there:
+           keys of half 1 -> LDS | barrier | S1 = K1 Q^T | keys of half 2, values -> LDS | barrier | S2 = K2 Q^T |
+           softmax of the block | O += P V
+       At the start of the kernel every workgroup of the grid waits for its queries and keys at once, at the rate the
+       memory delivers them: the second half of the first keys (and then the values) are asked for only when the
+       first half has arrived, so that everybody's first halves travel first. The first barrier also says that every
+       wave has finished the previous block's second half and its values, the second that every wave has finished
+       this block's first half. (Measured against it at the benchmark shape: the softmax of one half between the
+       MFMAs of the other half's products, 13.0 us where this order takes 12.8: the matrix pipe of a SIMD is kept busy
+       by its two waves either way.) */
+    constexpr int HJ = NJ / 2;           /* 16-key blocks per half */
+    constexpr int HL = LOADS / 2;        /* staging steps per half */
+    constexpr int PAIRS = HJ / 2;        /* the key fragments come from LDS two blocks of 16 keys at a time */
+    constexpr int STEPS = NT * PAIRS;    /* steps of 8 MFMAs of a half's first product */
+    static_assert(NJ % 4 == 0 && LOADS % 2 == 0, "two halves of pairs of 16-key blocks");
+
     for (int kb0 = 0; kb0 < lk; kb0 += KB) {
         const bool more = kb0 + KB < lk;
+        const bool second = kb0 + 16 * HJ < lk;          /* the second half holds a key: else it is not multiplied */
 
-        /* every wave is past the second barrier of the previous block: nobody reads Ks any more */
 #pragma unroll
-        for (int s = 0; s < LOADS; s++)
+        for (int s = 0; s < HL; s++)
             *reinterpret_cast<f32x4 *>(&Ks[sLdsK + s * RSTEP * KPK]) = kreg[s];
-        __syncthreads();                                 /* also: every wave has finished the previous block's Vs */
-        /* the first values are asked for only now: at the start every workgroup of the grid wants its keys and
-           queries at once, and values queued among them would hold back the keys of the workgroups that start later */
-        if (kb0 == 0)
+        __syncthreads();
+        if (kb0 == 0) {
+            load_k(0, HL, LOADS);
             load_v(0);
-        if (more)
-            load_k(kb0 + KB);
+        }
 
-        /* ---- S^T = K Q^T ------------------------------------------------------------------------ */
         f32x4 accS[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; j++)
             accS[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        /* The key fragments come from LDS two blocks of 16 keys at a time, one step ahead of the eight products
-           that use them (16 registers, where fragments for a whole group would be 64; the scheduling fences keep the
-           compiler from fetching further ahead). What that frees holds a mask that moves 16 bytes at a time, asked
-           for before the product begins and without a branch (keys past the end read the row's last ones and are
-           overwritten below), so that its loads travel together and behind the product. */
-        constexpr int PAIRS = NJ / 2, STEPS = NT * PAIRS;
+        /* a mask that moves 16 bytes at a time is asked for, half a block at a time, before the product begins and
+           without a branch (keys past the end read the row's last ones and are overwritten below), so that its loads
+           travel together and behind the product */
         const bool maskEarly = MK != nullptr && p.maskVec;
-        f32x4 kf[2][2], mk[NJ];
-        if (maskEarly) {
+        f32x4 kf[2][2], mk[HJ];
+        auto load_mask = [&](const int jb) {
+            if (maskEarly) {
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                const int key = kb0 + 16 * j + 4 * g;          /* lk is a multiple of 4 here: all four or none */
-                mk[j] = *reinterpret_cast<const f32x4 *>(MK + (key < lk ? key : lk - 4));
+                for (int j = 0; j < HJ; j++) {
+                    const int key = kb0 + 16 * (jb + j) + 4 * g;   /* lk is a multiple of 4 here: all four or none */
+                    mk[j] = *reinterpret_cast<const f32x4 *>(MK + (key < lk ? key : lk - 4));
+                }
             }
-        }
+        };
+        /* scale, mask and the end of the keys for the half that begins with block jb */
+        auto scale_and_mask = [&](const int jb) {
+            if (MK != nullptr) {
+                if (p.maskVec) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-            kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * i + m) * KPK + 4 * g]);
+                    for (int j = jb; j < jb + HJ; j++)
 #pragma unroll
-        for (int st = 0; st < STEPS; st++) {
-            const int t = st / PAIRS, j0 = 2 * (st % PAIRS);
-            if (st + 1 < STEPS) {
-                const int t1 = (st + 1) / PAIRS, j1 = 2 * ((st + 1) % PAIRS);
+                        for (int r = 0; r < 4; r++)
+                            accS[j][r] = fmaf(mk[j - jb][r], LOG2E, accS[j][r] * scale2);
+                }
+                else {
 #pragma unroll
-                for (int i = 0; i < 2; i++)
-                    kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KPK + 16 * t1 + 4 * g]);
-            }
+                    for (int j = jb; j < jb + HJ; j++)
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-                    accS[j0 + i] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st & 1][i][e], qf[t][e], accS[j0 + i], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-
-        /* ---- scale and mask ------ */
-        if (MK != nullptr) {
-            if (p.maskVec) {
-#pragma unroll
-                for (int j = 0; j < NJ; j++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        accS[j][r] = fmaf(mk[j][r], LOG2E, accS[j][r] * scale2);
+                        for (int r = 0; r < 4; r++) {
+                            int key = kb0 + 16 * j + 4 * g + r;
+                            key = key < lk ? key : lk - 1;
+                            accS[j][r] = fmaf(MK[key], LOG2E, accS[j][r] * scale2);
+                        }
+                }
             }
             else {
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
+                for (int j = jb; j < jb + HJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        int key = kb0 + 16 * j + 4 * g + r;
-                        key = key < lk ? key : lk - 1;
-                        accS[j][r] = fmaf(MK[key], LOG2E, accS[j][r] * scale2);
-                    }
+                    for (int r = 0; r < 4; r++)
+                        accS[j][r] *= scale2;
             }
-        }
+            if (kb0 + KB > lk) {                               /* last, partial block: keys past the end count for nothing */
+#pragma unroll
+                for (int j = jb; j < jb + HJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (kb0 + 16 * j + 4 * g + r >= lk)
+                            accS[j][r] = -INFINITY;
+            }
+        };
+        /* ---- S^T = K Q^T for the half that begins with block jb; the key fragments of a step are asked for one step
+           ahead (16 registers; the scheduling fences keep the compiler from fetching further ahead); the second half
+           carries the first half's scale and mask behind its first step ---- */
+        auto scores = [&](const int jb) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                kf[0][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (jb + i) + m) * KPK + 4 * g]);
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                const int t = st / PAIRS, j0 = jb + 2 * (st % PAIRS);
+                if (st + 1 < STEPS) {
+                    const int t1 = (st + 1) / PAIRS, j1 = jb + 2 * ((st + 1) % PAIRS);
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+                        kf[(st + 1) & 1][i] = *reinterpret_cast<const f32x4 *>(&Ks[(16 * (j1 + i) + m) * KPK + 16 * t1 + 4 * g]);
+                }
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+#pragma unroll
+                        for (int i = 0; i < 2; i++)
+                            accS[j0 + i] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[st & 1][i][e], qf[t][e], accS[j0 + i], 0, 0, 0);
+                }
+                if (jb > 0 && st == 0) {
+                    scale_and_mask(0);
+                    load_mask(HJ);                           /* the first half has used its own */
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        load_mask(0);
+        scores(0);
+
+        /* ---- the second half of the keys and the values into LDS ---- */
+#pragma unroll
+        for (int s = HL; s < LOADS; s++)
+            *reinterpret_cast<f32x4 *>(&Ks[sLdsK + s * RSTEP * KPK]) = kreg[s];
+#pragma unroll
+        for (int s = 0; s < LOADS; s++)
+            *reinterpret_cast<f32x4 *>(&Vs[sLds + s * RSTEP * KP]) = vreg[s];
+        __syncthreads();
+        if (more)
+            load_k(kb0 + KB, 0, LOADS);
+
+        if (second)
+            scores(HJ);
         else {
-#pragma unroll
-            for (int j = 0; j < NJ; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    accS[j][r] *= scale2;
+            scale_and_mask(0);
+            load_mask(HJ);
         }
-        if (kb0 + KB > lk) {                                   /* last, partial block: keys past the end count for nothing */
-#pragma unroll
-            for (int j = 0; j < NJ; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (kb0 + 16 * j + 4 * g + r >= lk)
-                        accS[j][r] = -INFINITY;
-        }
+        if (more)
+            load_v(kb0 + KB);
+        scale_and_mask(HJ);
 
         /* ---- running softmax of this lane's query row ------------------------------------------------ */
         float mx = accS[0][0];
@@ -238,14 +286,6 @@ attention_f32_kernel(const AttnParams p)
         for (int d = 0; d < NT; d++)
             accO[d] *= corr;
 
-        /* ---- values into LDS (every wave is past the first barrier: the previous block's Vs is done with) ---- */
-#pragma unroll
-        for (int s = 0; s < LOADS; s++)
-            *reinterpret_cast<f32x4 *>(&Vs[sLds + s * RSTEP * KP]) = vreg[s];
-        __syncthreads();                                 /* also: every wave has finished this block's Ks */
-        if (more)
-            load_v(kb0 + KB);
-
         /* ---- O^T += V^T P^T: the probabilities are operands as they lie ---------------------------------- */
         float vf[2][4][NT];
 #pragma unroll
@@ -253,22 +293,27 @@ attention_f32_kernel(const AttnParams p)
 #pragma unroll
             for (int d = 0; d < NT; d++)
                 vf[0][r][d] = Vs[(4 * g + r) * KP + m + 16 * d];
+        auto context = [&](const int jb) {
 #pragma unroll
-        for (int j = 0; j < NJ; j++) {
-            if (j + 1 < NJ) {
+            for (int j = jb; j < jb + HJ; j++) {
+                if (j + 1 < NJ) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int d = 0; d < NT; d++)
+                            vf[(j + 1) & 1][r][d] = Vs[(16 * (j + 1) + 4 * g + r) * KP + m + 16 * d];
+                }
 #pragma unroll
                 for (int r = 0; r < 4; r++)
 #pragma unroll
                     for (int d = 0; d < NT; d++)
-                        vf[(j + 1) & 1][r][d] = Vs[(16 * (j + 1) + 4 * g + r) * KP + m + 16 * d];
+                        accO[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j & 1][r][d], accS[j][r], accO[d], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-#pragma unroll
-                for (int d = 0; d < NT; d++)
-                    accO[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j & 1][r][d], accS[j][r], accO[d], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        };
+        context(0);
+        if (second)
+            context(HJ);
     }
 
     /* ---- out = result / row sum: register r of block d is column 16 d + 4 g + r of the lane's row ---- */
