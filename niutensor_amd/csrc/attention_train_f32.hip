@@ -352,12 +352,26 @@ int launch_attention_train_f32(const AttnParams & p0, hipStream_t stream)
     p.probsVec = (p.lk % 4 == 0 && (reinterpret_cast<uintptr_t>(p.probs) & 15) == 0 &&
                   (reinterpret_cast<uintptr_t>(p.dropMask) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.dropped) & 15) == 0) ? 1 : 0;
     dim3 grid((unsigned)(p.heads * p.batch * p.qTiles));
-    if (p.dh <= 16)
-        hipLaunchKernelGGL((attention_train_f32_kernel<16, 128>), grid, dim3(256), 0, stream, p);
-    else if (p.dh <= 32)
-        hipLaunchKernelGGL((attention_train_f32_kernel<32, 128>), grid, dim3(256), 0, stream, p);
-    else if (p.dh <= 64)
-        hipLaunchKernelGGL((attention_train_f32_kernel<64, 128>), grid, dim3(256), 0, stream, p);
+    /* at most 64 keys (short sentences): blocks of 64, so that no product multiplies 16-key blocks without a key */
+    const bool few = p.lk <= 64;
+    if (p.dh <= 16) {
+        if (few)
+            hipLaunchKernelGGL((attention_train_f32_kernel<16, 64>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_train_f32_kernel<16, 128>), grid, dim3(256), 0, stream, p);
+    }
+    else if (p.dh <= 32) {
+        if (few)
+            hipLaunchKernelGGL((attention_train_f32_kernel<32, 64>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_train_f32_kernel<32, 128>), grid, dim3(256), 0, stream, p);
+    }
+    else if (p.dh <= 64) {
+        if (few)
+            hipLaunchKernelGGL((attention_train_f32_kernel<64, 64>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_train_f32_kernel<64, 128>), grid, dim3(256), 0, stream, p);
+    }
     else
         hipLaunchKernelGGL((attention_train_f32_kernel<128, 64>), grid, dim3(256), 0, stream, p);
     return (int)hipGetLastError();

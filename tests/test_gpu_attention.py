@@ -59,6 +59,8 @@ def test_fixtures_of_the_compiled_reference(gpu, generated_attention):
     (2, 33, 65, 192, 2, True),         # head size 96 inside the 128 kernel
     (4, 9, 5, 8, 2, False),            # head size 4
     (1, 1, 1, 12, 1, False),           # a single score
+    (3, 70, 64, 192, 3, True),         # short sentences: the second half of the key block holds no key
+    (2, 50, 33, 64, 2, False),
 ])
 def test_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     q, k, v = oracle.normal((B, lq, H), 11), oracle.normal((B, lk, H), 12), oracle.normal((B, lk, H), 13)
@@ -132,6 +134,8 @@ def test_attention_shape_of_the_benchmark(gpu, oracle):
     (2, 40, 261, 256, 2, False),       # head size 128, ragged
     (4, 9, 5, 8, 2, False),            # head size 4
     (1, 1, 1, 12, 1, False),
+    (3, 70, 64, 192, 3, True),         # short sentences: blocks of 64 keys, 16-byte stores
+    (2, 50, 33, 64, 2, False),         # the same, ragged
 ])
 def test_probabilities_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     """The first half on its own (what the training path keeps): softmax(scale q k^T + mask) as a
@@ -169,6 +173,8 @@ def test_probabilities_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     (2, 40, 261, 256, 2, False, True),      # head size 128, ragged
     (4, 9, 5, 8, 2, False, False),          # head size 4, no dropout
     (2, 70, 200, 128, 4, True, False),
+    (3, 70, 64, 192, 3, True, True),        # short sentences: blocks of 64 keys
+    (2, 50, 33, 64, 2, False, True),
 ])
 def test_training_path_in_one_launch(gpu, oracle, B, lq, lk, H, nh, masked, dropout):
     """ntsamd_attention_train against the operator chain of the reference's training path put together from the
