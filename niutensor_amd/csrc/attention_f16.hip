@@ -36,11 +36,10 @@ namespace ntsamd {
    Two blocks of query rows go with blocks of 64 keys: scores and probabilities of 2 x 128 keys at once spilled 37
    registers and ran slower than one block of rows; with 64 keys the kernel fits 168 registers, three waves to a SIMD
    (heads of 128: 242 registers, two waves, as with one block of rows). */
-template <int DHM, int QR>
+template <int DHM, int QR, int KB = (QR == 2 ? 64 : 128)>   /* KB: keys per block in LDS */
 __global__ void __launch_bounds__(256, QR == 2 && DHM <= 64 ? 3 : 2)
 attention_f16_kernel(const AttnParams p)
 {
-    constexpr int KB = QR == 2 ? 64 : 128;   /* keys per block in LDS */
     constexpr int PITCH = DHM * 2 + 16;      /* bytes per LDS row: 16 mod 128, so 16-byte reads of consecutive rows
                                                 walk through the banks */
     constexpr int NT = DHM / 32;             /* k steps of the first product */
@@ -296,6 +295,14 @@ int launch_attention_f16(const AttnParams & p0, hipStream_t stream)
             hipLaunchKernelGGL((attention_f16_kernel<64, 2>), grid, dim3(256), 0, stream, p);
         else
             hipLaunchKernelGGL((attention_f16_kernel<128, 2>), grid, dim3(256), 0, stream, p);
+    }
+    else if (p.lk <= 64) {          /* short sentences: blocks of 64 keys, so that no product multiplies 16-key blocks without a key */
+        if (p.dh <= 32)
+            hipLaunchKernelGGL((attention_f16_kernel<32, 1, 64>), grid, dim3(256), 0, stream, p);
+        else if (p.dh <= 64)
+            hipLaunchKernelGGL((attention_f16_kernel<64, 1, 64>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attention_f16_kernel<128, 1, 64>), grid, dim3(256), 0, stream, p);
     }
     else if (p.dh <= 32)
         hipLaunchKernelGGL((attention_f16_kernel<32, 1>), grid, dim3(256), 0, stream, p);

@@ -258,6 +258,8 @@ def run_half(gpu, q, k, v, heads, scale, mask=None):
     (2, 33, 65, 80, 2, True),          # head size 40 inside the 64 kernel
     (4, 9, 5, 16, 2, False),           # head size 8
     (1, 1, 1, 8, 1, False),            # a single score
+    (3, 70, 64, 192, 3, True),         # short sentences: blocks of 64 keys
+    (2, 50, 33, 256, 2, False),        # the same with heads of 128, ragged
 ])
 def test_half_against_oracle(gpu, oracle, B, lq, lk, H, nh, masked):
     """Half tensors: the fp32 oracle on the half-rounded inputs, result within 1e-2 (the limit the
