@@ -1077,3 +1077,28 @@ def test_rectified_linear_layer_at_full_size(gpu, oracle):
     assert torch.equal(rect, torch.clamp_min(plain, 0.0))
     assert 0.3 < (rect == 0).float().mean().item() < 0.7
 
+
+
+@pytest.mark.parametrize("half,M,N,K,tb,beta", [
+    (True, 70000, 32768, 256, X_NOTRANS, 0.5),      # c: 4.6 GB, the walking kernel with the old c
+    (True, 2200000, 1024, 64, X_TRANS, 0.0),        # 2.2 million rows: the last rows start past 2^32 bytes
+    (False, 40000, 30011, 64, X_TRANS, 1.0),        # c: 4.8 GB of rows that are only 4-byte aligned
+])
+def test_results_of_more_than_four_gigabytes(gpu, half, M, N, K, tb, beta):
+    """A tile's base is a 64-bit address and only the offsets inside the tile's window are 32-bit: rows at the start,
+    in the middle and at the very end of a result of more than 2^32 bytes against float64 (the size-independent
+    check: the oracle would take minutes here), and no element of the first and the last 4096 rows left unwritten."""
+    torch = torch_()
+    dt = torch.float16 if half else torch.float32
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    a = torch.randn((M, K), device=gpu, generator=gen).to(dt)
+    b = torch.randn((N, K) if tb == X_TRANS else (K, N), device=gpu, generator=gen).to(dt)
+    c = torch.randn((M, N), device=gpu, generator=gen).to(dt) if beta else torch.full((M, N), float("nan"), device=gpu, dtype=dt)
+    rows = torch.tensor([0, 1, M // 2, M // 2 + 77, M - 2, M - 1], device=gpu)
+    old = c[rows].double() if beta else 0.0
+    nt.matrix_mul(a, X_NOTRANS, b, tb, c, 1.0, beta)
+    torch.cuda.synchronize()
+    ref = a[rows].double() @ (b.double().t() if tb == X_TRANS else b.double()) + beta * old
+    err = float((c[rows].double() - ref).abs().max() / ref.abs().max())
+    assert err <= (FP16_LIMIT if half else fp32_limit(K)), (err, nt.last_plan())
+    assert bool(torch.isfinite(c[:4096]).all()) and bool(torch.isfinite(c[M - 4096:]).all())
